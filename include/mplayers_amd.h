@@ -1,0 +1,100 @@
+/*
+ * C ABI of libmplayers_hip.so: min-sum message passing (TRWP, ISGMR) on grid MRFs for gfx950.
+ *
+ * Every pointer is a DEVICE pointer unless said otherwise; all tensors are contiguous with the
+ * label axis innermost.  The caller owns and allocates every buffer, exactly as the reference's
+ * operators require (pytorch/MP_module.py:26-50, 65-78); buffers marked "zero-filled" must come
+ * in zeroed, as the reference's caller provides them.  `stream` is a hipStream_t (NULL = the
+ * default stream).  Nothing here allocates device memory or synchronises with the host.
+ *
+ * Shapes:  B = batch * n_cv,  P = B*H*W pixels,  N = P*L.
+ *   unary, cost_final, unary_update, dcost_final, dunary, dunary_update   (B, H, W, L)  fp32
+ *   msg, msg_update, dmsg, dmsg_update                                    (n_dir, B, H, W, L) fp32
+ *   edge_weights, dedge_weights                                           (n_dir, B, H, W) fp32
+ *   msg_min_index   (n_iter, n_dir, B, H, W, L) uint8      msg_norm_index (n_iter, n_dir, B, H, W) uint8
+ *   label_all       (n_iter, B, H, W) uint8
+ *   context         ctx2d ? (L, L), entries [min(a,b)*L + max(a,b)] read : >= L floats, [|a-b|] read
+ *   dcontext        same shape as context (zero-filled; only off-diagonal / k>=1 entries are written)
+ *
+ * Return value: 0 on success, a negative MPL_E* code otherwise; mpl_last_error() then returns a
+ * message for the calling thread.  On error nothing has been launched.
+ */
+#ifndef MPLAYERS_AMD_H_
+#define MPLAYERS_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MPL_OK 0
+#define MPL_EINVAL (-1)   /* bad shape / null pointer / unsupported size */
+#define MPL_ELAUNCH (-2)  /* the HIP runtime refused a launch */
+
+#define MPL_MAX_LABELS 256 /* argmin indices are uint8 (reference: MAX_DISPARITY, MPLayers/setup.py:58) */
+#define MPL_MAX_DIRS 16    /* direction table of MPLayers/common.cpp:28-76 */
+
+typedef struct mpl_shape {
+  int n_dir;  /* 2..16, even: direction d pairs with d^1 (common.cpp:23-26) */
+  int batch;  /* batch * n_cv */
+  int height;
+  int width;
+  int n_disp; /* labels, <= MPL_MAX_LABELS */
+  int ctx2d;  /* 1: (L,L) context table (the reference selects it by n_disp == 21); needs L <= 64 */
+} mpl_shape;
+
+/* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.
+ * msg: initial messages in, final normalised messages out.  msg_min_index/msg_norm_index NULL =>
+ * inference (no index stores).  label_all NULL => no per-iteration labels.  unary_update: scratch
+ * plane (holds the running belief).  cost_final doubles as scratch until the final aggregation. */
+int mpl_trwp_forward(const mpl_shape* shape, float rho, int n_iter, int enable_min_a_dir,
+                     const float* unary, const float* context, const float* edge_weights,
+                     float* msg, float* cost_final, uint8_t* msg_min_index,
+                     uint8_t* msg_norm_index, float* unary_update, uint8_t* label_all,
+                     void* stream);
+
+/* Replaces lib_*.TRWP.backward: MPLayers/TRWP/TRWP.cpp:285-318 -> TRWP_backward.cu:277-433.
+ * dunary receives the gradient; dcontext and dedge_weights (zero-filled) accumulate; dmsg is
+ * scratch (n_dir planes, any contents); dunary_update is accepted and unused. */
+int mpl_trwp_backward(const mpl_shape* shape, float rho, int n_iter, const float* context,
+                      const float* edge_weights, const float* dcost_final,
+                      const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
+                      float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
+                      void* stream);
+
+/* Replaces lib_*.ISGMR.forward: MPLayers/ISGMR/ISGMR.cpp:300-342 -> ISGMR_forward.cu:433-665.
+ * msg_update: second message buffer (zero-filled); on return msg holds the final messages. */
+int mpl_isgmr_forward(const mpl_shape* shape, int enable_sgm, float rho, int n_iter,
+                      int enable_min_a_dir, const float* unary, const float* context,
+                      const float* edge_weights, float* msg, float* cost_final,
+                      uint8_t* msg_min_index, uint8_t* msg_norm_index, float* unary_update,
+                      float* msg_update, uint8_t* label_all, void* stream);
+
+/* Replaces lib_*.ISGMR.backward: MPLayers/ISGMR/ISGMR.cpp:344-379 -> ISGMR_backward.cu:290-493.
+ * dmsg_update is scratch (n_dir planes, any contents); dmsg and dunary_update are unused. */
+int mpl_isgmr_backward(const mpl_shape* shape, int enable_sgm, float rho, int n_iter,
+                       const float* context, const float* edge_weights, const float* dcost_final,
+                       const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
+                       float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
+                       float* dmsg_update, void* stream);
+
+/* Device check of the wavefront primitives the kernels are built on (cross-lane shifts, min/sum
+ * reductions, ballots).  out: 8 host ints, out[0] == 1 when every check passed.  Synchronises. */
+int mpl_selftest_wave_ops(int* out_host);
+
+/* Number of chains of direction `dir` (0..15) on an H x W grid; equals the reference's n_trees
+ * (common.cpp:78-87) minus chains that never enter the image.  Host-only helper. */
+int mpl_n_chains(int dir, int height, int width);
+
+/* Message of the last failed call on this thread ("" if none). */
+const char* mpl_last_error(void);
+
+/* Library version: major * 100 + minor. */
+int mpl_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MPLAYERS_AMD_H_ */

@@ -1,0 +1,48 @@
+"""ctypes binding of libmplayers_hip.so (the C ABI declared in include/mplayers_amd.h)."""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmplayers_hip.so")
+
+SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
+           "mpl_selftest_wave_ops", "mpl_n_chains", "mpl_last_error", "mpl_version")
+
+
+class Shape(ctypes.Structure):
+  """struct mpl_shape"""
+  _fields_ = [("n_dir", ctypes.c_int), ("batch", ctypes.c_int), ("height", ctypes.c_int),
+              ("width", ctypes.c_int), ("n_disp", ctypes.c_int), ("ctx2d", ctypes.c_int)]
+
+
+_lib = None
+
+
+def load():
+  """Loads the HIP library; raises if it has not been built (there is no fallback path)."""
+  global _lib
+  if _lib is not None:
+    return _lib
+  if not os.path.exists(LIB_PATH):
+    raise RuntimeError(
+        "libmplayers_hip.so is missing: build it with `python -m mplayers_amd._build` "
+        "(hipcc --offload-arch=gfx950); there is no CPU or PyTorch fallback for these operators")
+  lib = ctypes.CDLL(LIB_PATH)
+  vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+  sp = ctypes.POINTER(Shape)
+  lib.mpl_trwp_forward.argtypes = [sp, cf, ci, ci] + [vp] * 10
+  lib.mpl_trwp_backward.argtypes = [sp, cf, ci] + [vp] * 11
+  lib.mpl_isgmr_forward.argtypes = [sp, ci, cf, ci, ci] + [vp] * 11
+  lib.mpl_isgmr_backward.argtypes = [sp, ci, cf, ci] + [vp] * 12
+  lib.mpl_selftest_wave_ops.argtypes = [ctypes.POINTER(ci)]
+  lib.mpl_n_chains.argtypes = [ci, ci, ci]
+  lib.mpl_last_error.restype = ctypes.c_char_p
+  for name in SYMBOLS:
+    getattr(lib, name).restype = getattr(lib, name).restype or ci
+  _lib = lib
+  return lib
+
+
+def check(rc, what):
+  if rc != 0:
+    raise RuntimeError("%s failed (%d): %s" % (what, rc, load().mpl_last_error().decode()))

@@ -1,0 +1,165 @@
+"""Operator layer with the reference's extension signatures (lib_stereo / lib_seg modules).
+
+`TRWP.forward/backward` and `ISGMR.forward/backward` take exactly the positional arguments of
+the reference's pybind11 modules (MPLayers/TRWP/TRWP.cpp:245-256, 285-295, 324-325 and
+MPLayers/ISGMR/ISGMR.cpp:300-313, 344-356, 400-401): caller-allocated, zero-filled tensors that
+are filled in place; an empty index / label tensor switches that output off.  They hand raw device
+pointers and the current HIP stream to the C ABI of libmplayers_hip.so.
+
+Deviations from the reference, all towards failing loudly: more labels than 256 (the reference
+prints a message and returns zero-filled outputs, TRWP.cpp:269-273), CPU tensors (the reference
+runs its CPU loop, or prints "Does not support CPU backward", :315-316) and non-contiguous tensors
+raise RuntimeError.
+"""
+import torch
+
+from . import _lib
+
+
+def _ptr(t):
+  return None if t is None or t.numel() == 0 else t.data_ptr()
+
+
+def _check(name, t, dtype, numel=None):
+  if not isinstance(t, torch.Tensor):
+    raise TypeError("%s must be a tensor" % name)
+  if not t.is_cuda:
+    raise RuntimeError("%s is not on the GPU: these operators only run as HIP kernels" % name)
+  if not t.is_contiguous():
+    raise RuntimeError("%s must be contiguous" % name)  # CHECK_CONTIGUOUS, cudaUtils.hpp:10
+  if t.dtype != dtype:
+    raise RuntimeError("%s must be %s, got %s" % (name, dtype, t.dtype))
+  if numel is not None and t.numel() < numel:
+    raise RuntimeError("%s has %d elements, %d needed" % (name, t.numel(), numel))
+
+
+def _context_numel(L, ctx2d):
+  return L * L if ctx2d else L
+
+
+class _Op(object):
+  """Shared plumbing of the two operator namespaces."""
+
+  @staticmethod
+  def _shape_from_msg(msg):
+    if msg.dim() != 6:
+      raise RuntimeError("msg must be (n_dir, batch, cv, h, w, n_disp)")
+    n_dir, b, cv, h, w, L = msg.shape
+    ctx2d = (L == 21)  # the reference switches to the (L, L) table by n_disp == 21
+    return _lib.Shape(n_dir, b * cv, h, w, L, int(ctx2d)), b * cv * h * w, L, ctx2d
+
+  @staticmethod
+  def _shape_from_index(msg_min_index):
+    if msg_min_index.dim() != 7:
+      raise RuntimeError("msg_min_index must be (n_iter, n_dir, batch, cv, h, w, n_disp)")
+    n_iter, n_dir, b, cv, h, w, L = msg_min_index.shape
+    ctx2d = (L == 21)
+    return _lib.Shape(n_dir, b * cv, h, w, L, int(ctx2d)), n_iter, b * cv * h * w, L, ctx2d
+
+  @staticmethod
+  def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+  @staticmethod
+  def _check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
+                     msg_norm_index, unary_update, label_all, n_iter):
+    shape, P, L, ctx2d = _Op._shape_from_msg(msg)
+    N = P * L
+    f32, u8 = torch.float32, torch.uint8
+    _check("unary", unary, f32, N)
+    _check("context", context, f32, _context_numel(L, ctx2d))
+    _check("edge_weights", edge_weights, f32, shape.n_dir * P)
+    _check("msg", msg, f32, shape.n_dir * N)
+    _check("cost_final", cost_final, f32, N)
+    _check("unary_update", unary_update, f32, N)
+    training = msg_min_index.numel() > 0
+    if training:
+      _check("msg_min_index", msg_min_index, u8, n_iter * shape.n_dir * N)
+      _check("msg_norm_index", msg_norm_index, u8, n_iter * shape.n_dir * P)
+    if label_all.numel() > 0:
+      _check("label_all", label_all, u8, n_iter * P)
+    return shape, P, N
+
+
+class TRWP(object):
+  """Drop-in for the reference's `lib_stereo.TRWP` / `lib_seg.TRWP` extension modules."""
+
+  @staticmethod
+  def forward(rho, n_iter, enable_min_a_dir, unary, context, edge_weights, msg, cost_final,
+              msg_min_index, msg_norm_index, unary_update, label_all):
+    lib = _lib.load()
+    shape, _, _ = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
+                                     msg_norm_index, unary_update, label_all, n_iter)
+    with torch.cuda.device(unary.device):
+      rc = lib.mpl_trwp_forward(shape, float(rho), int(n_iter), int(enable_min_a_dir),
+                                _ptr(unary), _ptr(context), _ptr(edge_weights), _ptr(msg),
+                                _ptr(cost_final), _ptr(msg_min_index), _ptr(msg_norm_index),
+                                _ptr(unary_update), _ptr(label_all), _Op._stream(unary))
+    _lib.check(rc, "TRWP.forward")
+
+  @staticmethod
+  def backward(rho, context, edge_weights, dcost_final, msg_min_index, msg_norm_index, dunary,
+               dcontext, dedge_weights, dmsg, dunary_update):
+    lib = _lib.load()
+    shape, n_iter, P, L, ctx2d = _Op._shape_from_index(msg_min_index)
+    N = P * L
+    f32, u8 = torch.float32, torch.uint8
+    _check("context", context, f32, _context_numel(L, ctx2d))
+    _check("edge_weights", edge_weights, f32, shape.n_dir * P)
+    _check("dcost_final", dcost_final, f32, N)
+    _check("msg_min_index", msg_min_index, u8, n_iter * shape.n_dir * N)
+    _check("msg_norm_index", msg_norm_index, u8, n_iter * shape.n_dir * P)
+    _check("dunary", dunary, f32, N)
+    _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
+    _check("dedge_weights", dedge_weights, f32, shape.n_dir * P)
+    _check("dmsg", dmsg, f32, shape.n_dir * N)
+    with torch.cuda.device(dcost_final.device):
+      rc = lib.mpl_trwp_backward(shape, float(rho), int(n_iter), _ptr(context),
+                                 _ptr(edge_weights), _ptr(dcost_final), _ptr(msg_min_index),
+                                 _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
+                                 _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),
+                                 _Op._stream(dcost_final))
+    _lib.check(rc, "TRWP.backward")
+
+
+class ISGMR(object):
+  """Drop-in for the reference's `lib_stereo.ISGMR` / `lib_seg.ISGMR` extension modules."""
+
+  @staticmethod
+  def forward(enable_sgm, rho, n_iter, enable_min_a_dir, unary, context, edge_weights, msg,
+              cost_final, msg_min_index, msg_norm_index, unary_update, msg_update, label_all):
+    lib = _lib.load()
+    shape, _, N = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
+                                     msg_norm_index, unary_update, label_all, n_iter)
+    _check("msg_update", msg_update, torch.float32, shape.n_dir * N)
+    with torch.cuda.device(unary.device):
+      rc = lib.mpl_isgmr_forward(shape, int(enable_sgm), float(rho), int(n_iter),
+                                 int(enable_min_a_dir), _ptr(unary), _ptr(context),
+                                 _ptr(edge_weights), _ptr(msg), _ptr(cost_final),
+                                 _ptr(msg_min_index), _ptr(msg_norm_index), _ptr(unary_update),
+                                 _ptr(msg_update), _ptr(label_all), _Op._stream(unary))
+    _lib.check(rc, "ISGMR.forward")
+
+  @staticmethod
+  def backward(enable_sgm, rho, context, edge_weights, dcost_final, msg_min_index,
+               msg_norm_index, dunary, dcontext, dedge_weights, dmsg, dunary_update, dmsg_update):
+    lib = _lib.load()
+    shape, n_iter, P, L, ctx2d = _Op._shape_from_index(msg_min_index)
+    N = P * L
+    f32, u8 = torch.float32, torch.uint8
+    _check("context", context, f32, _context_numel(L, ctx2d))
+    _check("edge_weights", edge_weights, f32, shape.n_dir * P)
+    _check("dcost_final", dcost_final, f32, N)
+    _check("msg_min_index", msg_min_index, u8, n_iter * shape.n_dir * N)
+    _check("msg_norm_index", msg_norm_index, u8, n_iter * shape.n_dir * P)
+    _check("dunary", dunary, f32, N)
+    _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
+    _check("dedge_weights", dedge_weights, f32, shape.n_dir * P)
+    _check("dmsg_update", dmsg_update, f32, shape.n_dir * N)
+    with torch.cuda.device(dcost_final.device):
+      rc = lib.mpl_isgmr_backward(shape, int(enable_sgm), float(rho), int(n_iter), _ptr(context),
+                                  _ptr(edge_weights), _ptr(dcost_final), _ptr(msg_min_index),
+                                  _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
+                                  _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),
+                                  _ptr(dmsg_update), _Op._stream(dcost_final))
+    _lib.check(rc, "ISGMR.backward")

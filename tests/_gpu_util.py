@@ -1,0 +1,86 @@
+"""Helpers of the GPU parity tests: run the HIP operators through the reference-style operator
+layer (which calls the C ABI) and compare with the CPU oracle."""
+import numpy as np
+import torch
+
+from mplayers_amd import lib_stereo
+
+DEV = "cuda:0"
+
+
+def _t(a, dtype=torch.float32):
+  return torch.as_tensor(np.ascontiguousarray(a), dtype=dtype).to(DEV).contiguous()
+
+
+def gpu_forward(mode, unary, context, edge_weights, n_dir, n_iter, rho, training=True,
+                saving_label=False, enable_min_a_dir=False, enable_sgm=False, msg_init=None):
+  unary = _t(unary)
+  b, cv, h, w, L = unary.shape
+  context = _t(context)
+  if edge_weights is None:
+    edge_weights = np.ones((n_dir, b, cv, h, w), dtype=np.float32)
+  edge_weights = _t(edge_weights)
+  msg = unary.new_zeros(n_dir, b, cv, h, w, L) if msg_init is None else _t(msg_init)
+  cost = unary.new_zeros(b, cv, h, w, L)
+  scratch = unary.new_zeros(b, cv, h, w, L)
+  u8 = dict(dtype=torch.uint8)
+  imin = unary.new_zeros(n_iter, n_dir, b, cv, h, w, L, **u8) if training else torch.empty(0, **u8)
+  inorm = unary.new_zeros(n_iter, n_dir, b, cv, h, w, **u8) if training else torch.empty(0, **u8)
+  label = unary.new_zeros(n_iter, b, cv, h, w, **u8) if saving_label else torch.empty(0, **u8)
+  if mode == "TRWP":
+    lib_stereo.TRWP.forward(rho, n_iter, int(enable_min_a_dir), unary, context, edge_weights, msg,
+                            cost, imin, inorm, scratch, label)
+  else:
+    msg_update = torch.zeros_like(msg)
+    lib_stereo.ISGMR.forward(int(enable_sgm), rho, n_iter, int(enable_min_a_dir), unary, context,
+                             edge_weights, msg, cost, imin, inorm, scratch, msg_update, label)
+  torch.cuda.synchronize()
+  return dict(msg=msg.cpu().numpy(), cost_final=cost.cpu().numpy(),
+              msg_min_index=imin.cpu().numpy() if training else None,
+              msg_norm_index=inorm.cpu().numpy() if training else None,
+              label_all=label.cpu().numpy() if saving_label else None,
+              _dev=dict(context=context, edge_weights=edge_weights, imin=imin, inorm=inorm))
+
+
+def gpu_backward(mode, context, edge_weights, dcost, msg_min_index, msg_norm_index, rho,
+                 enable_sgm=False, garbage_scratch=False):
+  n_iter, n_dir, b, cv, h, w, L = msg_min_index.shape
+  context = _t(context)
+  if edge_weights is None:
+    edge_weights = np.ones((n_dir, b, cv, h, w), dtype=np.float32)
+  edge_weights = _t(edge_weights)
+  dcost = _t(dcost)
+  imin = _t(msg_min_index, torch.uint8)
+  inorm = _t(msg_norm_index, torch.uint8)
+  dunary = dcost.new_zeros(b, cv, h, w, L)
+  make = (lambda *s: torch.full(s, 7.25, device=DEV)) if garbage_scratch else dcost.new_zeros
+  dmsg = make(n_dir, b, cv, h, w, L)
+  dunary_update = make(b, cv, h, w, L)
+  dedge = dcost.new_zeros(n_dir, b, cv, h, w)
+  dctx = dcost.new_zeros(L, L) if L == 21 else dcost.new_zeros(L)
+  if mode == "TRWP":
+    lib_stereo.TRWP.backward(rho, context, edge_weights, dcost, imin, inorm, dunary, dctx, dedge,
+                             dmsg, dunary_update)
+  else:
+    dmsg_update = make(n_dir, b, cv, h, w, L)
+    lib_stereo.ISGMR.backward(int(enable_sgm), rho, context, edge_weights, dcost, imin, inorm,
+                              dunary, dctx, dedge, dmsg, dunary_update, dmsg_update)
+  torch.cuda.synchronize()
+  return dunary.cpu().numpy(), dctx.cpu().numpy(), dedge.cpu().numpy()
+
+
+def assert_values_close(got, ref, rel=1e-5, what=""):
+  """|got - ref| <= rel * max(1, max|ref|): the 1e-5 relative bar of the parity contract."""
+  scale = max(1.0, float(np.abs(ref).max()))
+  err = float(np.abs(got.astype(np.float64) - ref.astype(np.float64)).max())
+  assert err <= rel * scale, "%s: max abs err %.3e > %.1e * %.3g" % (what, err, rel, scale)
+
+
+def assert_indices_match_off_ties(got, ref, gap, tol, what=""):
+  """Indices must be identical except where the oracle's best and second best candidates are
+  closer than tol (a tie within tolerance)."""
+  bad = got != ref
+  if bad.any():
+    assert float(gap[bad].max()) <= tol, "%s: %d index mismatches, largest gap %.3e > %.1e" % (
+        what, int(bad.sum()), float(gap[bad].max()), tol)
+  return int(bad.sum())

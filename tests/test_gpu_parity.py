@@ -1,0 +1,213 @@
+"""GPU parity: the HIP kernels (called through the C ABI) against the CPU oracle.
+
+Tolerances: messages and beliefs within 1e-5 relative (fp32); argmin indices and labels identical
+except at ties within tolerance; bit-exact on integer-valued inputs where fp32 arithmetic is exact.
+"""
+import zlib
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+  import torch
+  assert torch.cuda.is_available(), "these tests need the MI355X"
+  from mplayers_amd import _lib
+  _lib.load()
+  from tests import _gpu_util
+  return _gpu_util
+
+
+def test_wave_primitives(gpu):
+  import ctypes
+  from mplayers_amd import _lib
+  out = (ctypes.c_int * 8)()
+  _lib.check(_lib.load().mpl_selftest_wave_ops(out), "selftest")
+  assert out[0] == 1, "lanes failing: %08x %08x" % (out[2] & 0xffffffff, out[1] & 0xffffffff)
+
+
+def _seed(*parts):
+  return zlib.crc32(repr(parts).encode())
+
+
+def _context(rng, kind, L):
+  if kind == "tl2":
+    return np.minimum(np.arange(L), 2).astype(np.float32) * 0.25
+  if kind == "tl3":
+    return np.minimum(np.arange(L), 3).astype(np.float32) * 0.3
+  if kind == "tl4":
+    return np.minimum(np.arange(L), 4).astype(np.float32) * 0.5
+  if kind == "potts":
+    c = np.ones(L, dtype=np.float32)
+    c[0] = 0
+    return c
+  if kind == "tq":
+    return np.minimum(np.arange(L) ** 2, 40).astype(np.float32) * 0.05
+  if kind == "npotts":  # negative centre tap, constant elsewhere
+    c = np.zeros(L, dtype=np.float32)
+    c[0] = -1
+    return c
+  if kind == "bump":  # constant tail but c[0] is not the smallest tap
+    c = np.full(L, 0.7, dtype=np.float32)
+    c[0], c[1], c[2] = 0.3, 0.1, 0.5
+    return c
+  if kind == "dense1d":  # no constant tail at all
+    return np.concatenate([[0], rng.random(L - 1)]).astype(np.float32)
+  if kind == "dense2d":
+    return np.triu(rng.random((L, L)), 1).astype(np.float32)
+  raise KeyError(kind)
+
+
+CASES = [
+    # mode, n_dir, B, H, W, L, context kind, n_iter
+    ("ISGMR", 4, 1, 5, 7, 16, "tl4", 2),
+    ("TRWP", 4, 1, 5, 7, 16, "tl4", 2),
+    ("TRWP", 4, 2, 6, 5, 21, "dense2d", 2),
+    ("ISGMR", 8, 2, 6, 5, 21, "dense2d", 2),
+    ("TRWP", 8, 1, 7, 9, 96, "tl2", 2),
+    ("ISGMR", 8, 1, 7, 9, 192, "tl3", 2),
+    ("TRWP", 8, 1, 6, 6, 192, "tl3", 2),
+    ("ISGMR", 4, 1, 6, 6, 256, "tq", 2),
+    ("TRWP", 4, 1, 5, 6, 65, "tl3", 2),
+    ("ISGMR", 4, 1, 5, 6, 97, "potts", 2),
+    ("TRWP", 4, 1, 5, 6, 130, "tq", 2),
+    ("ISGMR", 4, 1, 4, 5, 200, "bump", 2),
+    ("TRWP", 4, 1, 4, 5, 33, "npotts", 2),
+    ("ISGMR", 4, 1, 5, 4, 48, "dense1d", 2),
+    ("TRWP", 8, 1, 5, 4, 70, "dense1d", 1),
+    ("ISGMR", 16, 1, 9, 8, 12, "tl2", 2),
+    ("TRWP", 16, 1, 8, 9, 12, "dense1d", 2),
+    ("ISGMR", 4, 1, 1, 9, 8, "tl2", 2),
+    ("TRWP", 4, 1, 9, 1, 8, "tl2", 2),
+    ("TRWP", 8, 3, 2, 2, 5, "tl2", 3),
+    ("ISGMR", 2, 1, 3, 40, 3, "potts", 3),
+]
+
+
+@pytest.mark.parametrize("mode,n_dir,B,H,W,L,kind,n_iter", CASES)
+@pytest.mark.parametrize("training", [True, False])
+def test_forward_matches_oracle(gpu, oracle, mode, n_dir, B, H, W, L, kind, n_iter, training):
+  rng = np.random.default_rng(_seed(mode, n_dir, L, kind))
+  rho = 0.5 if mode == "TRWP" else 1.0
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32) * 3
+  ctx = _context(rng, kind, L)
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  print("case", mode, n_dir, B, H, W, L, kind, n_iter, training, flush=True)
+  ref = oracle.forward(mode, unary, ctx, ew, n_dir, n_iter, rho, training=training,
+                       saving_label=True, want_gaps=training)
+  got = gpu.gpu_forward(mode, unary, ctx, ew, n_dir, n_iter, rho, training=training,
+                        saving_label=True)
+  gpu.assert_values_close(got["msg"], ref["msg"], what="msg")
+  gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
+  if training:
+    tol = 2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max()))
+    gpu.assert_indices_match_off_ties(got["msg_min_index"], ref["msg_min_index"], ref["gap_min"],
+                                      tol, "msg_min_index")
+    gpu.assert_indices_match_off_ties(got["msg_norm_index"], ref["msg_norm_index"],
+                                      ref["gap_norm"], tol, "msg_norm_index")
+  assert (got["label_all"] != ref["label_all"]).mean() < 0.02
+
+
+@pytest.mark.parametrize("mode,n_dir,L,kind", [
+    ("ISGMR", 8, 16, "int1d"), ("ISGMR", 4, 21, "int2d"), ("TRWP", 4, 70, "int1d"),
+    ("ISGMR", 16, 130, "int_tl"), ("TRWP", 4, 21, "int2d"), ("ISGMR", 4, 192, "int_tl"),
+])
+def test_integer_inputs_are_bit_exact(gpu, oracle, mode, n_dir, L, kind):
+  """Integer-valued inputs (the reference's own test inputs, pytorch/test_parallel_grad.py:
+  102-110) make every fp32 operation exact and produce many exact ties: values, indices and
+  labels must then be identical, tie rules included."""
+  rng = np.random.default_rng(L * 31 + n_dir)
+  B, H, W = 2, 6, 7
+  rho = 0.5 if mode == "TRWP" else 1.0
+  n_iter = 1 if mode == "TRWP" else 3  # rho = 0.5 halves the grid every sweep
+  unary = rng.integers(0, 16, (B, 1, H, W, L)).astype(np.float32) * (4 if mode == "TRWP" else 1)
+  if kind == "int2d":
+    ctx = np.triu(rng.integers(0, 5, (L, L)), 1).astype(np.float32)
+  elif kind == "int_tl":
+    ctx = np.minimum(np.arange(L), 3).astype(np.float32) * 2
+  else:
+    ctx = np.concatenate([[0], rng.integers(0, 5, L - 1)]).astype(np.float32)
+  if mode == "TRWP":
+    ctx = ctx * 4
+  ew = rng.integers(1, 4, (n_dir, B, 1, H, W)).astype(np.float32)
+  print("case", mode, n_dir, L, kind, flush=True)
+  ref = oracle.forward(mode, unary, ctx, ew, n_dir, n_iter, rho, saving_label=True)
+  got = gpu.gpu_forward(mode, unary, ctx, ew, n_dir, n_iter, rho, saving_label=True)
+  for k in ("msg", "cost_final", "msg_min_index", "msg_norm_index", "label_all"):
+    assert np.array_equal(got[k], ref[k]), k
+
+
+def test_negative_edge_weights_take_the_dense_path(gpu, oracle):
+  rng = np.random.default_rng(77)
+  B, H, W, L, n_dir = 1, 5, 6, 40, 4
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ctx = _context(rng, "tl3", L)
+  ew = (rng.random((n_dir, B, 1, H, W)) - 0.3).astype(np.float32)
+  for mode, rho in (("TRWP", 0.5), ("ISGMR", 1.0)):
+    ref = oracle.forward(mode, unary, ctx, ew, n_dir, 2, rho, want_gaps=True)
+    got = gpu.gpu_forward(mode, unary, ctx, ew, n_dir, 2, rho)
+    gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
+    gpu.assert_indices_match_off_ties(got["msg_min_index"], ref["msg_min_index"], ref["gap_min"],
+                                      2e-5, "msg_min_index")
+
+
+@pytest.mark.parametrize("mode,n_dir,B,H,W,L,kind,n_iter", CASES)
+def test_backward_matches_oracle(gpu, oracle, mode, n_dir, B, H, W, L, kind, n_iter):
+  rng = np.random.default_rng(_seed(mode, n_dir, L, kind, 1))
+  rho = 0.5 if mode == "TRWP" else 1.0
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32) * 3
+  ctx = _context(rng, kind, L)
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  dcost = rng.standard_normal(unary.shape).astype(np.float32)
+  print("case", mode, n_dir, B, H, W, L, kind, n_iter, flush=True)
+  # same indices on both sides: the backward pass is checked on its own
+  fwd = oracle.forward(mode, unary, ctx, ew, n_dir, n_iter, rho)
+  ref = oracle.backward(mode, ctx.astype(np.float64), ew.astype(np.float64),
+                        dcost.astype(np.float64), fwd["msg_min_index"], fwd["msg_norm_index"], rho)
+  got = gpu.gpu_backward(mode, ctx, ew, dcost, fwd["msg_min_index"], fwd["msg_norm_index"], rho,
+                         garbage_scratch=True)
+  for g, r, name in zip(got, ref, ("dunary", "dcontext", "dedge_weights")):
+    scale = max(1.0, float(np.abs(r).max()))
+    assert np.abs(g - r).max() <= 1e-4 * scale, (name, float(np.abs(g - r).max()), scale)
+  if ctx.ndim == 2:
+    assert np.all(np.tril(got[1]) == 0)
+  else:
+    assert got[1][0] == 0
+
+
+def test_sgm_flag(gpu, oracle):
+  rng = np.random.default_rng(5)
+  B, H, W, L, n_dir = 1, 6, 7, 24, 8
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ctx = _context(rng, "tl2", L)
+  ref = oracle.forward("SGM", unary, ctx, None, n_dir, 1, 1.0, enable_sgm=True, want_gaps=True)
+  got = gpu.gpu_forward("SGM", unary, ctx, None, n_dir, 1, 1.0, enable_sgm=True)
+  gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
+  dcost = rng.standard_normal(unary.shape).astype(np.float32)
+  r = oracle.backward("SGM", ctx, None, dcost, ref["msg_min_index"], ref["msg_norm_index"], 1.0,
+                      enable_sgm=True)
+  g = gpu.gpu_backward("SGM", ctx, None, dcost, ref["msg_min_index"], ref["msg_norm_index"], 1.0,
+                       enable_sgm=True)
+  for a, b in zip(g, r):
+    assert np.abs(a - b).max() <= 1e-4 * max(1.0, float(np.abs(b).max()))
+
+
+def test_min_a_dir_and_initial_messages(gpu, oracle):
+  rng = np.random.default_rng(9)
+  B, H, W, L, n_dir = 1, 5, 6, 10, 4
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ctx = _context(rng, "tl2", L)
+  for mode, rho in (("TRWP", 0.5), ("ISGMR", 1.0)):
+    ref = oracle.forward(mode, unary, ctx, None, n_dir, 3, rho, enable_min_a_dir=True,
+                         saving_label=True)
+    got = gpu.gpu_forward(mode, unary, ctx, None, n_dir, 3, rho, enable_min_a_dir=True,
+                          saving_label=True)
+    gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final min_a_dir")
+  # TRWP continues from the messages it is given (msg is an in/out tensor in the reference)
+  first = oracle.forward("TRWP", unary, ctx, None, n_dir, 1, 0.5)
+  ref = oracle.forward("TRWP", unary, ctx, None, n_dir, 2, 0.5)
+  got = gpu.gpu_forward("TRWP", unary, ctx, None, n_dir, 1, 0.5, msg_init=first["msg"])
+  gpu.assert_values_close(got["msg"], ref["msg"], what="continued msg")
