@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Benchmark of the TRWP / ISGMR message-passing path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C5] [--alg both|TRWP|ISGMR]
+
+A step is one forward + backward pass of the selected algorithm(s) over one synthetic batch of
+the configuration (default: the large 1500x2000, 192-label, 8-direction one), inputs resident in
+HBM, every buffer pre-allocated as the reference's operator interface has the caller do it; the
+message tensor is re-zeroed inside the timed region (the operators take it as initial messages).
+Prints ONE JSON line: throughput in pixel*label*iter/s, the roofline position of the dominant
+kernel (HIP-event timings taken inside the library on the launch stream during the timed steps)
+and the reference's CPU forward path timed on a bounded crop on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=3)
+  ap.add_argument("--warmup", type=int, default=1)
+  ap.add_argument("--config", default="C5")
+  ap.add_argument("--scale", type=float, default=1.0, help="shrink H and W (debugging only)")
+  ap.add_argument("--alg", default="both", choices=["both", "TRWP", "ISGMR"])
+  ap.add_argument("--fwd-only", action="store_true", help="inference forward only (C2/C3 style)")
+  ap.add_argument("--no-cpu-baseline", action="store_true")
+  return ap.parse_args()
+
+
+def cpu_baseline(cfg, budget_s=20.0):
+  """Times the reference's CPU forward path (built from the reference sources into oracle/_ref)
+  or, where that build is absent, the oracle's restatement of the same loop nest, on a crop of
+  the workload: one iteration, unit edge weights (that path ignores them), forward only (the
+  reference has no CPU backward)."""
+  import numpy as np
+  from oracle import mp_oracle, ref_cpu
+  L, n_dir = cfg["L"], cfg["n_dir"]
+  mode = "TRWP" if cfg["mode"] == "TRWP" else "ISGMR"
+  # cost model of that loop nest: L^2 * n_dir inner steps per pixel and sweep, ~1e9 steps/s/thread
+  threads = 16
+  per_pixel = float(L) * L * n_dir * n_dir
+  pixels = max(64, int(budget_s * 1.0e9 * threads / per_pixel / 4))
+  h = max(2, min(cfg["H"], 32))
+  w = max(2, min(cfg["W"], pixels // h))
+  unary = cfg["unary"][:1, :, :h, :w, :].contiguous().numpy()
+  ctx = cfg["context"].numpy()
+  if ctx.ndim == 1:
+    ii = np.abs(np.arange(L)[:, None] - np.arange(L)[None, :])
+    table = ctx[ii]
+  else:
+    table = ctx + ctx.T
+  table = np.ascontiguousarray(np.broadcast_to(table, (n_dir, L, L)), dtype=np.float32)
+  if ref_cpu.available():
+    kind = "reference"
+    run = lambda: ref_cpu.forward(mode, unary, table, n_dir, 1, cfg["rho"])
+  else:
+    kind = "port"
+    run = lambda: mp_oracle.refcpu_forward(mode, unary, table, n_dir, 1, cfg["rho"],
+                                           n_threads=threads, context_per_dir=True, ctx2d=(L == 21))
+  t0 = time.perf_counter()
+  run()
+  dt = time.perf_counter() - t0
+  units = h * w * L * 1
+  return {"value": units / dt, "unit": "pixel*label*iter/s", "cores": threads, "kind": kind,
+          "sample": "%s forward only (no CPU backward exists), crop %dx%d px of %s, %d labels, "
+                    "%d dirs, 1 iteration, unit edge weights, %.1f s" % (mode, h, w, cfg["name"], L,
+                                                                        n_dir, dt)}
+
+
+def main():
+  a = parse()
+  if a.gpus != 1:
+    print("bench.py: this build drives one GPU only (the path shards by batch item or by "
+          "direction, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+    return 2
+  import torch
+  from mplayers_amd import _lib, lib_stereo, synthetic
+  _lib.load()
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+
+  cfg = synthetic.make_config(a.config, seed=0, scale=a.scale)
+  B, H, W, L, n_dir, n_iter = (cfg[k] for k in ("B", "H", "W", "L", "n_dir", "n_iter"))
+  algs = ["TRWP", "ISGMR"] if a.alg == "both" else [a.alg]
+  training = not a.fwd_only
+  N = B * H * W * L
+  P = B * H * W
+
+  unary = cfg["unary"].to(dev)
+  context = cfg["context"].to(dev)
+  edge = cfg["edge_weights"].to(dev)
+  dcost = synthetic.upstream_grad(cfg).to(dev) if training else None
+  f32 = dict(dtype=torch.float32, device=dev)
+  u8 = dict(dtype=torch.uint8, device=dev)
+  msg = torch.zeros(n_dir, B, 1, H, W, L, **f32)
+  msg_tmp = torch.zeros(n_dir, B, 1, H, W, L, **f32) if "ISGMR" in algs else None
+  cost = torch.zeros(B, 1, H, W, L, **f32)
+  belief = torch.zeros(B, 1, H, W, L, **f32)
+  empty = torch.empty(0, dtype=torch.uint8)
+  if training:
+    imin = torch.zeros(n_iter, n_dir, B, 1, H, W, L, **u8)
+    inorm = torch.zeros(n_iter, n_dir, B, 1, H, W, **u8)
+    dunary = torch.zeros(B, 1, H, W, L, **f32)
+    dmsg = torch.zeros(n_dir, B, 1, H, W, L, **f32)
+    dmsg_tmp = torch.zeros(n_dir, B, 1, H, W, L, **f32) if "ISGMR" in algs else None
+    dscratch = torch.zeros(B, 1, H, W, L, **f32)
+    dedge = torch.zeros(n_dir, B, 1, H, W, **f32)
+    dctx = torch.zeros((L, L) if L == 21 else (L,), **f32)
+  else:
+    imin = inorm = empty
+
+  def step():
+    for alg in algs:
+      rho = 0.5 if alg == "TRWP" else 1.0
+      msg.zero_()
+      if alg == "TRWP":
+        lib_stereo.TRWP.forward(rho, n_iter, 0, unary, context, edge, msg, cost, imin, inorm,
+                                belief, empty)
+        if training:
+          lib_stereo.TRWP.backward(rho, context, edge, dcost, imin, inorm, dunary, dctx, dedge,
+                                   dmsg, dscratch)
+      else:
+        lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, context, edge, msg, cost, imin, inorm,
+                                 belief, msg_tmp, empty)
+        if training:
+          lib_stereo.ISGMR.backward(0, rho, context, edge, dcost, imin, inorm, dunary, dctx,
+                                    dedge, dmsg, dscratch, dmsg_tmp)
+
+  for _ in range(a.warmup):
+    step()
+  torch.cuda.synchronize()
+  _lib.profile_begin()
+  t0 = time.perf_counter()
+  for _ in range(a.steps):
+    step()
+  torch.cuda.synchronize()
+  dt = time.perf_counter() - t0
+  stats = _lib.profile_end()
+
+  units_per_step = cfg["units"] * len(algs)
+  value = units_per_step * a.steps / dt
+
+  # roofline of the dominant kernel: algorithmic bytes per label and direction sweep
+  #   forward 20 B (read S, m_d, m_inv; write m_d, S) + 1 B argmin index + 1/L B norm index when
+  #   training; backward 25 B + 1/L (read index; read+reset h_d; update h_inv; update A).
+  # One launch handles N labels of one direction (TRWP) or of all n_dir directions (ISGMR).
+  fwd_b = (21.0 + 1.0 / L) if training else 20.0
+  bwd_b = 25.0 + 1.0 / L
+  # kind -> (bytes per label and direction sweep, direction sweeps per launch)
+  model = {"fwd_sweep": (fwd_b, 1), "bwd_sweep": (bwd_b, 1),
+           "fwd_sweep_all": (fwd_b, n_dir), "bwd_sweep_all": (bwd_b, n_dir)}
+  kernels = {}
+  for kind, (bpl, dirs_per_launch) in model.items():
+    n, ms = stats[kind]
+    if n == 0:
+      continue
+    per_launch = bpl * N * dirs_per_launch  # algorithmic bytes one launch moves
+    kernels[kind] = {"launches": n, "avg_ms": ms / n, "total_ms": ms,
+                     "bytes_per_launch": per_launch,
+                     "achieved_GBs": per_launch / (ms / n * 1e-3) / 1e9,
+                     "bytes_per_label_sweep": bpl}
+  dominant = max(kernels, key=lambda k: kernels[k]["total_ms"])
+  roofline = {"bound": "hbm", "kernel": dominant, "achieved": kernels[dominant]["achieved_GBs"],
+              "peak": HBM_PEAK_GBS, "unit": "GB/s",
+              "frac": kernels[dominant]["achieved_GBs"] / HBM_PEAK_GBS, "traffic": None,
+              "avg_launch_ms": kernels[dominant]["avg_ms"]}
+  # whole-step roofline fraction against the contract bytes per unit (n_dir * (fwd + bwd))
+  contract = n_dir * (fwd_b + (bwd_b if training else 0.0))
+  whole = contract * value / 1e9 / HBM_PEAK_GBS
+
+  out = {
+      "metric": "pixel*label*iter/s, %s %s" % (" & ".join(algs), "fwd+bwd" if training else "fwd"),
+      "value": value, "unit": "pixel*label*iter/s", "n_gpus": 1, "steps": a.steps,
+      "warmup": a.warmup, "ms_per_step": dt / a.steps * 1e3, "higher_is_better": True,
+      "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+      "config": {"workload": "%s: %s %s, batch %d, grid %dx%d, %d labels, %d directions, %d "
+                             "iterations" % (cfg["name"], "+".join(algs),
+                                             "fwd+bwd" if training else "fwd", B, H, W, L, n_dir,
+                                             n_iter),
+                 "scale": a.scale},
+      "roofline": roofline,
+      "whole_step_frac_of_hbm_roofline": whole,
+      "contract_bytes_per_unit": contract,
+      "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()}
+                  for k, v in kernels.items()},
+      "other_kernels_ms": {k: round(stats[k][1], 3) for k in stats if k not in kernels},
+  }
+  if not a.no_cpu_baseline:
+    out["cpu_baseline"] = cpu_baseline(cfg)
+  print(json.dumps(out))
+  return 0
+
+
+if __name__ == "__main__":
+  sys.exit(main())

@@ -83,8 +83,30 @@ int mpl_isgmr_backward(const mpl_shape* shape, int enable_sgm, float rho, int n_
  * reductions, ballots).  out: 8 host ints, out[0] == 1 when every check passed.  Synchronises. */
 int mpl_selftest_wave_ops(int* out_host);
 
-/* Number of chains of direction `dir` (0..15) on an H x W grid; equals the reference's n_trees
- * (common.cpp:78-87) minus chains that never enter the image.  Host-only helper. */
+/* Per-kernel timing for benchmarks (no counterpart in the reference, which times whole calls with
+ * time.time(), MPLayers/main.py:271-313).  Between mpl_profile_begin() and mpl_profile_end() every
+ * kernel launch of this library is bracketed by HIP events on its own stream; mpl_profile_end()
+ * waits for them and fills stats[kind] for kind < n_stats.  Events cost a few microseconds per
+ * launch; nothing is recorded outside such a bracket.  One bracket at a time per process. */
+#define MPL_KERNEL_FWD_SWEEP 0      /* forward scan of one direction (TRWP) */
+#define MPL_KERNEL_BWD_SWEEP 1      /* reverse scan of one direction (TRWP) */
+#define MPL_KERNEL_BELIEF 2         /* S = unary + sum of messages */
+#define MPL_KERNEL_AGGREGATE 3      /* cost_final */
+#define MPL_KERNEL_LABEL 4          /* per-iteration labels */
+#define MPL_KERNEL_COMBINE 5        /* ISGMR backward: per-iteration gradient recombination */
+#define MPL_KERNEL_OTHER 6
+#define MPL_KERNEL_FWD_SWEEP_ALL 7  /* forward scan of all directions in one launch (ISGMR) */
+#define MPL_KERNEL_BWD_SWEEP_ALL 8  /* reverse scan of all directions in one launch (ISGMR) */
+#define MPL_KERNEL_KINDS 9
+typedef struct mpl_kernel_stat {
+  int launches;
+  double total_ms;
+} mpl_kernel_stat;
+int mpl_profile_begin(void);
+int mpl_profile_end(mpl_kernel_stat* stats, int n_stats);
+
+/* Number of chains of direction `dir` (0..15) on an H x W grid: the reference's n_trees
+ * (common.cpp:78-87).  Host-only helper. */
 int mpl_n_chains(int dir, int height, int width);
 
 /* Message of the last failed call on this thread ("" if none). */

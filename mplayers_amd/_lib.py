@@ -3,16 +3,25 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmplayers_hip.so")
+LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hip.so"))
 
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
-           "mpl_selftest_wave_ops", "mpl_n_chains", "mpl_last_error", "mpl_version")
+           "mpl_selftest_wave_ops", "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
+           "mpl_last_error", "mpl_version")
+
+KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combine", "other",
+                "fwd_sweep_all", "bwd_sweep_all")
 
 
 class Shape(ctypes.Structure):
   """struct mpl_shape"""
   _fields_ = [("n_dir", ctypes.c_int), ("batch", ctypes.c_int), ("height", ctypes.c_int),
               ("width", ctypes.c_int), ("n_disp", ctypes.c_int), ("ctx2d", ctypes.c_int)]
+
+
+class KernelStat(ctypes.Structure):
+  """struct mpl_kernel_stat"""
+  _fields_ = [("launches", ctypes.c_int), ("total_ms", ctypes.c_double)]
 
 
 _lib = None
@@ -36,11 +45,24 @@ def load():
   lib.mpl_isgmr_backward.argtypes = [sp, ci, cf, ci] + [vp] * 12
   lib.mpl_selftest_wave_ops.argtypes = [ctypes.POINTER(ci)]
   lib.mpl_n_chains.argtypes = [ci, ci, ci]
-  lib.mpl_last_error.restype = ctypes.c_char_p
+  lib.mpl_profile_begin.argtypes = []
+  lib.mpl_profile_end.argtypes = [ctypes.POINTER(KernelStat), ci]
   for name in SYMBOLS:
-    getattr(lib, name).restype = getattr(lib, name).restype or ci
+    getattr(lib, name).restype = ci
+  lib.mpl_last_error.restype = ctypes.c_char_p
   _lib = lib
   return lib
+
+
+def profile_begin():
+  check(load().mpl_profile_begin(), "profile_begin")
+
+
+def profile_end():
+  """Returns {kind: (launches, total_ms)} for the kernels launched since profile_begin()."""
+  stats = (KernelStat * len(KERNEL_KINDS))()
+  check(load().mpl_profile_end(stats, len(KERNEL_KINDS)), "profile_end")
+  return {k: (stats[i].launches, stats[i].total_ms) for i, k in enumerate(KERNEL_KINDS)}
 
 
 def check(rc, what):

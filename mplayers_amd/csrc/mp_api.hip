@@ -1,0 +1,610 @@
+// C ABI, host orchestration and the element-wise kernels of the TRWP / ISGMR path (gfx950).
+// The scan kernels live in mp_fwd.hip / mp_bwd.hip; shared device helpers in mp_common.h.
+//
+// Traffic model: instead of re-summing all messages for every sweep (UpdateUnaryKernel of the
+// reference, TRWP_forward.cu:60-80), a belief plane S = unary + sum_k m_k is kept, so a sweep of
+// direction d reads S, m_d, m_inv and writes m_d (and S for TRWP): 20 B per label.  The backward
+// pass keeps the gradient planes as g_k = A + h_k with one shared plane A (which ends up being
+// dunary) for the same reason.
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <mutex>
+#include <vector>
+
+#include "mp_common.h"
+
+using namespace mpl;
+
+namespace {
+
+// 1-D context c[0..L-1]: find the constant tail.  One wave.
+__global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __restrict__ ctx, int L,
+                                                                int ctx2d, CtxDesc* __restrict__ d) {
+  if (threadIdx.x != 0) return;
+  CtxDesc r;
+  r.band_k = 0;
+  r.c0_is_min = 0;
+  r.cmax = 0.f;
+  r.pad = 0;
+  if (!ctx2d) {
+    float tail = ctx[L - 1];
+    int k = L - 1;
+    while (k > 0 && ctx[k - 1] == tail) --k;  // c[k..L-1] == tail
+    bool ok = (tail == tail);
+    bool c0min = true;
+    for (int i = 0; i < L; ++i) {
+      float v = ctx[i];
+      if (!(v <= tail)) ok = false;
+      if (!(ctx[0] <= v)) c0min = false;
+    }
+    if (k < 1) k = 1;  // a constant context: the centre tap alone is the band
+    if (ok && k <= kMaxBandK) {
+      r.band_k = k;
+      r.cmax = tail;
+      r.c0_is_min = c0min ? 1 : 0;
+    }
+  }
+  *d = r;
+}
+
+// ------------------------------------------------------------------------------------------------
+// elementwise kernels
+// ------------------------------------------------------------------------------------------------
+// S = unary + sum_k m_k  (k ascending, as UpdateUnaryKernel sums, TRWP_forward.cu:70-73)
+__global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ unary,
+                                                     const float* __restrict__ msg, int n_dir,
+                                                     int64_t N, float* __restrict__ S) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    float v = unary[i];
+    for (int k = 0; k < n_dir; ++k) v += msg[(int64_t)k * N + i];
+    S[i] = v;
+  }
+}
+
+// cost = factor*unary + sum_k m_k  (or + min_k m_k): CostAggregateKernel, TRWP_forward.cu:31-58,
+// ISGMR_forward.cu:69-99.  copy_to != null: also mirror the message planes there.
+__global__ void __launch_bounds__(256) aggregate_kernel(const float* __restrict__ unary,
+                                                        const float* __restrict__ msg, int n_dir,
+                                                        int64_t N, float factor, int min_a_dir,
+                                                        float* __restrict__ cost,
+                                                        float* __restrict__ copy_to) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    float v = unary[i] * factor;
+    if (min_a_dir) {
+      float mn = msg[i];
+      if (copy_to) copy_to[i] = mn;
+      for (int k = 1; k < n_dir; ++k) {
+        float m = msg[(int64_t)k * N + i];
+        if (copy_to) copy_to[(int64_t)k * N + i] = m;
+        if (m < mn) mn = m;
+      }
+      v += mn;
+    } else {
+      for (int k = 0; k < n_dir; ++k) {
+        float m = msg[(int64_t)k * N + i];
+        if (copy_to) copy_to[(int64_t)k * N + i] = m;
+        v += m;
+      }
+    }
+    cost[i] = v;
+  }
+}
+
+// label = argmin_l cost(l), smallest label on ties: CalLabelKernel, TRWP_forward.cu:8-29, with the
+// cost of CostAggregateKernel recomputed on the fly.  One wave per pixel.
+__global__ void __launch_bounds__(256) label_kernel(const float* __restrict__ unary,
+                                                    const float* __restrict__ msg, int n_dir,
+                                                    int64_t P, int L, float factor, int min_a_dir,
+                                                    uint8_t* __restrict__ label) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t N = P * L;
+  const int64_t wave0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  const int64_t n_waves = ((int64_t)gridDim.x * blockDim.x) / kWave;
+  for (int64_t pix = wave0; pix < P; pix += n_waves) {
+    float best = INFINITY;
+    int arg = 0x7fffffff;
+    for (int l = lane; l < L; l += kWave) {
+      int64_t i = pix * L + l;
+      float v = unary[i] * factor;
+      if (min_a_dir) {
+        float mn = msg[i];
+        for (int k = 1; k < n_dir; ++k) {
+          float m = msg[(int64_t)k * N + i];
+          if (m < mn) mn = m;
+        }
+        v += mn;
+      } else {
+        for (int k = 0; k < n_dir; ++k) v += msg[(int64_t)k * N + i];
+      }
+      if (v < best) {
+        best = v;
+        arg = l;
+      }
+    }
+    float gmin = wave_min(best);
+    // smallest label among the lanes that hold the minimum; a lane's own arg is its smallest
+    float cand = (best == gmin) ? (float)arg : INFINITY;
+    float amin = wave_min(cand);
+    if (lane == 0) label[pix] = (uint8_t)((amin < (float)L) ? (int)amin : 0);
+  }
+}
+
+// ISGMR: after all directions of an iteration have been scanned back (X_k = dU_k):
+//   dunary += rho * sum_k X_k ;  gu_k = rho * (sum - X_k) - X_{k^1}
+// (UpdateUnaryKernelBack summed over directions + SumMsgKernel, ISGMR_backward.cu:39-60, 482-483)
+__global__ void __launch_bounds__(256) isgmr_combine_kernel(float* __restrict__ X, int n_dir,
+                                                            int64_t N, float rho,
+                                                            const float* __restrict__ dcost,
+                                                            float factor, int init_dunary,
+                                                            int write_gu,
+                                                            float* __restrict__ dunary) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    float x[kMaxDirs];
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < kMaxDirs; ++k) {
+      x[k] = (k < n_dir) ? X[(int64_t)k * N + i] : 0.f;
+    }
+    for (int k = n_dir - 1; k >= 0; --k) sum += x[k];
+    float du = init_dunary ? factor * dcost[i] : dunary[i];
+    dunary[i] = fmaf(rho, sum, du);
+    if (write_gu) {
+#pragma unroll
+      for (int k = 0; k < kMaxDirs; ++k)
+        if (k < n_dir) X[(int64_t)k * N + i] = fmaf(rho, sum - x[k], -x[k ^ 1]);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// wave-primitive self test
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(kWave) selftest_kernel(int* out) {
+  const int lane = threadIdx.x;
+  int ok = 1;
+  float x = (float)(lane * 3 % 17) + 100.f;
+  float up = wave_shl1(x, -1.f);
+  float dn = wave_shr1(x, -2.f);
+  float eu = lane < 63 ? (float)((lane + 1) * 3 % 17) + 100.f : -1.f;
+  float ed = lane > 0 ? (float)((lane - 1) * 3 % 17) + 100.f : -2.f;
+  if (up != eu || dn != ed) ok = 0;
+  float y = (float)((lane * 37 + 11) % 64);  // a permutation of 0..63
+  if (wave_min(y) != 0.f) ok = 0;
+  for (int special = 0; special < 64; special += 9)  // the minimum sits in every row and bank
+    if (wave_min(y + (lane == special ? -100.f : 0.f)) != (float)((special * 37 + 11) % 64) - 100.f)
+      ok = 0;
+  if (wave_sum((float)lane) != 2016.f) ok = 0;
+  bool pr[2] = {lane == 5 || lane == 40, lane == 40};
+  if (last_label<2>(pr, -1) != 81) ok = 0;
+  bool pn[2] = {false, false};
+  if (last_label<2>(pn, -7) != -7) ok = 0;
+  uint64_t b = ballot(ok != 0);
+  if (lane == 0) {
+    out[0] = (b == ~0ull) ? 1 : 0;
+    out[1] = (int)(b & 0xffffffffu);
+    out[2] = (int)(b >> 32);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// Optional per-kernel timing with HIP events on the launch stream (off unless mpl_profile_begin
+// was called): lets a benchmark read each kernel's average duration without an external profiler.
+struct ProfRec {
+  int kind;
+  hipEvent_t start, stop;
+};
+struct Profiler {
+  bool on = false;
+  std::vector<ProfRec> recs;
+  std::vector<hipEvent_t> pool;
+  hipEvent_t get_event() {
+    if (!pool.empty()) {
+      hipEvent_t e = pool.back();
+      pool.pop_back();
+      return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+  }
+};
+Profiler g_prof;
+std::mutex g_prof_mu;
+
+struct Timed {
+  hipStream_t st;
+  hipEvent_t stop = nullptr;
+  Timed(int kind, hipStream_t s) : st(s) {
+    if (!g_prof.on) return;
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    ProfRec r;
+    r.kind = kind;
+    r.start = g_prof.get_event();
+    r.stop = g_prof.get_event();
+    if (r.start == nullptr || r.stop == nullptr) return;
+    (void)hipEventRecord(r.start, st);
+    stop = r.stop;
+    g_prof.recs.push_back(r);
+  }
+  ~Timed() {
+    if (stop != nullptr) (void)hipEventRecord(stop, st);
+  }
+};
+
+int check_shape(const mpl_shape* s, int n_iter) {
+  if (s == nullptr) return fail(MPL_EINVAL, "shape is null");
+  if (s->n_dir < 2 || s->n_dir > kMaxDirs || (s->n_dir & 1))
+    return fail(MPL_EINVAL, "n_dir must be even and in [2, %d], got %d", kMaxDirs, s->n_dir);
+  if (s->batch < 1 || s->height < 1 || s->width < 1)
+    return fail(MPL_EINVAL, "batch/height/width must be positive, got %d/%d/%d", s->batch,
+                s->height, s->width);
+  if (s->n_disp < 1 || s->n_disp > kMaxL)
+    return fail(MPL_EINVAL, "n_disp must be in [1, %d] (uint8 argmin indices), got %d", kMaxL,
+                s->n_disp);
+  if (s->ctx2d && s->n_disp > kMaxCtx2dL)
+    return fail(MPL_EINVAL, "a 2-D context table needs n_disp <= %d, got %d", kMaxCtx2dL,
+                s->n_disp);
+  if (n_iter < 1) return fail(MPL_EINVAL, "n_iter must be positive, got %d", n_iter);
+  int64_t P = (int64_t)s->batch * s->height * s->width;
+  if (P > 0x7fffffff) return fail(MPL_EINVAL, "more than 2^31 pixels");
+  // pixels are addressed with 32-bit byte offsets from the first pixel of their batch item
+  if ((int64_t)s->height * s->width * s->n_disp * 4 > 0xffffffffll)
+    return fail(MPL_EINVAL, "one batch item (height*width*n_disp floats) must stay below 4 GiB");
+  int64_t max_blocks = 0;
+  for (int d = 0; d < s->n_dir; ++d)
+    max_blocks += (int64_t)s->batch * make_dir(d, s->height, s->width).n_chains;
+  if (max_blocks > 0x7fffffff) return fail(MPL_EINVAL, "more than 2^31 chains");
+  return MPL_OK;
+}
+
+int launch_ok(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MPL_ELAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return MPL_OK;
+}
+
+int elementwise_blocks(int64_t n) {
+  int64_t b = (n + 256 * 4 - 1) / (256 * 4);
+  if (b < 1) b = 1;
+  if (b > 256 * 32) b = 256 * 32;
+  return (int)b;
+}
+
+void fill_dirs(const mpl_shape* s, int first, int count, int* dirs, int* prefix, int* n_dirs) {
+  *n_dirs = count;
+  prefix[0] = 0;
+  for (int i = 0; i < count; ++i) {
+    dirs[i] = first + i;
+    prefix[i + 1] = prefix[i] + s->batch * make_dir(first + i, s->height, s->width).n_chains;
+  }
+}
+
+void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+  Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st);
+  switch ((p.L + kWave - 1) / kWave) {
+    case 1: launch_sweep_fwd<1>(p, train, jacobi, st); break;
+    case 2: launch_sweep_fwd<2>(p, train, jacobi, st); break;
+    case 3: launch_sweep_fwd<3>(p, train, jacobi, st); break;
+    default: launch_sweep_fwd<4>(p, train, jacobi, st); break;
+  }
+}
+
+void launch_bwd(const BackParams& p, bool jacobi, hipStream_t st) {
+  Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st);
+  switch ((p.L + kWave - 1) / kWave) {
+    case 1: launch_sweep_bwd<1>(p, jacobi, st); break;
+    case 2: launch_sweep_bwd<2>(p, jacobi, st); break;
+    case 3: launch_sweep_bwd<3>(p, jacobi, st); break;
+    default: launch_sweep_bwd<4>(p, jacobi, st); break;
+  }
+}
+
+SweepParams base_fwd_params(const mpl_shape* s, float rho, const float* edge, const float* ctx,
+                            const CtxDesc* desc) {
+  SweepParams p;
+  memset(&p, 0, sizeof(p));
+  p.B = s->batch;
+  p.H = s->height;
+  p.W = s->width;
+  p.L = s->n_disp;
+  p.ctx2d = s->ctx2d ? 1 : 0;
+  p.rho = rho;
+  p.edge = edge;
+  p.ctx = ctx;
+  p.desc = desc;
+  return p;
+}
+
+// cost_final is not written before the final aggregation, so its first bytes carry the context
+// descriptor during the sweeps (no allocation, no state shared between streams).
+const CtxDesc* make_desc(const mpl_shape* s, const float* ctx, float* cost_final, hipStream_t st) {
+  int64_t N = (int64_t)s->batch * s->height * s->width * s->n_disp;
+  if (N * (int64_t)sizeof(float) < (int64_t)sizeof(CtxDesc)) return nullptr;  // dense path
+  CtxDesc* d = reinterpret_cast<CtxDesc*>(cost_final);
+  Timed timed(MPL_KERNEL_OTHER, st);
+  analyze_context_kernel<<<1, kWave, 0, st>>>(ctx, s->n_disp, s->ctx2d ? 1 : 0, d);
+  return d;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------------
+extern "C" {
+
+const char* mpl_last_error(void) { return g_err; }
+
+int mpl_version(void) { return 100; }
+
+int mpl_profile_begin(void) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  for (auto& r : g_prof.recs) {
+    g_prof.pool.push_back(r.start);
+    g_prof.pool.push_back(r.stop);
+  }
+  g_prof.recs.clear();
+  g_prof.on = true;
+  return MPL_OK;
+}
+
+int mpl_profile_end(mpl_kernel_stat* stats, int n_stats) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof.on = false;
+  for (int i = 0; i < n_stats; ++i) {
+    stats[i].launches = 0;
+    stats[i].total_ms = 0.0;
+  }
+  int rc = MPL_OK;
+  for (auto& r : g_prof.recs) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(r.stop);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, r.start, r.stop);
+    if (e != hipSuccess) {
+      rc = fail(MPL_ELAUNCH, "profile_end: %s", hipGetErrorString(e));
+    } else if (r.kind >= 0 && r.kind < n_stats) {
+      stats[r.kind].launches += 1;
+      stats[r.kind].total_ms += ms;
+    }
+    g_prof.pool.push_back(r.start);
+    g_prof.pool.push_back(r.stop);
+  }
+  g_prof.recs.clear();
+  return rc;
+}
+
+int mpl_n_chains(int dir, int height, int width) {
+  if (dir < 0 || dir >= kMaxDirs || height < 1 || width < 1) return -1;
+  return make_dir(dir, height, width).n_chains;
+}
+
+int mpl_selftest_wave_ops(int* out_host) {
+  if (out_host == nullptr) return fail(MPL_EINVAL, "out_host is null");
+  int* d = nullptr;
+  if (hipMalloc(&d, 8 * sizeof(int)) != hipSuccess) return fail(MPL_ELAUNCH, "hipMalloc failed");
+  (void)hipMemset(d, 0, 8 * sizeof(int));
+  selftest_kernel<<<1, kWave>>>(d);
+  hipError_t e = hipDeviceSynchronize();
+  if (e == hipSuccess) e = hipMemcpy(out_host, d, 8 * sizeof(int), hipMemcpyDeviceToHost);
+  (void)hipFree(d);
+  if (e != hipSuccess) return fail(MPL_ELAUNCH, "selftest: %s", hipGetErrorString(e));
+  return MPL_OK;
+}
+
+int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a_dir,
+                     const float* unary, const float* context, const float* edge_weights,
+                     float* msg, float* cost_final, uint8_t* msg_min_index,
+                     uint8_t* msg_norm_index, float* unary_update, uint8_t* label_all,
+                     void* stream) {
+  int rc = check_shape(s, n_iter);
+  if (rc) return rc;
+  if (!unary || !context || !edge_weights || !msg || !cost_final || !unary_update)
+    return fail(MPL_EINVAL, "trwp_forward: null tensor pointer");
+  if ((msg_min_index == nullptr) != (msg_norm_index == nullptr))
+    return fail(MPL_EINVAL, "trwp_forward: msg_min_index and msg_norm_index go together");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t P = (int64_t)s->batch * s->height * s->width;
+  const int64_t N = P * s->n_disp;
+  const bool train = msg_min_index != nullptr;
+
+  const CtxDesc* desc = make_desc(s, context, cost_final, st);
+  {
+    Timed timed(MPL_KERNEL_BELIEF, st);
+    belief_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, msg, s->n_dir, N, unary_update);
+  }
+
+  SweepParams p = base_fwd_params(s, rho, edge_weights, context, desc);
+  p.belief = unary_update;
+  p.belief_out = unary_update;
+  p.msg_in = msg;
+  p.msg_out = msg;
+  for (int it = 0; it < n_iter; ++it) {
+    for (int d = 0; d < s->n_dir; ++d) {  // Gauss-Seidel over directions: TRWP_forward.cu:440-518
+      fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
+      if (train) {
+        p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
+        p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
+      }
+      launch_fwd(p, train, false, st);
+    }
+    if (label_all) {
+      int64_t waves = (P < 256 * 64) ? P : 256 * 64;
+      Timed timed(MPL_KERNEL_LABEL, st);
+      label_kernel<<<(int)((waves + 3) / 4), 256, 0, st>>>(unary, msg, s->n_dir, P, s->n_disp, 1.f,
+                                                           enable_min_a_dir, label_all + it * P);
+    }
+  }
+  {
+    Timed timed(MPL_KERNEL_AGGREGATE, st);
+    aggregate_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, msg, s->n_dir, N, 1.f,
+                                                            enable_min_a_dir, cost_final, nullptr);
+  }
+  return launch_ok("trwp_forward");
+}
+
+int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
+                      int enable_min_a_dir, const float* unary, const float* context,
+                      const float* edge_weights, float* msg, float* cost_final,
+                      uint8_t* msg_min_index, uint8_t* msg_norm_index, float* unary_update,
+                      float* msg_update, uint8_t* label_all, void* stream) {
+  int rc = check_shape(s, n_iter);
+  if (rc) return rc;
+  if (!unary || !context || !edge_weights || !msg || !cost_final || !unary_update || !msg_update)
+    return fail(MPL_EINVAL, "isgmr_forward: null tensor pointer");
+  if ((msg_min_index == nullptr) != (msg_norm_index == nullptr))
+    return fail(MPL_EINVAL, "isgmr_forward: msg_min_index and msg_norm_index go together");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t P = (int64_t)s->batch * s->height * s->width;
+  const int64_t N = P * s->n_disp;
+  const bool train = msg_min_index != nullptr;
+  const float factor = enable_sgm ? (float)s->n_dir : 1.f;
+
+  const CtxDesc* desc = make_desc(s, context, cost_final, st);
+  SweepParams p = base_fwd_params(s, rho, edge_weights, context, desc);
+  p.belief = unary_update;
+  p.belief_out = nullptr;
+  fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
+  float* buf[2] = {msg, msg_update};
+  for (int it = 0; it < n_iter; ++it) {
+    // Jacobi over directions (ISGMR_forward.cu:506-622): every direction reads the old messages;
+    // the two buffers alternate instead of being copied.
+    const float* cur = buf[it & 1];
+    float* nxt = buf[(it + 1) & 1];
+    {
+      Timed timed(MPL_KERNEL_BELIEF, st);
+      belief_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, cur, s->n_dir, N, unary_update);
+    }
+    p.msg_in = cur;
+    p.msg_out = nxt;
+    if (train) {
+      p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
+      p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
+    }
+    launch_fwd(p, train, true, st);
+    if (label_all) {
+      int64_t waves = (P < 256 * 64) ? P : 256 * 64;
+      Timed timed(MPL_KERNEL_LABEL, st);
+      label_kernel<<<(int)((waves + 3) / 4), 256, 0, st>>>(unary, nxt, s->n_dir, P, s->n_disp,
+                                                           factor, enable_min_a_dir,
+                                                           label_all + it * P);
+    }
+  }
+  const float* fin = buf[n_iter & 1];
+  {
+    Timed timed(MPL_KERNEL_AGGREGATE, st);
+    aggregate_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, fin, s->n_dir, N, factor,
+                                                            enable_min_a_dir, cost_final,
+                                                            (n_iter & 1) ? msg : nullptr);
+  }
+  return launch_ok("isgmr_forward");
+}
+
+int mpl_trwp_backward(const mpl_shape* s, float rho, int n_iter, const float* context,
+                      const float* edge_weights, const float* dcost_final,
+                      const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
+                      float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
+                      void* stream) {
+  (void)dunary_update;
+  int rc = check_shape(s, n_iter);
+  if (rc) return rc;
+  if (!context || !edge_weights || !dcost_final || !msg_min_index || !msg_norm_index || !dunary ||
+      !dcontext || !dedge_weights || !dmsg)
+    return fail(MPL_EINVAL, "trwp_backward: null tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t P = (int64_t)s->batch * s->height * s->width;
+  const int64_t N = P * s->n_disp;
+
+  BackParams p;
+  memset(&p, 0, sizeof(p));
+  p.B = s->batch;
+  p.H = s->height;
+  p.W = s->width;
+  p.L = s->n_disp;
+  p.ctx2d = s->ctx2d ? 1 : 0;
+  p.rho = rho;
+  p.a_out = dunary;
+  p.h = dmsg;
+  p.edge = edge_weights;
+  p.ctx = context;
+  p.dedge = dedge_weights;
+  p.dctx = dcontext;
+  bool first = true;
+  for (int it = n_iter - 1; it >= 0; --it) {
+    for (int d = s->n_dir - 1; d >= 0; --d) {  // TRWP_backward.cu:337-424
+      fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
+      p.a_in = first ? dcost_final : dunary;  // CostAggregateKernelBack: every g_k starts as dcost
+      p.first_touch = (it == n_iter - 1) && (d & 1);
+      p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
+      p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
+      launch_bwd(p, false, st);
+      first = false;
+    }
+  }
+  return launch_ok("trwp_backward");
+}
+
+int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
+                       const float* context, const float* edge_weights, const float* dcost_final,
+                       const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
+                       float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
+                       float* dmsg_update, void* stream) {
+  (void)dmsg;
+  (void)dunary_update;
+  int rc = check_shape(s, n_iter);
+  if (rc) return rc;
+  if (!context || !edge_weights || !dcost_final || !msg_min_index || !msg_norm_index || !dunary ||
+      !dcontext || !dedge_weights || !dmsg_update)
+    return fail(MPL_EINVAL, "isgmr_backward: null tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t P = (int64_t)s->batch * s->height * s->width;
+  const int64_t N = P * s->n_disp;
+  const float factor = enable_sgm ? (float)s->n_dir : 1.f;
+
+  BackParams p;
+  memset(&p, 0, sizeof(p));
+  p.B = s->batch;
+  p.H = s->height;
+  p.W = s->width;
+  p.L = s->n_disp;
+  p.ctx2d = s->ctx2d ? 1 : 0;
+  p.rho = rho;
+  p.du_out = dmsg_update;
+  p.edge = edge_weights;
+  p.ctx = context;
+  p.dedge = dedge_weights;
+  p.dctx = dcontext;
+  fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
+  for (int it = n_iter - 1; it >= 0; --it) {
+    const bool first = (it == n_iter - 1);
+    p.gu_in = first ? dcost_final : dmsg_update;  // gu_k = dcost_final for every k at the start
+    p.gu_stride = first ? 0 : N;
+    p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
+    p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
+    launch_bwd(p, true, st);
+    Timed timed(MPL_KERNEL_COMBINE, st);
+    isgmr_combine_kernel<<<elementwise_blocks(N), 256, 0, st>>>(
+        dmsg_update, s->n_dir, N, rho, dcost_final, factor, first ? 1 : 0, it > 0 ? 1 : 0, dunary);
+  }
+  return launch_ok("isgmr_backward");
+}
+
+}  // extern "C"

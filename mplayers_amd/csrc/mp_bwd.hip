@@ -1,0 +1,345 @@
+// Reverse scan of TRWP / ISGMR for gfx950: one wavefront per chain, see mp_common.h.
+//
+// Follows HorizontalKernelBack / DiagonalKernelWideBack / DiagonalKernelNarrowBack
+// (TRWP_backward.cu:49-275, ISGMR_backward.cu:62-288) fused with UpdateUnaryKernelBack
+// (TRWP_backward.cu:26-47) and the memsets after it (:421-422).  Per pixel p, visited in reverse
+// chain order, with g the gradient w.r.t. the normalised message of p:
+//     g[norm_index[p]] -= sum(g)                                    (MsgNormNaiveBack)
+//     for cd: fd = min_index[p, cd];  dU[q, fd] += g[cd];  g_dir[q, fd] += rho * g[cd]
+//             dedge[p] += ctx(cd, fd) * g[cd];  dctx[ctx index] += w[p] * g[cd]  if cd != fd
+// The scatter target dU[q, :] stays in LDS/registers: it is the only thing the next step needs.
+//
+// TRWP keeps the per-direction gradient planes as g_k = A + h_k (A ends up being dunary), so the
+// "for all k" updates of UpdateUnaryKernelBack touch one plane instead of n_dir.
+//
+// Compiled once per R (labels per lane) with -DMPL_INST_R=<R>.
+
+#include "mp_common.h"
+
+namespace mpl {
+namespace {
+
+// LDS float atomics cost ~190 clocks per wave instruction on this hardware and serialise per CU,
+// so the common cases of the scatter and of the dcontext histogram are done without them:
+//   * argmin indices that point at the two most popular targets of the pixel (taken from the first
+//     and the last label; with a truncated pairwise term nearly every label points at argmin(a))
+//     are summed with a wave reduction,
+//   * indices within kNear labels of their own label are moved with DPP label shifts,
+//   * only what is left goes through LDS atomics.
+constexpr int kNear = 3;
+
+template <int R>
+struct PixB {
+  float a[R], hd[R], hi[R];
+  int fd[R];
+  int nidx;
+  float w, de;
+};
+
+template <int R, bool VEC, bool MASK, bool JACOBI>
+__global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
+  extern __shared__ float smem[];
+  const int L = p.L;
+  const int n_ctx = p.ctx2d ? L * L : L;
+  float* sc_s = smem;              // kMaxL floats: scatter target of the slow path
+  float* g0_s = sc_s + kMaxL;      // kMaxL floats: weighted gradients of popular class 0, by label
+  float* g1_s = g0_s + kMaxL;      // same for class 1
+  float* ctx_s = g1_s + kMaxL;     // context table
+  float* hist_s = ctx_s + n_ctx;   // dcontext accumulator of the slow path (and of 2-D contexts)
+  const int lane = threadIdx.x;
+  const int64_t P = (int64_t)p.B * p.H * p.W;
+  const int64_t N = P * L;
+  const ChainCtx ch = locate_chain(p);
+  const int dir = ch.dir;
+  const int n = ch.n;
+
+  for (int i = lane; i < n_ctx; i += kWave) {
+    ctx_s[i] = p.ctx[i];
+    hist_s[i] = 0.f;
+  }
+  for (int i = lane; i < 3 * kMaxL; i += kWave) sc_s[i] = 0.f;  // sc_s, g0_s, g1_s
+  __syncthreads();
+
+  const int64_t HW = (int64_t)p.H * p.W;
+  const int64_t img_p = (int64_t)ch.bv * HW;  // first pixel of this batch item
+  const int64_t img_e = img_p * L;
+  const int vbytes = L * 4;
+  const bool read_h = !JACOBI && !p.first_touch;
+  // plane bases of this batch item and direction; label-vector descriptors are formed per access
+  const float* __restrict__ bA = (JACOBI ? p.gu_in + (int64_t)dir * p.gu_stride : p.a_in) + img_e;
+  float* __restrict__ bAo = (JACOBI ? p.du_out + (int64_t)dir * N : p.a_out) + img_e;
+  float* hbase = JACOBI ? p.du_out : p.h;  // Jacobi never touches these two planes
+  float* __restrict__ bHd = hbase + (int64_t)dir * N + img_e;
+  float* __restrict__ bHi = hbase + (int64_t)(dir ^ 1) * N + img_e;
+  const uint8_t* __restrict__ bImin = p.idx_min + (int64_t)dir * N + img_e;
+  const int img_bytes_p = (int)(HW * 4 > 0x7fffffff ? 0x7fffffff : HW * 4);
+  const rsrc_t dInorm = make_rsrc(p.idx_norm + (int64_t)dir * P + img_p, (int)HW);
+  const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P + img_p, img_bytes_p);
+  const rsrc_t dDe = make_rsrc(p.dedge + (int64_t)dir * P + img_p, img_bytes_p);
+  const float rho = p.rho;
+  const int lab0 = R * lane;
+  const int foff = lab0 * 4;
+
+  bool valid[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) valid[j] = MASK ? (lab0 + j < L) : true;
+
+  // loads run from the last pixel of the chain down to the first; past it the first is refetched
+  int ld_t = n - 1;
+  int ld_p = ch.pix0 + (n - 1) * ch.pstep;
+  auto load_next = [&]() {
+    PixB<R> r;
+    const unsigned pp = (unsigned)uniform_i(ld_t >= 0 ? ld_p : ch.pix0);
+    const unsigned so = pp * (unsigned)vbytes;
+    const int nrec = (int)(so + (unsigned)vbytes);
+    buf_load<R, VEC>(make_rsrc(bA, nrec), foff, so, r.a);
+    if (!JACOBI) {
+      // before the first write of these planes they count as zero: an empty descriptor reads 0
+      buf_load<R, VEC>(make_rsrc(bHd, read_h ? nrec : 0), foff, so, r.hd);
+      buf_load<R, VEC>(make_rsrc(bHi, read_h ? nrec : 0), foff, so, r.hi);
+    } else {
+#pragma unroll
+      for (int j = 0; j < R; ++j) r.hd[j] = r.hi[j] = 0.f;
+    }
+    buf_load_u8<R, VEC>(make_rsrc(bImin, (int)(pp * (unsigned)L + (unsigned)L)), lab0,
+                        pp * (unsigned)L, r.fd);
+    r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, 0, pp, 0);
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, 0, pp * 4u, 0));
+    r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dDe, 0, pp * 4u, 0));
+    ld_t -= 1;
+    ld_p -= ch.pstep;
+    return r;
+  };
+
+  PixB<R> ring[kPrefetch];
+#pragma unroll
+  for (int u = 0; u < kPrefetch; ++u) ring[u] = load_next();
+
+  float sc[R];  // dU of the current pixel: what the previous step scattered into it
+  float hist_reg[R];        // dcontext[label] partial sums of this lane's own labels (1-D context)
+  float near_acc[kNear + 1];  // dcontext[k] partial sums for k <= kNear (1-D context)
+#pragma unroll
+  for (int j = 0; j < R; ++j) sc[j] = hist_reg[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k <= kNear; ++k) near_acc[k] = 0.f;
+  const int last_lane = (L - 1) / R, last_reg = (L - 1) % R;
+
+  int st_p = ch.pix0 + (n - 1) * ch.pstep;
+  for (int s0 = 0; s0 < n; s0 += kPrefetch) {
+#pragma unroll
+    for (int u = 0; u < kPrefetch; ++u) {
+      const int t = n - 1 - (s0 + u);
+      const PixB<R> px = ring[u];
+      ring[u] = load_next();
+      float scn[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) scn[j] = 0.f;
+      float det = 0.f;
+      if (t >= 1) {  // the chain start (t == 0) has no incoming edge
+        const float w = uniform_f(px.w);
+        const int nidx = __builtin_amdgcn_readfirstlane(px.nidx);
+        float gv[R];
+        float part = 0.f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          // gradient w.r.t. the normalised message of this pixel, including what the previous
+          // step added through the recurrence (dmsg[front] += rho * value, TRWP_backward.cu:108)
+          float base = JACOBI ? px.a[j] : (px.a[j] + px.hd[j]);
+          gv[j] = valid[j] ? fmaf(rho, sc[j], base) : 0.f;
+          part += gv[j];
+        }
+        const float tot = wave_sum(part);  // MsgNormNaiveBack, commonCUDA.cuh:131-145
+        // the two popular targets: where the first and the last label point
+        const int f0 = __builtin_amdgcn_readlane(px.fd[0], 0);
+        int f1 = 0;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          int v = __builtin_amdgcn_readlane(px.fd[j], last_lane);
+          f1 = (j == last_reg) ? v : f1;
+        }
+        int off[R];
+        bool m0[R], m1[R], rem[R], left[R];
+        float p0 = 0.f, p1 = 0.f, de = 0.f;
+        bool any_left = false;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const int cd = lab0 + j, fd = px.fd[j];
+          if (cd == nidx) gv[j] -= tot;
+          off[j] = fd - cd;
+          m0[j] = fd == f0;
+          m1[j] = (fd == f1) && !m0[j];
+          rem[j] = !m0[j] && !m1[j];
+          const int ao = off[j] < 0 ? -off[j] : off[j];
+          left[j] = rem[j] && (ao > kNear) && valid[j];
+          any_left = any_left || left[j];
+          p0 += m0[j] ? gv[j] : 0.f;
+          p1 += m1[j] ? gv[j] : 0.f;
+          // dedge_weights[cur] += ctx(cd, fd) * value
+          const int ci = !valid[j] ? 0 : (p.ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
+          de = fmaf(ctx_s[ci], gv[j], de);
+        }
+        const float s0sum = wave_sum(p0);
+        const float s1sum = wave_sum(p1);
+        // near targets: sc_next[l] += g[l - o] where index(l - o) == l, |o| <= kNear
+        float tp[R], tn[R], near_t[kNear + 1];
+#pragma unroll
+        for (int j = 0; j < R; ++j) tp[j] = tn[j] = 0.f;
+#pragma unroll
+        for (int o = kNear; o >= 1; --o) {
+          float cp[R], cn[R];
+          near_t[o] = 0.f;
+#pragma unroll
+          for (int j = 0; j < R; ++j) {
+            cp[j] = (rem[j] && off[j] == o) ? gv[j] : 0.f;
+            cn[j] = (rem[j] && off[j] == -o) ? gv[j] : 0.f;
+            near_t[o] += cp[j] + cn[j];
+            tp[j] += cp[j];
+            tn[j] += cn[j];
+          }
+          // move one label up (tp) / down (tn)
+          const float up_in = wave_shr1(tp[R - 1], 0.f);
+          const float dn_in = wave_shl1(tn[0], 0.f);
+#pragma unroll
+          for (int j = R - 1; j > 0; --j) tp[j] = tp[j - 1];
+          tp[0] = up_in;
+#pragma unroll
+          for (int j = 0; j < R - 1; ++j) tn[j] = tn[j + 1];
+          tn[R - 1] = dn_in;
+        }
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const int cd = lab0 + j;
+          float own = (rem[j] && off[j] == 0) ? gv[j] : 0.f;
+          scn[j] = own + tp[j] + tn[j] + (cd == f0 ? s0sum : 0.f) + (cd == f1 ? s1sum : 0.f);
+        }
+        // dcontext += edge_weight * value where cd != fd (TRWP_backward.cu:111-112)
+        if (!p.ctx2d) {
+#pragma unroll
+          for (int o = 1; o <= kNear; ++o) near_acc[o] = fmaf(w, near_t[o], near_acc[o]);
+          // popular classes: bin |cd - f| is reached from labels f + k and f - k; gather through LDS
+#pragma unroll
+          for (int j = 0; j < R; ++j)
+            if (valid[j]) g0_s[lab0 + j] = m0[j] ? w * gv[j] : 0.f;
+          __syncthreads();
+#pragma unroll
+          for (int j = 0; j < R; ++j) {
+            const int k = lab0 + j;
+            const int hi_l = f0 + k, lo_l = f0 - k;
+            float a = (k >= 1 && hi_l < L) ? g0_s[hi_l < L ? hi_l : 0] : 0.f;
+            float b = (k >= 1 && lo_l >= 0) ? g0_s[lo_l >= 0 ? lo_l : 0] : 0.f;
+            hist_reg[j] += a + b;
+          }
+          if (f1 != f0) {
+#pragma unroll
+            for (int j = 0; j < R; ++j)
+              if (valid[j]) g1_s[lab0 + j] = m1[j] ? w * gv[j] : 0.f;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+              const int k = lab0 + j;
+              const int hi_l = f1 + k, lo_l = f1 - k;
+              float a = (k >= 1 && hi_l < L) ? g1_s[hi_l < L ? hi_l : 0] : 0.f;
+              float b = (k >= 1 && lo_l >= 0) ? g1_s[lo_l >= 0 ? lo_l : 0] : 0.f;
+              hist_reg[j] += a + b;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < R; ++j) {
+            const int cd = lab0 + j, fd = px.fd[j];
+            if (valid[j] && cd != fd)
+              atomicAdd(&hist_s[cd < fd ? cd * L + fd : fd * L + cd], w * gv[j]);
+          }
+        }
+        // whatever is neither popular nor near: LDS atomics
+        if (ballot(any_left) != 0) {
+#pragma unroll
+          for (int j = 0; j < R; ++j) {
+            if (left[j]) {
+              atomicAdd(&sc_s[px.fd[j]], gv[j]);
+              if (!p.ctx2d) atomicAdd(&hist_s[off[j] < 0 ? -off[j] : off[j]], w * gv[j]);
+            }
+          }
+          __syncthreads();
+#pragma unroll
+          for (int j = 0; j < R; ++j)
+            if (valid[j]) scn[j] += atomicExch(&sc_s[lab0 + j], 0.f);  // read and clear
+        }
+        det = wave_sum(de);
+      }
+      // pixel-local part of UpdateUnaryKernelBack with dU[pix] = sc; nothing is stored for t < 0
+      const unsigned sp = (unsigned)uniform_i(st_p);
+      const unsigned so = sp * (unsigned)vbytes;
+      const int nrec = t >= 0 ? (int)(so + (unsigned)vbytes) : 0;
+      if (JACOBI) {
+        buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, sc);
+      } else {
+        float an[R], hdn[R], hin[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          an[j] = fmaf(rho, sc[j], px.a[j]);  // g_k += rho*dU for every k, dunary too
+          hdn[j] = -an[j];                    // g_dir = 0 after its sweep
+          hin[j] = px.hi[j] - sc[j];          // g_inv -= dU
+        }
+        buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, an);
+        buf_store<R, VEC>(make_rsrc(bHd, nrec), foff, so, hdn);
+        buf_store<R, VEC>(make_rsrc(bHi, nrec), foff, so, hin);
+      }
+      // each pixel receives over exactly one edge per direction: plain read-modify-write
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
+                                            t >= 1 ? 0 : kDeadOffset, sp * 4u, 0);
+#pragma unroll
+      for (int j = 0; j < R; ++j) sc[j] = scn[j];
+      st_p -= ch.pstep;
+    }
+  }
+  __syncthreads();
+  for (int i = lane; i < n_ctx; i += kWave) {
+    float v = hist_s[i];
+    if (v != 0.f) atomicAdd(&p.dctx[i], v);
+  }
+  if (!p.ctx2d) {
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+      if (valid[j] && hist_reg[j] != 0.f) atomicAdd(&p.dctx[lab0 + j], hist_reg[j]);
+#pragma unroll
+    for (int k = 1; k <= kNear; ++k) {
+      const float v = wave_sum(near_acc[k]);
+      if (lane == 0 && k < L && v != 0.f) atomicAdd(&p.dctx[k], v);
+    }
+  }
+}
+
+template <int R, bool VEC, bool MASK>
+void launch_vm(const BackParams& p, bool jacobi, hipStream_t st) {
+  const int blocks = p.block_prefix[p.n_dirs];
+  const size_t lds =
+      sizeof(float) * (3 * kMaxL + 2 * (p.ctx2d ? p.L * p.L : p.L));
+  if (jacobi)
+    sweep_bwd_kernel<R, VEC, MASK, true><<<blocks, kWave, lds, st>>>(p);
+  else
+    sweep_bwd_kernel<R, VEC, MASK, false><<<blocks, kWave, lds, st>>>(p);
+}
+
+}  // namespace
+
+template <int R>
+void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st) {
+  if (p.block_prefix[p.n_dirs] <= 0) return;
+  const bool vec = (p.L % R) == 0;
+  const bool mask = p.L != R * kWave;
+  if constexpr (R > 1) {
+    if (!vec) {
+      launch_vm<R, false, true>(p, jacobi, st);
+      return;
+    }
+  }
+  if (mask)
+    launch_vm<R, true, true>(p, jacobi, st);
+  else
+    launch_vm<R, true, false>(p, jacobi, st);
+}
+
+template void launch_sweep_bwd<MPL_INST_R>(const BackParams&, bool, hipStream_t);
+
+}  // namespace mpl

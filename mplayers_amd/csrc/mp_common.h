@@ -1,0 +1,355 @@
+// Shared device helpers of the TRWP / ISGMR kernels for gfx950 (CDNA4, wave64).
+//
+// Mapping used by every scan kernel: one 64-lane wavefront walks one chain (a row, column or
+// diagonal segment) of one direction.  The L labels of a pixel are spread over the lanes in
+// blocks: lane i owns labels R*i .. R*i+R-1 with R = ceil(L/64).  A pixel's label vector is then
+// one R-dword buffer access per lane, a one-label shift is a single DPP wave shift plus register
+// renaming, and the min / sum over labels is a DPP reduction.
+//
+// Memory is accessed through buffer descriptors whose base is the first label vector of the batch
+// item.  The pixel is selected with the scalar offset `so`, the lane's labels with the vector
+// offset; gfx9 range-checks their sum against num_records, so every access passes
+// num_records = so + (size of one label vector): lanes whose labels do not exist fall outside the
+// descriptor, their loads return 0 and their stores are dropped by the hardware.  This keeps the
+// scan loop free of branches around memory instructions, which is what lets the loads of the next
+// pixels stay in flight (the hardware counter the compiler waits on counts memory operations in
+// order, so a branch that may skip one forces a conservative wait).  Offsets are 32-bit: one image
+// (H*W*L floats) must stay below 4 GiB; batch items are reached through the base.
+#ifndef MPLAYERS_AMD_MP_COMMON_H_
+#define MPLAYERS_AMD_MP_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+
+#include "../../include/mplayers_amd.h"
+
+namespace mpl {
+
+constexpr int kWave = 64;
+constexpr int kMaxL = MPL_MAX_LABELS;
+constexpr int kMaxDirs = MPL_MAX_DIRS;
+constexpr int kMaxCtx2dL = 64;  // (L,L) context table kept in LDS
+constexpr int kMaxBandK = 32;   // widest band handled by the O(L*K) path
+
+#ifndef MPL_PREFETCH
+#define MPL_PREFETCH 6
+#endif
+constexpr int kPrefetch = MPL_PREFETCH;  // pixels in flight per wave
+
+// ------------------------------------------------------------------------------------------------
+// wavefront primitives
+// ------------------------------------------------------------------------------------------------
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf>
+__device__ __forceinline__ float dpp_f(float old, float src) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, src),
+                                         CTRL, ROW_MASK, BANK_MASK, false));
+}
+// lane i <- lane i+1 (lane 63 <- fill)
+__device__ __forceinline__ float wave_shl1(float x, float fill) { return dpp_f<0x130>(fill, x); }
+// lane i <- lane i-1 (lane 0 <- fill)
+__device__ __forceinline__ float wave_shr1(float x, float fill) { return dpp_f<0x138>(fill, x); }
+
+__device__ __forceinline__ float readlane_f(float x, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));
+}
+// tells the compiler that x is wave-uniform (keeps addressing in scalar registers)
+__device__ __forceinline__ int uniform_i(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ float uniform_f(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+}
+
+// min over the 64 lanes, returned wave-uniform
+__device__ __forceinline__ float wave_min(float x) {
+  const float inf = INFINITY;
+  x = fminf(x, dpp_f<0x111>(inf, x));       // row_shr:1
+  x = fminf(x, dpp_f<0x112>(inf, x));       // row_shr:2
+  x = fminf(x, dpp_f<0x114>(inf, x));       // row_shr:4
+  x = fminf(x, dpp_f<0x118>(inf, x));       // row_shr:8: lane 15 of each row holds the row min
+  x = fminf(x, dpp_f<0x142, 0xa>(inf, x));  // row_bcast:15 into rows 1 and 3
+  x = fminf(x, dpp_f<0x143, 0xc>(inf, x));  // row_bcast:31 into rows 2 and 3
+  return readlane_f(x, 63);
+}
+
+// sum over the 64 lanes, returned wave-uniform
+__device__ __forceinline__ float wave_sum(float x) {
+  x += dpp_f<0x111>(0.f, x);
+  x += dpp_f<0x112>(0.f, x);
+  x += dpp_f<0x114>(0.f, x);
+  x += dpp_f<0x118>(0.f, x);
+  x += dpp_f<0x142, 0xa>(0.f, x);
+  x += dpp_f<0x143, 0xc>(0.f, x);
+  return readlane_f(x, 63);
+}
+
+__device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
+
+// largest label (R*lane + j) whose predicate is set; `dflt` when none is
+template <int R>
+__device__ __forceinline__ int last_label(const bool (&pred)[R], int dflt) {
+  uint64_t m[R];
+  uint64_t any = 0;
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    m[j] = ballot(pred[j]);
+    any |= m[j];
+  }
+  if (any == 0) return dflt;
+  int lane = 63 - __builtin_clzll(any);
+  int jj = 0;
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+    if ((m[j] >> lane) & 1) jj = j;
+  return R * lane + jj;
+}
+
+// ------------------------------------------------------------------------------------------------
+// buffer access.  A descriptor covers `bytes` bytes at p; accesses beyond it read 0 / are dropped.
+// ------------------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x3 __attribute__((ext_vector_type(3)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x3 __attribute__((ext_vector_type(3)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+constexpr int kDeadOffset = 0x7ffffff0;  // a vector offset no descriptor covers: access suppressed
+
+// R consecutive floats at vector byte offset `off` (range-checked) + scalar byte offset `so`.
+// VEC: one R-dword access (used when every lane's block lies entirely inside or entirely outside
+// the pixel vector, i.e. L % R == 0); otherwise R single-dword accesses, each checked on its own.
+template <int R, bool VEC>
+__device__ __forceinline__ void buf_load(rsrc_t r, int off, unsigned so, float (&x)[R]) {
+  if (VEC && R == 2) {
+    f32x2 t = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, off, so, 0));
+    x[0] = t[0];
+    x[1] = t[1];
+  } else if (VEC && R == 3) {
+    f32x3 t = __builtin_bit_cast(f32x3, __builtin_amdgcn_raw_buffer_load_b96(r, off, so, 0));
+    x[0] = t[0];
+    x[1] = t[1];
+    x[2] = t[2];
+  } else if (VEC && R == 4) {
+    f32x4 t = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, so, 0));
+    x[0] = t[0];
+    x[1] = t[1];
+    x[2] = t[2];
+    x[3] = t[3];
+  } else {
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+      x[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off + 4 * j, so, 0));
+  }
+}
+
+template <int R, bool VEC>
+__device__ __forceinline__ void buf_store(rsrc_t r, int off, unsigned so, const float (&x)[R]) {
+  if (VEC && R == 2) {
+    f32x2 t = {x[0], x[1]};
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, t), r, off, so, 0);
+  } else if (VEC && R == 3) {
+    f32x3 t = {x[0], x[1], x[2]};
+    __builtin_amdgcn_raw_buffer_store_b96(__builtin_bit_cast(u32x3, t), r, off, so, 0);
+  } else if (VEC && R == 4) {
+    f32x4 t = {x[0], x[1], x[2], x[3]};
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, t), r, off, so, 0);
+  } else {
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[j]), r, off + 4 * j, so, 0);
+  }
+}
+
+// R consecutive uint8 at byte offset `off`
+template <int R, bool VEC>
+__device__ __forceinline__ void buf_load_u8(rsrc_t r, int off, unsigned so, int (&x)[R]) {
+  if (VEC && R == 4) {
+    unsigned t = __builtin_amdgcn_raw_buffer_load_b32(r, off, so, 0);
+    x[0] = t & 0xff;
+    x[1] = (t >> 8) & 0xff;
+    x[2] = (t >> 16) & 0xff;
+    x[3] = t >> 24;
+  } else if (VEC && R == 2) {
+    unsigned t = __builtin_amdgcn_raw_buffer_load_b16(r, off, so, 0);
+    x[0] = t & 0xff;
+    x[1] = (t >> 8) & 0xff;
+  } else {
+#pragma unroll
+    for (int j = 0; j < R; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b8(r, off + j, so, 0);
+  }
+}
+
+template <int R, bool VEC>
+__device__ __forceinline__ void buf_store_u8(rsrc_t r, int off, unsigned so, const int (&x)[R]) {
+  if (VEC && R == 4) {
+    unsigned t = (unsigned)x[0] | ((unsigned)x[1] << 8) | ((unsigned)x[2] << 16) | ((unsigned)x[3] << 24);
+    __builtin_amdgcn_raw_buffer_store_b32(t, r, off, so, 0);
+  } else if (VEC && R == 2) {
+    unsigned short t = (unsigned short)((unsigned)x[0] | ((unsigned)x[1] << 8));
+    __builtin_amdgcn_raw_buffer_store_b16(t, r, off, so, 0);
+  } else {
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+      __builtin_amdgcn_raw_buffer_store_b8((unsigned char)x[j], r, off + j, so, 0);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// chain geometry.  Direction table: MPLayers/common.cpp:28-76.  A chain starts at every pixel whose
+// front neighbour (pixel - step) lies outside the image; that reproduces the reference's trees
+// (common.cpp:78-87 and the start formulas of the scan kernels) without empty chains.
+// ------------------------------------------------------------------------------------------------
+struct DirGeom {
+  int hs, ws;   // step of the forward scan
+  int ha, wa;   // |hs|, |ws| clipped to the image
+  int count_a;  // chains starting in the first ha rows the scan enters
+  int n_chains;
+};
+
+__host__ __device__ inline void dir_step(int dir, int* hs, int* ws) {
+  const int tab[16][2] = {{0, 1},  {0, -1}, {1, 0},  {-1, 0},  {1, 1},  {-1, -1}, {1, -1}, {-1, 1},
+                          {1, 2},  {-1, -2}, {2, 1}, {-2, -1}, {2, -1}, {-2, 1},  {1, -2}, {-1, 2}};
+  *hs = tab[dir][0];
+  *ws = tab[dir][1];
+}
+
+__host__ __device__ inline DirGeom make_dir(int dir, int H, int W) {
+  DirGeom g;
+  dir_step(dir, &g.hs, &g.ws);
+  int ha = g.hs < 0 ? -g.hs : g.hs, wa = g.ws < 0 ? -g.ws : g.ws;
+  g.ha = ha < H ? ha : H;
+  g.wa = wa < W ? wa : W;
+  g.count_a = g.ha * W;
+  g.n_chains = g.count_a + (H - g.ha) * g.wa;
+  return g;
+}
+
+// start pixel (h, w) and number of pixels n (>= 1) of chain c
+__device__ __forceinline__ void chain_start(const DirGeom& g, int H, int W, int c, int* h, int* w,
+                                            int* n) {
+  int hh, ww;
+  if (c < g.count_a) {
+    int r = c / W;
+    ww = c - r * W;
+    hh = g.hs > 0 ? r : H - 1 - r;
+  } else {
+    int cc = c - g.count_a;
+    int r = cc / g.wa;
+    int k = cc - r * g.wa;
+    hh = g.hs > 0 ? g.ha + r : (g.hs < 0 ? H - 1 - g.ha - r : r);
+    ww = g.ws > 0 ? k : W - 1 - k;
+  }
+  int nh = 0x7fffffff, nw = 0x7fffffff;
+  if (g.hs > 0) nh = (H - 1 - hh) / g.hs;
+  if (g.hs < 0) nh = hh / (-g.hs);
+  if (g.ws > 0) nw = (W - 1 - ww) / g.ws;
+  if (g.ws < 0) nw = ww / (-g.ws);
+  *h = hh;
+  *w = ww;
+  *n = 1 + (nh < nw ? nh : nw);
+}
+
+struct ChainCtx {
+  int bv;     // batch item
+  int pix0;   // pixel index of the chain start inside its image
+  int pstep;  // pixel stride along the chain
+  int n;      // pixels in the chain
+  int dir;
+};
+
+// which (direction, batch item, chain) a workgroup owns
+template <typename Params>
+__device__ __forceinline__ ChainCtx locate_chain(const Params& p) {
+  int di = 0;
+  while (di + 1 < p.n_dirs && (int)blockIdx.x >= p.block_prefix[di + 1]) ++di;
+  const int dir = p.dirs[di];
+  const int local = (int)blockIdx.x - p.block_prefix[di];
+  const DirGeom g = make_dir(dir, p.H, p.W);
+  const int bv = local / g.n_chains;
+  const int c = local - bv * g.n_chains;
+  int h0, w0, n;
+  chain_start(g, p.H, p.W, c, &h0, &w0, &n);
+  ChainCtx ch;
+  ch.bv = bv;
+  ch.pix0 = h0 * p.W + w0;
+  ch.pstep = g.hs * p.W + g.ws;
+  ch.n = n;
+  ch.dir = dir;
+  return ch;
+}
+
+// ------------------------------------------------------------------------------------------------
+// context descriptor, computed on the device so that no host round trip is needed
+// ------------------------------------------------------------------------------------------------
+struct CtxDesc {
+  int band_k;     // > 0: c[k] == cmax for all k >= band_k and c[k] <= cmax below; 0: dense path
+  int c0_is_min;  // c[0] <= c[k] for all k
+  float cmax;
+  int pad;
+};
+
+// ------------------------------------------------------------------------------------------------
+// kernel parameter blocks
+// ------------------------------------------------------------------------------------------------
+struct SweepParams {
+  int B, H, W, L;
+  int ctx2d;
+  int n_dirs;                      // directions in this launch
+  int dirs[kMaxDirs];              // their ids
+  int block_prefix[kMaxDirs + 1];  // prefix sums of B * n_chains
+  float rho;
+  const float* belief;             // S plane (N)
+  float* belief_out;               // TRWP: == belief; Jacobi: unused
+  const float* msg_in;             // (n_dir_total, N) planes read
+  float* msg_out;                  // (n_dir_total, N) planes written
+  const float* edge;               // (n_dir_total, P)
+  const float* ctx;
+  const CtxDesc* desc;             // may be null: dense path
+  uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
+  uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
+};
+
+struct BackParams {
+  int B, H, W, L;
+  int ctx2d;
+  int n_dirs;
+  int dirs[kMaxDirs];
+  int block_prefix[kMaxDirs + 1];
+  float rho;
+  // TRWP: g_k = A + h_k.  a_in: plane read as A (dcost_final on the first sweep), a_out: dunary.
+  const float* a_in;
+  float* a_out;
+  float* h;                 // (n_dir_total, N) planes h_k
+  int first_touch;          // h_dir and h_inv have not been written yet: read as zero
+  // ISGMR: gu_in planes (plane stride gu_stride; 0 on the first iteration where gu_k = dcost_final),
+  // du_out (n_dir_total, N) receives dU_d in place of gu_d
+  const float* gu_in;
+  int64_t gu_stride;
+  float* du_out;
+  const float* edge;        // (n_dir_total, P)
+  const float* ctx;
+  const uint8_t* idx_min;   // (n_dir_total, N) of this iteration
+  const uint8_t* idx_norm;  // (n_dir_total, P)
+  float* dedge;             // (n_dir_total, P) accumulates
+  float* dctx;              // accumulates
+};
+
+// launchers, one translation unit per R so that the instantiations compile in parallel
+template <int R>
+void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st);
+template <int R>
+void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
+
+inline size_t fwd_lds_bytes(int L, int ctx2d) {
+  return sizeof(float) * (kMaxL + (ctx2d ? L * L : L));
+}
+
+}  // namespace mpl
+
+#endif  // MPLAYERS_AMD_MP_COMMON_H_

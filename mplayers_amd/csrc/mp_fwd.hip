@@ -1,0 +1,369 @@
+// Forward scan of TRWP / ISGMR for gfx950: one wavefront per chain, see mp_common.h.
+//
+// Per pixel p of a chain (front pixel q = p - step), following HorizontalKernel /
+// DiagonalKernelWide / DiagonalKernelNarrow of the reference (TRWP_forward.cu:82-376,
+// ISGMR_forward.cu:123-431):
+//     a[fd]  = U[q, fd] + rho * m[q, fd]                  (m[q] = message just computed, 0 at the start)
+//     v[cd]  = min_fd a[fd] + w[p] * ctx(cd, fd)          (largest fd on ties)
+//     m[p,:] = v - min_cd v                               (largest cd on ties)
+// with U = rho * (S - m_dir_old) - m_inv_old taken from the belief plane S = unary + sum_k m_k
+// instead of re-summing all messages (UpdateUnaryKernel, TRWP_forward.cu:60-80).
+//
+// Compiled once per R (labels per lane) with -DMPL_INST_R=<R>.
+
+#include "mp_common.h"
+
+namespace mpl {
+namespace {
+
+template <int R>
+struct PixF {
+  float s[R], md[R], mi[R];
+  float w;
+};
+
+// Dense O(L^2) step: v[cd] = min_fd( a[fd] + w * ctx(cd, fd) ), largest fd on ties.
+// HorizontalKernel inner loop, TRWP_forward.cu:127-153.  a_s / ctx_s live in LDS.
+template <int R, bool TRAIN>
+__device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&valid)[R], float w,
+                                           int L, int ctx2d, int lab0, float* a_s,
+                                           const float* ctx_s, float (&v)[R], int (&fd_idx)[R]) {
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+    if (valid[j]) a_s[lab0 + j] = a[j];
+  __syncthreads();
+  int labc[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    int l = lab0 + j;
+    labc[j] = l < L ? l : L - 1;
+    v[j] = INFINITY;
+    fd_idx[j] = L - 1;
+  }
+  for (int fd = L - 1; fd >= 0; --fd) {
+    float af = a_s[fd];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      int cd = labc[j];
+      int ci = ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : (cd > fd ? cd - fd : fd - cd);
+      float val = fmaf(w, ctx_s[ci], af);
+      bool take = (fd == L - 1) || (val < v[j]);
+      v[j] = take ? val : v[j];
+      if (TRAIN) fd_idx[j] = take ? fd : fd_idx[j];
+    }
+  }
+  __syncthreads();
+}
+
+// Band O(L*K) step for 1-D contexts with a constant tail (c[k] == cmax for k >= K, c[k] <= cmax
+// below), exact for w >= 0:
+//   v[cd] = min( min_{|k|<K} a[cd+k] + w*c[|k|],  min_fd a[fd] + w*cmax )
+// The second term is an upper bound for every label and is attained by all labels farther than the
+// band from argmin(a); fp32 addition is monotone, so the values are bit-identical to the dense scan.
+// KT > 0: K known at compile time, taps c[] in registers.  KT == 0: K at run time, taps in LDS.
+template <int R, bool TRAIN, int KT>
+__device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, const float* c_reg,
+                                          const float* ctx_s, float cmax, float amin, int fstar,
+                                          int lab0, float (&v)[R], int (&fd_idx)[R]) {
+  const float inf = INFINITY;
+  float up[R], dn[R];
+  int off[R];
+  const float c0 = KT > 0 ? c_reg[0] : ctx_s[0];
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    up[j] = a[j];
+    dn[j] = a[j];
+    v[j] = fmaf(w, c0, a[j]);
+    off[j] = 0;
+  }
+  auto tap = [&](int k, float ck) {
+    // one-label shifts: up[j] <- a[label + k], dn[j] <- a[label - k]
+    float tu = wave_shl1(up[0], inf);
+    float td = wave_shr1(dn[R - 1], inf);
+#pragma unroll
+    for (int j = 0; j < R - 1; ++j) up[j] = up[j + 1];
+    up[R - 1] = tu;
+#pragma unroll
+    for (int j = R - 1; j > 0; --j) dn[j] = dn[j - 1];
+    dn[0] = td;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      float cu = fmaf(w, ck, up[j]);
+      float cd = fmaf(w, ck, dn[j]);
+      if (TRAIN) {
+        bool tk = cu <= v[j];  // larger front label wins ties
+        v[j] = tk ? cu : v[j];
+        off[j] = tk ? k : off[j];
+        bool tk2 = cd < v[j];  // smaller front label loses ties
+        v[j] = tk2 ? cd : v[j];
+        off[j] = tk2 ? -k : off[j];
+      } else {
+        v[j] = fminf(v[j], fminf(cu, cd));
+      }
+    }
+  };
+  if (KT > 0) {
+#pragma unroll
+    for (int k = 1; k < KT; ++k) tap(k, c_reg[k]);
+  } else {
+    for (int k = 1; k < K; ++k) tap(k, ctx_s[k]);
+  }
+  const float far = fmaf(w, cmax, amin);
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    if (TRAIN) {
+      int fb = lab0 + j + off[j];
+      bool lt = far < v[j];
+      bool eq = far == v[j];
+      int fe = fb > fstar ? fb : fstar;
+      fd_idx[j] = lt ? fstar : (eq ? fe : fb);
+      v[j] = lt ? far : v[j];
+    } else {
+      v[j] = fminf(v[j], far);
+    }
+  }
+}
+
+// One chain.  KT: > 0 band with compile-time K, 0 band with run-time K, -1 dense.
+// VEC: L % R == 0 (vector accesses).  MASK: some lanes own labels >= L.
+template <int R, bool VEC, bool MASK, bool TRAIN, bool JACOBI, int KT>
+__device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
+                                              const ChainCtx& ch, float* a_s, const float* ctx_s) {
+  const int L = p.L;
+  const int64_t HW = (int64_t)p.H * p.W;
+  const int64_t P = (int64_t)p.B * HW;
+  const int64_t N = P * L;
+  const int dir = ch.dir;
+  const int64_t img_p = (int64_t)ch.bv * HW;  // first pixel of this batch item
+  const int64_t img_e = img_p * L;
+  const int vbytes = L * 4;
+  // plane bases of this batch item and direction; descriptors are formed per access
+  const float* __restrict__ bS = p.belief + img_e;
+  const float* __restrict__ bMd = p.msg_in + (int64_t)dir * N + img_e;
+  const float* __restrict__ bMi = p.msg_in + (int64_t)(dir ^ 1) * N + img_e;
+  float* __restrict__ bMo = p.msg_out + (int64_t)dir * N + img_e;
+  float* __restrict__ bSo = (JACOBI ? nullptr : p.belief_out + img_e);
+  uint8_t* __restrict__ bImin = TRAIN ? p.idx_min + (int64_t)dir * N + img_e : nullptr;
+  const int img_bytes_p = (int)(HW * 4 > 0x7fffffff ? 0x7fffffff : HW * 4);
+  const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P + img_p, img_bytes_p);
+  const rsrc_t dInorm = make_rsrc(TRAIN ? p.idx_norm + (int64_t)dir * P + img_p : nullptr,
+                                  TRAIN ? (int)HW : 0);
+  const float rho = p.rho;
+  const float inf = INFINITY;
+  const int lane = threadIdx.x;
+  const int lab0 = R * lane;
+  const int foff = lab0 * 4;  // byte offset of this lane's block inside a pixel's float vector
+  const int n = ch.n;
+
+  bool valid[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) valid[j] = MASK ? (lab0 + j < L) : true;
+
+  float c_reg[KT > 0 ? KT : 1];
+  if (KT > 0) {
+#pragma unroll
+    for (int k = 0; k < KT; ++k) c_reg[k] = p.ctx[k];
+  }
+  const int K = desc.band_k;
+  const float cmax = desc.cmax;
+  const bool c0min = desc.c0_is_min != 0;
+
+  // loads of the next pixel; past the end of the chain the last pixel is fetched again
+  const int last_p = ch.pix0 + (n - 1) * ch.pstep;
+  int ld_p = ch.pix0;
+  int ld_t = 0;
+  auto load_next = [&]() {
+    PixF<R> r;
+    const unsigned pp = (unsigned)uniform_i(ld_t < n ? ld_p : last_p);
+    const unsigned so = pp * (unsigned)vbytes;
+    const int nrec = (int)(so + (unsigned)vbytes);
+    buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
+    buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
+    buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, 0, pp * 4u, 0));
+    ld_p += ch.pstep;
+    ld_t += 1;
+    return r;
+  };
+
+  // chain start: its front lies outside the image and the reference never writes it.  The Jacobi
+  // buffers alternate, so there the start pixel is written with the zeros it keeps in the reference.
+  float prev[R], uf[R];
+  {
+    const PixF<R> p0 = load_next();
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      prev[j] = 0.f;
+      float tt = p0.s[j] - p0.md[j];
+      float un = fmaf(tt, rho, -p0.mi[j]);
+      uf[j] = valid[j] ? un : inf;
+    }
+    if (JACOBI) {
+      float z[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) z[j] = 0.f;
+      const unsigned so = (unsigned)ch.pix0 * (unsigned)vbytes;
+      buf_store<R, VEC>(make_rsrc(bMo, (int)(so + (unsigned)vbytes)), foff, so, z);
+    }
+  }
+
+  PixF<R> ring[kPrefetch];
+#pragma unroll
+  for (int u = 0; u < kPrefetch; ++u) ring[u] = load_next();
+
+  int st_p = ch.pix0 + ch.pstep;
+  for (int t0 = 1; t0 < n; t0 += kPrefetch) {
+#pragma unroll
+    for (int u = 0; u < kPrefetch; ++u) {
+      const int t = t0 + u;
+      const bool live = t < n;  // steps past the end compute on stale data and store nothing
+      const PixF<R> px = ring[u];
+      ring[u] = load_next();
+      float tt[R], un[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        tt[j] = px.s[j] - px.md[j];             // unary + the other directions' messages
+        float x = fmaf(tt[j], rho, -px.mi[j]);  // UpdateUnaryKernel, TRWP_forward.cu:70-78
+        un[j] = valid[j] ? x : inf;
+      }
+      const float w = uniform_f(px.w);
+      float a[R], v[R];
+      int fd_idx[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) a[j] = fmaf(rho, prev[j], uf[j]);
+      float nmin;
+      bool need_nmin = true;
+      if (KT >= 0 && w >= 0.f) {
+        float am = a[0];
+#pragma unroll
+        for (int j = 1; j < R; ++j) am = fminf(am, a[j]);
+        const float amin = wave_min(am);
+        int fstar = L - 1;
+        if (TRAIN) {
+          bool pr[R];
+#pragma unroll
+          for (int j = 0; j < R; ++j) pr[j] = (a[j] == amin);
+          fstar = last_label<R>(pr, L - 1);
+        }
+        band_step<R, TRAIN, (KT > 0 ? KT : 0)>(a, w, K, c_reg, ctx_s, cmax, amin, fstar, lab0, v,
+                                               fd_idx);
+        if (c0min) {
+          // every candidate is >= amin + w*c[0], which the centre tap of label argmin(a) attains
+          nmin = fmaf(w, KT > 0 ? c_reg[0] : ctx_s[0], amin);
+          need_nmin = false;
+        }
+      } else if (live) {
+        dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
+      } else {
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          v[j] = 0.f;
+          fd_idx[j] = 0;
+        }
+      }
+      if (need_nmin) {
+        float vm = inf;
+#pragma unroll
+        for (int j = 0; j < R; ++j) vm = fminf(vm, valid[j] ? v[j] : inf);
+        nmin = wave_min(vm);
+      }
+      float m[R], sn[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        m[j] = v[j] - nmin;  // MsgNormNaive, commonCUDA.cuh:126-128
+        sn[j] = tt[j] + m[j];
+        prev[j] = valid[j] ? m[j] : 0.f;
+        uf[j] = un[j];
+      }
+      const unsigned sp = (unsigned)uniform_i(st_p);
+      const unsigned so = sp * (unsigned)vbytes;
+      const int nrec = live ? (int)(so + (unsigned)vbytes) : 0;  // nothing is stored past the end
+      buf_store<R, VEC>(make_rsrc(bMo, nrec), foff, so, m);
+      if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, nrec), foff, so, sn);
+      if (TRAIN) {
+        const unsigned sob = sp * (unsigned)L;
+        buf_store_u8<R, VEC>(make_rsrc(bImin, live ? (int)(sob + (unsigned)L) : 0), lab0, sob, fd_idx);
+        bool pr[R];
+#pragma unroll
+        for (int j = 0; j < R; ++j) pr[j] = valid[j] && (v[j] == nmin);
+        const int nidx = last_label<R>(pr, L - 1);
+        // every lane stores the same byte to the same address
+        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm, live ? 0 : kDeadOffset, sp, 0);
+      }
+      st_p += ch.pstep;
+    }
+  }
+}
+
+template <int R, bool VEC, bool MASK, bool TRAIN, bool JACOBI>
+__global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
+  extern __shared__ float smem[];
+  float* a_s = smem;            // kMaxL floats
+  float* ctx_s = smem + kMaxL;  // L or L*L floats
+  const int lane = threadIdx.x;
+  const int L = p.L;
+  const ChainCtx ch = locate_chain(p);
+  if (!JACOBI && ch.n < 2) return;  // nothing to write
+
+  CtxDesc desc;
+  if (p.desc != nullptr) {
+    desc = *p.desc;
+  } else {
+    desc.band_k = 0;
+    desc.c0_is_min = 0;
+    desc.cmax = 0.f;
+    desc.pad = 0;
+  }
+  // context table into LDS (dense path, run-time band taps, negative-weight fallback)
+  const int n_ctx = p.ctx2d ? L * L : L;
+  for (int i = lane; i < n_ctx; i += kWave) ctx_s[i] = p.ctx[i];
+  __syncthreads();
+
+  switch (desc.band_k) {
+    case 0: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -1>(p, desc, ch, a_s, ctx_s); break;
+    case 2: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 2>(p, desc, ch, a_s, ctx_s); break;
+    case 3: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 3>(p, desc, ch, a_s, ctx_s); break;
+    case 4: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 4>(p, desc, ch, a_s, ctx_s); break;
+    default: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0>(p, desc, ch, a_s, ctx_s); break;
+  }
+}
+
+template <int R, bool VEC, bool MASK>
+void launch_vm(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+  const int blocks = p.block_prefix[p.n_dirs];
+  const size_t lds = fwd_lds_bytes(p.L, p.ctx2d);
+  if (train) {
+    if (jacobi)
+      sweep_fwd_kernel<R, VEC, MASK, true, true><<<blocks, kWave, lds, st>>>(p);
+    else
+      sweep_fwd_kernel<R, VEC, MASK, true, false><<<blocks, kWave, lds, st>>>(p);
+  } else {
+    if (jacobi)
+      sweep_fwd_kernel<R, VEC, MASK, false, true><<<blocks, kWave, lds, st>>>(p);
+    else
+      sweep_fwd_kernel<R, VEC, MASK, false, false><<<blocks, kWave, lds, st>>>(p);
+  }
+}
+
+}  // namespace
+
+template <int R>
+void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+  if (p.block_prefix[p.n_dirs] <= 0) return;
+  const bool vec = (p.L % R) == 0;
+  const bool mask = p.L != R * kWave;
+  if constexpr (R > 1) {
+    if (!vec) {
+      launch_vm<R, false, true>(p, train, jacobi, st);
+      return;
+    }
+  }
+  if (mask)
+    launch_vm<R, true, true>(p, train, jacobi, st);
+  else
+    launch_vm<R, true, false>(p, train, jacobi, st);
+}
+
+template void launch_sweep_fwd<MPL_INST_R>(const SweepParams&, bool, bool, hipStream_t);
+
+}  // namespace mpl
