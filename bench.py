@@ -36,22 +36,17 @@ def parse():
   return ap.parse_args()
 
 
-def cpu_baseline(cfg, budget_s=20.0):
+def cpu_baseline(cfg, budget_s=15.0):
   """Times the reference's CPU forward path (built from the reference sources into oracle/_ref)
   or, where that build is absent, the oracle's restatement of the same loop nest, on a crop of
-  the workload: one iteration, unit edge weights (that path ignores them), forward only (the
-  reference has no CPU backward)."""
+  the workload: full-width rows, one iteration, unit edge weights (that path ignores them),
+  forward only (the reference has no CPU backward).  A short calibration run sizes the crop so
+  that the timed run takes about budget_s seconds."""
   import numpy as np
   from oracle import mp_oracle, ref_cpu
-  L, n_dir = cfg["L"], cfg["n_dir"]
+  L, n_dir, W = cfg["L"], cfg["n_dir"], cfg["W"]
   mode = "TRWP" if cfg["mode"] == "TRWP" else "ISGMR"
-  # cost model of that loop nest: L^2 * n_dir inner steps per pixel and sweep, ~1e9 steps/s/thread
-  threads = 16
-  per_pixel = float(L) * L * n_dir * n_dir
-  pixels = max(64, int(budget_s * 1.0e9 * threads / per_pixel / 4))
-  h = max(2, min(cfg["H"], 32))
-  w = max(2, min(cfg["W"], pixels // h))
-  unary = cfg["unary"][:1, :, :h, :w, :].contiguous().numpy()
+  threads = 16  # NUM_THREADS of the reference (tools/cpp/utils.h:17)
   ctx = cfg["context"].numpy()
   if ctx.ndim == 1:
     ii = np.abs(np.arange(L)[:, None] - np.arange(L)[None, :])
@@ -59,21 +54,27 @@ def cpu_baseline(cfg, budget_s=20.0):
   else:
     table = ctx + ctx.T
   table = np.ascontiguousarray(np.broadcast_to(table, (n_dir, L, L)), dtype=np.float32)
-  if ref_cpu.available():
-    kind = "reference"
-    run = lambda: ref_cpu.forward(mode, unary, table, n_dir, 1, cfg["rho"])
-  else:
-    kind = "port"
-    run = lambda: mp_oracle.refcpu_forward(mode, unary, table, n_dir, 1, cfg["rho"],
-                                           n_threads=threads, context_per_dir=True, ctx2d=(L == 21))
-  t0 = time.perf_counter()
-  run()
-  dt = time.perf_counter() - t0
-  units = h * w * L * 1
+  kind = "reference" if ref_cpu.available() else "port"
+
+  def run(rows):
+    unary = cfg["unary"][:1, :, :rows, :, :].contiguous().numpy()
+    t0 = time.perf_counter()
+    if kind == "reference":
+      ref_cpu.forward(mode, unary, table, n_dir, 1, cfg["rho"])
+    else:
+      mp_oracle.refcpu_forward(mode, unary, table, n_dir, 1, cfg["rho"], n_threads=threads,
+                               context_per_dir=True, ctx2d=(L == 21))
+    return time.perf_counter() - t0
+
+  rows0 = min(cfg["H"], 4)
+  dt0 = run(rows0)
+  rows = int(max(rows0, min(cfg["H"], rows0 * budget_s / max(dt0, 1e-3))))
+  dt = run(rows) if rows > rows0 else dt0
+  units = rows * W * L * 1
   return {"value": units / dt, "unit": "pixel*label*iter/s", "cores": threads, "kind": kind,
-          "sample": "%s forward only (no CPU backward exists), crop %dx%d px of %s, %d labels, "
-                    "%d dirs, 1 iteration, unit edge weights, %.1f s" % (mode, h, w, cfg["name"], L,
-                                                                        n_dir, dt)}
+          "sample": "%s forward only (the reference has no CPU backward), first %d rows x %d "
+                    "columns of %s, %d labels, %d directions, 1 iteration, unit edge weights, "
+                    "%.1f s" % (mode, rows, W, cfg["name"], L, n_dir, dt)}
 
 
 def main():

@@ -106,7 +106,9 @@ int mpl_profile_begin(void);
 int mpl_profile_end(mpl_kernel_stat* stats, int n_stats);
 
 /* Number of chains of direction `dir` (0..15) on an H x W grid: the reference's n_trees
- * (common.cpp:78-87).  Host-only helper. */
+ * (common.cpp:78-87) for images of at least 2 x 2 pixels (on thinner images the reference also
+ * counts trees of the two-pixel steps that never enter the image).  Host-only helper; -1 for a
+ * direction outside the table. */
 int mpl_n_chains(int dir, int height, int width);
 
 /* Message of the last failed call on this thread ("" if none). */

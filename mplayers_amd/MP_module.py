@@ -180,7 +180,8 @@ class MPModule(torch.nn.Module):
       norm = nn.Softmax(dim=0)(valid)
       label_context[self.label_context_loc] = norm * valid.max() / norm.max()
     if mode in {'sigmoid', 'softmax'}:
-      label_context[self.label_context_diag_loc] = self.args.mpnet_diag_value
+      diag = self.label_context_diag_loc
+      label_context[tuple(diag) if isinstance(diag, list) else diag] = self.args.mpnet_diag_value
     return label_context
 
   def forward(self, unary, edge_weights=None):

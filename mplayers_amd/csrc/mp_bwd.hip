@@ -103,17 +103,22 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     }
     buf_load_u8<R, VEC>(make_rsrc(bImin, (int)(pp * (unsigned)L + (unsigned)L)), lab0,
                         pp * (unsigned)L, r.fd);
-    r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, 0, pp, 0);
-    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, 0, pp * 4u, 0));
-    r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dDe, 0, pp * 4u, 0));
+    r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, (int)pp, 0, 0);
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
+    r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dDe, (int)(pp * 4u), 0, 0));
     ld_t -= 1;
     ld_p -= ch.pstep;
     return r;
   };
 
-  PixB<R> ring[kPrefetch];
+  // memory instructions per step: label vectors, indices, norm index, weight, dedge in;
+  // label vectors and dedge out
+  constexpr int kOps = (JACOBI ? 1 : 3) * vec_ops(R, VEC) + byte_ops(R, VEC) + 3 +
+                       (JACOBI ? 1 : 3) * vec_ops(R, VEC) + 1;
+  constexpr int D = ring_depth(kOps);
+  PixB<R> ring[D];
 #pragma unroll
-  for (int u = 0; u < kPrefetch; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) ring[u] = load_next();
 
   float sc[R];  // dU of the current pixel: what the previous step scattered into it
   float hist_reg[R];        // dcontext[label] partial sums of this lane's own labels (1-D context)
@@ -125,10 +130,12 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const int last_lane = (L - 1) / R, last_reg = (L - 1) % R;
 
   int st_p = ch.pix0 + (n - 1) * ch.pstep;
-  for (int s0 = 0; s0 < n; s0 += kPrefetch) {
+  for (int s0 = 0; s0 < n; s0 += D) {
 #pragma unroll
-    for (int u = 0; u < kPrefetch; ++u) {
+    for (int u = 0; u < D; ++u) {
       const int t = n - 1 - (s0 + u);
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
       const PixB<R> px = ring[u];
       ring[u] = load_next();
       float scn[R];
@@ -157,23 +164,24 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           int v = __builtin_amdgcn_readlane(px.fd[j], last_lane);
           f1 = (j == last_reg) ? v : f1;
         }
+        // off[j] = front label - own label; kPopular marks labels whose front label is one of the
+        // two popular targets (they are summed with wave reductions instead of being moved)
+        constexpr int kPopular = 0x4000;
         int off[R];
-        bool m0[R], m1[R], rem[R], left[R];
         float p0 = 0.f, p1 = 0.f, de = 0.f;
         bool any_left = false;
 #pragma unroll
         for (int j = 0; j < R; ++j) {
           const int cd = lab0 + j, fd = px.fd[j];
           if (cd == nidx) gv[j] -= tot;
-          off[j] = fd - cd;
-          m0[j] = fd == f0;
-          m1[j] = (fd == f1) && !m0[j];
-          rem[j] = !m0[j] && !m1[j];
-          const int ao = off[j] < 0 ? -off[j] : off[j];
-          left[j] = rem[j] && (ao > kNear) && valid[j];
-          any_left = any_left || left[j];
-          p0 += m0[j] ? gv[j] : 0.f;
-          p1 += m1[j] ? gv[j] : 0.f;
+          const int d = fd - cd;
+          const int ao = d < 0 ? -d : d;
+          const bool c0 = fd == f0;
+          const bool c1 = (fd == f1) && !c0;
+          p0 += c0 ? gv[j] : 0.f;
+          p1 += c1 ? gv[j] : 0.f;
+          off[j] = (c0 || c1) ? kPopular : d;
+          any_left = any_left || (!(c0 || c1) && ao > kNear && valid[j]);
           // dedge_weights[cur] += ctx(cd, fd) * value
           const int ci = !valid[j] ? 0 : (p.ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
           de = fmaf(ctx_s[ci], gv[j], de);
@@ -186,15 +194,14 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
         for (int j = 0; j < R; ++j) tp[j] = tn[j] = 0.f;
 #pragma unroll
         for (int o = kNear; o >= 1; --o) {
-          float cp[R], cn[R];
           near_t[o] = 0.f;
 #pragma unroll
           for (int j = 0; j < R; ++j) {
-            cp[j] = (rem[j] && off[j] == o) ? gv[j] : 0.f;
-            cn[j] = (rem[j] && off[j] == -o) ? gv[j] : 0.f;
-            near_t[o] += cp[j] + cn[j];
-            tp[j] += cp[j];
-            tn[j] += cn[j];
+            const float cp = (off[j] == o) ? gv[j] : 0.f;
+            const float cn = (off[j] == -o) ? gv[j] : 0.f;
+            near_t[o] += cp + cn;
+            tp[j] += cp;
+            tn[j] += cn;
           }
           // move one label up (tp) / down (tn)
           const float up_in = wave_shr1(tp[R - 1], 0.f);
@@ -209,7 +216,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
         for (int j = 0; j < R; ++j) {
           const int cd = lab0 + j;
-          float own = (rem[j] && off[j] == 0) ? gv[j] : 0.f;
+          const float own = (off[j] == 0) ? gv[j] : 0.f;
           scn[j] = own + tp[j] + tn[j] + (cd == f0 ? s0sum : 0.f) + (cd == f1 ? s1sum : 0.f);
         }
         // dcontext += edge_weight * value where cd != fd (TRWP_backward.cu:111-112)
@@ -219,27 +226,27 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           // popular classes: bin |cd - f| is reached from labels f + k and f - k; gather through LDS
 #pragma unroll
           for (int j = 0; j < R; ++j)
-            if (valid[j]) g0_s[lab0 + j] = m0[j] ? w * gv[j] : 0.f;
+            if (valid[j]) g0_s[lab0 + j] = (px.fd[j] == f0) ? w * gv[j] : 0.f;
           __syncthreads();
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             const int k = lab0 + j;
             const int hi_l = f0 + k, lo_l = f0 - k;
-            float a = (k >= 1 && hi_l < L) ? g0_s[hi_l < L ? hi_l : 0] : 0.f;
-            float b = (k >= 1 && lo_l >= 0) ? g0_s[lo_l >= 0 ? lo_l : 0] : 0.f;
+            const float a = (k >= 1 && hi_l < L) ? g0_s[hi_l < L ? hi_l : 0] : 0.f;
+            const float b = (k >= 1 && lo_l >= 0) ? g0_s[lo_l >= 0 ? lo_l : 0] : 0.f;
             hist_reg[j] += a + b;
           }
           if (f1 != f0) {
 #pragma unroll
             for (int j = 0; j < R; ++j)
-              if (valid[j]) g1_s[lab0 + j] = m1[j] ? w * gv[j] : 0.f;
+              if (valid[j]) g1_s[lab0 + j] = (px.fd[j] == f1) ? w * gv[j] : 0.f;
             __syncthreads();
 #pragma unroll
             for (int j = 0; j < R; ++j) {
               const int k = lab0 + j;
               const int hi_l = f1 + k, lo_l = f1 - k;
-              float a = (k >= 1 && hi_l < L) ? g1_s[hi_l < L ? hi_l : 0] : 0.f;
-              float b = (k >= 1 && lo_l >= 0) ? g1_s[lo_l >= 0 ? lo_l : 0] : 0.f;
+              const float a = (k >= 1 && hi_l < L) ? g1_s[hi_l < L ? hi_l : 0] : 0.f;
+              const float b = (k >= 1 && lo_l >= 0) ? g1_s[lo_l >= 0 ? lo_l : 0] : 0.f;
               hist_reg[j] += a + b;
             }
           }
@@ -255,9 +262,10 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
         if (ballot(any_left) != 0) {
 #pragma unroll
           for (int j = 0; j < R; ++j) {
-            if (left[j]) {
+            const int ao = off[j] < 0 ? -off[j] : off[j];
+            if (valid[j] && off[j] != kPopular && ao > kNear) {
               atomicAdd(&sc_s[px.fd[j]], gv[j]);
-              if (!p.ctx2d) atomicAdd(&hist_s[off[j] < 0 ? -off[j] : off[j]], w * gv[j]);
+              if (!p.ctx2d) atomicAdd(&hist_s[ao], w * gv[j]);
             }
           }
           __syncthreads();
@@ -287,7 +295,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
       }
       // each pixel receives over exactly one edge per direction: plain read-modify-write
       __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
-                                            t >= 1 ? 0 : kDeadOffset, sp * 4u, 0);
+                                            t >= 1 ? (int)(sp * 4u) : kDeadOffset, 0, 0);
 #pragma unroll
       for (int j = 0; j < R; ++j) sc[j] = scn[j];
       st_p -= ch.pstep;

@@ -7,10 +7,12 @@
 // renaming, and the min / sum over labels is a DPP reduction.
 //
 // Memory is accessed through buffer descriptors whose base is the first label vector of the batch
-// item.  The pixel is selected with the scalar offset `so`, the lane's labels with the vector
-// offset; gfx9 range-checks their sum against num_records, so every access passes
-// num_records = so + (size of one label vector): lanes whose labels do not exist fall outside the
-// descriptor, their loads return 0 and their stores are dropped by the hardware.  This keeps the
+// item.  The offset of an access is (pixel offset `so`) + (offset of the lane's labels); it is
+// range-checked against num_records, so every access passes num_records = so + (size of one label
+// vector): lanes whose labels do not exist fall outside the descriptor, their loads return 0 and
+// their stores are dropped by the hardware.  The whole offset travels in the vector-offset operand
+// (none in the scalar-offset register): multi-dword stores that used a scalar-offset register had
+// their data overwritten by the instructions that followed them on the MI355X.  This keeps the
 // scan loop free of branches around memory instructions, which is what lets the loads of the next
 // pixels stay in flight (the hardware counter the compiler waits on counts memory operations in
 // order, so a branch that may skip one forces a conservative wait).  Offsets are 32-bit: one image
@@ -33,9 +35,29 @@ constexpr int kMaxCtx2dL = 64;  // (L,L) context table kept in LDS
 constexpr int kMaxBandK = 32;   // widest band handled by the O(L*K) path
 
 #ifndef MPL_PREFETCH
-#define MPL_PREFETCH 6
+#define MPL_PREFETCH 8
 #endif
-constexpr int kPrefetch = MPL_PREFETCH;  // pixels in flight per wave
+constexpr int kPrefetch = MPL_PREFETCH;  // upper limit of pixels in flight per wave
+
+// The hardware counter of outstanding vector-memory operations of a wave has 6 bits; runs with more
+// than 63 loads and stores in flight per wave returned corrupted data.  The prefetch ring is
+// therefore sized from the number of memory instructions a step issues, to stay below kMaxInFlight.
+constexpr int kMaxInFlight = 52;
+constexpr int ring_depth(int ops_per_step) {
+  int d = kMaxInFlight / (ops_per_step > 0 ? ops_per_step : 1);
+  return d < 1 ? 1 : (d > kPrefetch ? kPrefetch : d);
+}
+// Explicit wait until at most N vector-memory operations of this wave are outstanding (gfx9
+// encoding of s_waitcnt: vmcnt in bits [3:0] and [15:14]; the other counters left at their maxima).
+template <int N>
+__device__ __forceinline__ void wait_vmem() {
+  constexpr int n = N > 62 ? 62 : (N < 0 ? 0 : N);
+  __builtin_amdgcn_s_waitcnt((n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8));
+}
+
+// number of instructions one R-label access of floats / of bytes takes
+constexpr int vec_ops(int R, bool vec) { return vec ? 1 : R; }
+constexpr int byte_ops(int R, bool vec) { return (vec && (R == 4 || R == 2)) ? 1 : R; }
 
 // ------------------------------------------------------------------------------------------------
 // wavefront primitives
@@ -126,17 +148,17 @@ constexpr int kDeadOffset = 0x7ffffff0;  // a vector offset no descriptor covers
 // the pixel vector, i.e. L % R == 0); otherwise R single-dword accesses, each checked on its own.
 template <int R, bool VEC>
 __device__ __forceinline__ void buf_load(rsrc_t r, int off, unsigned so, float (&x)[R]) {
-  if (VEC && R == 2) {
-    f32x2 t = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, off, so, 0));
+  if constexpr (VEC && R == 2) {
+    f32x2 t = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)((unsigned)off + so), 0, 0));
     x[0] = t[0];
     x[1] = t[1];
-  } else if (VEC && R == 3) {
-    f32x3 t = __builtin_bit_cast(f32x3, __builtin_amdgcn_raw_buffer_load_b96(r, off, so, 0));
+  } else if constexpr (VEC && R == 3) {
+    f32x3 t = __builtin_bit_cast(f32x3, __builtin_amdgcn_raw_buffer_load_b96(r, (int)((unsigned)off + so), 0, 0));
     x[0] = t[0];
     x[1] = t[1];
     x[2] = t[2];
-  } else if (VEC && R == 4) {
-    f32x4 t = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, so, 0));
+  } else if constexpr (VEC && R == 4) {
+    f32x4 t = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)((unsigned)off + so), 0, 0));
     x[0] = t[0];
     x[1] = t[1];
     x[2] = t[2];
@@ -144,59 +166,59 @@ __device__ __forceinline__ void buf_load(rsrc_t r, int off, unsigned so, float (
   } else {
 #pragma unroll
     for (int j = 0; j < R; ++j)
-      x[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off + 4 * j, so, 0));
+      x[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)((unsigned)(off + 4 * j) + so), 0, 0));
   }
 }
 
 template <int R, bool VEC>
 __device__ __forceinline__ void buf_store(rsrc_t r, int off, unsigned so, const float (&x)[R]) {
-  if (VEC && R == 2) {
+  if constexpr (VEC && R == 2) {
     f32x2 t = {x[0], x[1]};
-    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, t), r, off, so, 0);
-  } else if (VEC && R == 3) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, t), r, (int)((unsigned)off + so), 0, 0);
+  } else if constexpr (VEC && R == 3) {
     f32x3 t = {x[0], x[1], x[2]};
-    __builtin_amdgcn_raw_buffer_store_b96(__builtin_bit_cast(u32x3, t), r, off, so, 0);
-  } else if (VEC && R == 4) {
+    __builtin_amdgcn_raw_buffer_store_b96(__builtin_bit_cast(u32x3, t), r, (int)((unsigned)off + so), 0, 0);
+  } else if constexpr (VEC && R == 4) {
     f32x4 t = {x[0], x[1], x[2], x[3]};
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, t), r, off, so, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, t), r, (int)((unsigned)off + so), 0, 0);
   } else {
 #pragma unroll
     for (int j = 0; j < R; ++j)
-      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[j]), r, off + 4 * j, so, 0);
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[j]), r, (int)((unsigned)(off + 4 * j) + so), 0, 0);
   }
 }
 
 // R consecutive uint8 at byte offset `off`
 template <int R, bool VEC>
 __device__ __forceinline__ void buf_load_u8(rsrc_t r, int off, unsigned so, int (&x)[R]) {
-  if (VEC && R == 4) {
-    unsigned t = __builtin_amdgcn_raw_buffer_load_b32(r, off, so, 0);
+  if constexpr (VEC && R == 4) {
+    unsigned t = __builtin_amdgcn_raw_buffer_load_b32(r, (int)((unsigned)off + so), 0, 0);
     x[0] = t & 0xff;
     x[1] = (t >> 8) & 0xff;
     x[2] = (t >> 16) & 0xff;
     x[3] = t >> 24;
-  } else if (VEC && R == 2) {
-    unsigned t = __builtin_amdgcn_raw_buffer_load_b16(r, off, so, 0);
+  } else if constexpr (VEC && R == 2) {
+    unsigned t = __builtin_amdgcn_raw_buffer_load_b16(r, (int)((unsigned)off + so), 0, 0);
     x[0] = t & 0xff;
     x[1] = (t >> 8) & 0xff;
   } else {
 #pragma unroll
-    for (int j = 0; j < R; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b8(r, off + j, so, 0);
+    for (int j = 0; j < R; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b8(r, (int)((unsigned)(off + j) + so), 0, 0);
   }
 }
 
 template <int R, bool VEC>
 __device__ __forceinline__ void buf_store_u8(rsrc_t r, int off, unsigned so, const int (&x)[R]) {
-  if (VEC && R == 4) {
+  if constexpr (VEC && R == 4) {
     unsigned t = (unsigned)x[0] | ((unsigned)x[1] << 8) | ((unsigned)x[2] << 16) | ((unsigned)x[3] << 24);
-    __builtin_amdgcn_raw_buffer_store_b32(t, r, off, so, 0);
-  } else if (VEC && R == 2) {
+    __builtin_amdgcn_raw_buffer_store_b32(t, r, (int)((unsigned)off + so), 0, 0);
+  } else if constexpr (VEC && R == 2) {
     unsigned short t = (unsigned short)((unsigned)x[0] | ((unsigned)x[1] << 8));
-    __builtin_amdgcn_raw_buffer_store_b16(t, r, off, so, 0);
+    __builtin_amdgcn_raw_buffer_store_b16(t, r, (int)((unsigned)off + so), 0, 0);
   } else {
 #pragma unroll
     for (int j = 0; j < R; ++j)
-      __builtin_amdgcn_raw_buffer_store_b8((unsigned char)x[j], r, off + j, so, 0);
+      __builtin_amdgcn_raw_buffer_store_b8((unsigned char)x[j], r, (int)((unsigned)(off + j) + so), 0, 0);
   }
 }
 

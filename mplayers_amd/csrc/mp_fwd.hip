@@ -180,7 +180,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
     buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
     buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
-    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, 0, pp * 4u, 0));
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
     ld_p += ch.pstep;
     ld_t += 1;
     return r;
@@ -207,16 +207,22 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     }
   }
 
-  PixF<R> ring[kPrefetch];
+  // memory instructions per step: 3 label vectors + the weight in, 1-2 label vectors (+ indices) out
+  constexpr int kOps = 3 * vec_ops(R, VEC) + 1 + (JACOBI ? 1 : 2) * vec_ops(R, VEC) +
+                       (TRAIN ? byte_ops(R, VEC) + 1 : 0);
+  constexpr int D = ring_depth(kOps);
+  PixF<R> ring[D];
 #pragma unroll
-  for (int u = 0; u < kPrefetch; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) ring[u] = load_next();
 
   int st_p = ch.pix0 + ch.pstep;
-  for (int t0 = 1; t0 < n; t0 += kPrefetch) {
+  for (int t0 = 1; t0 < n; t0 += D) {
 #pragma unroll
-    for (int u = 0; u < kPrefetch; ++u) {
+    for (int u = 0; u < D; ++u) {
       const int t = t0 + u;
       const bool live = t < n;  // steps past the end compute on stale data and store nothing
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
       const PixF<R> px = ring[u];
       ring[u] = load_next();
       float tt[R], un[R];
@@ -288,7 +294,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         for (int j = 0; j < R; ++j) pr[j] = valid[j] && (v[j] == nmin);
         const int nidx = last_label<R>(pr, L - 1);
         // every lane stores the same byte to the same address
-        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm, live ? 0 : kDeadOffset, sp, 0);
+        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm, live ? (int)sp : kDeadOffset, 0, 0);
       }
       st_p += ch.pstep;
     }

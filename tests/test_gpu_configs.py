@@ -1,0 +1,265 @@
+"""GPU parity on the benchmark configurations (scaled to sizes the CPU oracle finishes in seconds),
+on the reference-built fixtures, through the nn.Module surface, and -- at the full size of the large
+configuration -- through size-independent properties."""
+import argparse
+import glob
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module")
+def gpu():
+  import torch
+  assert torch.cuda.is_available(), "these tests need the MI355X"
+  from mplayers_amd import _lib
+  _lib.load()
+  from tests import _gpu_util
+  return _gpu_util
+
+
+CONFIG_CASES = [
+    # config, mode, scale, n_iter override
+    ("C1", "ISGMR", 1.0, None),
+    ("C2", "TRWP", 0.1, None),
+    ("C3", "ISGMR", 0.12, 5),
+    ("C4", "TRWP", 1.0, None),
+    ("C4", "ISGMR", 1.0, None),
+    ("C5", "TRWP", 0.02, None),
+    ("C5", "ISGMR", 0.02, None),
+]
+
+
+@pytest.mark.parametrize("name,mode,scale,n_iter", CONFIG_CASES)
+def test_config_matches_oracle(gpu, oracle, name, mode, scale, n_iter):
+  from mplayers_amd import synthetic
+  cfg = synthetic.make_config(name, seed=0, scale=scale, mode=mode)
+  n_iter = n_iter or cfg["n_iter"]
+  unary, ctx, ew = cfg["unary"].numpy(), cfg["context"].numpy(), cfg["edge_weights"].numpy()
+  train = cfg["training"]
+  print("config", name, mode, unary.shape, "n_iter", n_iter, flush=True)
+  ref = oracle.forward(mode, unary, ctx, ew, cfg["n_dir"], n_iter, cfg["rho"], training=train,
+                       want_gaps=train, saving_label=True)
+  got = gpu.gpu_forward(mode, unary, ctx, ew, cfg["n_dir"], n_iter, cfg["rho"], training=train,
+                        saving_label=True)
+  gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=ref["cost_final"])
+  gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
+  assert (got["label_all"][-1] != ref["label_all"][-1]).mean() < 0.01
+  if not train:
+    return
+  tol = 2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max()))
+  n_bad = gpu.assert_indices_match_off_ties(got["msg_min_index"], ref["msg_min_index"],
+                                            ref["gap_min"], tol, "msg_min_index")
+  assert n_bad <= 1e-3 * ref["msg_min_index"].size
+  gpu.assert_indices_match_off_ties(got["msg_norm_index"], ref["msg_norm_index"], ref["gap_norm"],
+                                    tol, "msg_norm_index")
+  # backward on the oracle's indices, against the fp64 oracle
+  dcost = synthetic.upstream_grad(cfg).numpy()
+  r = oracle.backward(mode, ctx.astype(np.float64), ew.astype(np.float64), dcost.astype(np.float64),
+                      ref["msg_min_index"], ref["msg_norm_index"], cfg["rho"])
+  g = gpu.gpu_backward(mode, ctx, ew, dcost, ref["msg_min_index"], ref["msg_norm_index"],
+                       cfg["rho"])
+  for a, b, what in zip(g, r, ("dunary", "dcontext", "dedge_weights")):
+    scale_ = max(1.0, float(np.abs(b).max()))
+    assert np.abs(a - b).max() <= 1e-4 * scale_, (what, float(np.abs(a - b).max()), scale_)
+  assert abs(g[0].astype(np.float64).sum() - dcost.astype(np.float64).sum()) <= 1e-3 * np.abs(dcost).sum() ** 0.5 + 1e-2
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "refcpu_*.npz"))),
+                         ids=lambda p: os.path.basename(p)[7:-4])
+def test_reference_cpu_fixtures(gpu, path):
+  """Outputs of the reference's own compiled CPU forward (tests/golden/make_refcpu_golden.py).
+  The GPU operator reads one context for all directions, so only the fixtures whose per-direction
+  tables are one shared symmetric Toeplitz table apply; unit edge weights as on that CPU path."""
+  z = np.load(path)
+  ctx = z["context"]
+  n_dir, L, _ = ctx.shape
+  ii = np.abs(np.arange(L)[:, None] - np.arange(L)[None, :])
+  shared = all(np.array_equal(ctx[0], ctx[d]) for d in range(n_dir)) and \
+      np.array_equal(ctx[0], ctx[0][0][ii])
+  if not shared:
+    pytest.skip("per-direction context tables exist only on the reference's CPU path")
+  mode, rho, n_iter = str(z["mode"]), float(z["rho"]), int(z["n_iter"])
+  c = ctx[0] if L == 21 else ctx[0, 0]
+  got = gpu.gpu_forward(mode, z["unary"], c, None, n_dir, n_iter, rho, saving_label=True)
+  gpu.assert_values_close(got["msg"], z["msg"], what="msg", belief=z["cost_final"])
+  gpu.assert_values_close(got["cost_final"], z["cost_final"], what="cost_final")
+  if "int" in path and mode == "ISGMR":
+    assert np.array_equal(got["msg"], z["msg"]) and np.array_equal(got["label_all"], z["label_all"])
+
+
+@pytest.mark.parametrize("mode,L,train_mode", [("TRWP", 21, "sigmoid"), ("ISGMR", 21, ""),
+                                               ("ISGMR", 12, "softmax"), ("TRWP", 40, "")])
+def test_module_forward_backward(gpu, oracle, mode, L, train_mode):
+  """The drop-in surface: MPModule -> autograd Function -> operators -> C ABI."""
+  import torch
+  from mplayers_amd import MPModule
+  rng = np.random.default_rng(L)
+  B, H, W, n_dir, n_iter = 2, 7, 9, 4 if mode == "TRWP" else 8, 2
+  args = argparse.Namespace(mpnet_mrf_mode=mode, mpnet_max_iter=n_iter, mpnet_n_dirs=n_dir,
+                            n_classes=L, mpnet_term_weight=1.5, mpnet_smoothness_train=train_mode,
+                            mpnet_smoothness_mode="TL", mpnet_smoothness_trunct_value=3,
+                            mpnet_smoothness_trunct_loc=-1, mpnet_diag_value=0.0,
+                            enable_symmetric=True, enable_cuda=True)
+  mod = MPModule(args, enable_create_label_context=True, enable_saving_label=True).cuda().train()
+  unary = rng.standard_normal((B, 1, L, H, W)).astype(np.float32)
+  ew = (0.1 + 0.9 * rng.random((B, n_dir, H, W))).astype(np.float32)
+  dcost = rng.standard_normal((B, 1, L, H, W)).astype(np.float32)
+  u = torch.from_numpy(unary).cuda().requires_grad_(True)
+  e = torch.from_numpy(ew).cuda().requires_grad_(True)
+  cost, lc_out, labels, _, _ = mod(u, e)
+  assert cost.shape == (B, 1, L, H, W) and labels.shape == (n_iter, B, 1, H, W)
+  assert lc_out.shape[0] == 1
+  cost.backward(torch.from_numpy(dcost).cuda())
+  torch.cuda.synchronize()
+  ctx = lc_out[0].detach().cpu().numpy()
+  un = np.ascontiguousarray(unary.transpose(0, 1, 3, 4, 2))
+  en = np.ascontiguousarray(ew[:, None].transpose(2, 0, 1, 3, 4))
+  dn = np.ascontiguousarray(dcost.transpose(0, 1, 3, 4, 2))
+  rho = 0.5 if mode == "TRWP" else 1.0
+  ref = oracle.forward(mode, un, ctx, en, n_dir, n_iter, rho, saving_label=True)
+  gpu.assert_values_close(cost.detach().cpu().numpy().transpose(0, 1, 3, 4, 2), ref["cost_final"],
+                          what="module cost")
+  assert (labels.cpu().numpy() != ref["label_all"]).mean() < 0.01
+  du, dc, de = oracle.backward(mode, ctx.astype(np.float64), en.astype(np.float64),
+                               dn.astype(np.float64), ref["msg_min_index"], ref["msg_norm_index"], rho)
+  assert np.abs(u.grad.cpu().numpy().transpose(0, 1, 3, 4, 2) - du).max() <= 1e-4 * max(1, np.abs(du).max())
+  assert np.abs(e.grad.cpu().numpy()[:, None].transpose(2, 0, 1, 3, 4) - de).max() <= 1e-4 * max(1, np.abs(de).max())
+  if train_mode:  # the context parameter is learnable: its gradient flows through the re-parameterisation
+    lc = torch.from_numpy(mod.label_context.detach().cpu().numpy().astype(np.float64)).requires_grad_(True)
+    loc, diag = mod.label_context_loc, mod.label_context_diag_loc
+    eff = lc * 1
+    if train_mode == "sigmoid":
+      eff[loc] = 2 * args.mpnet_term_weight * torch.sigmoid(eff[loc].flatten())
+    else:
+      v = eff[loc].flatten()
+      sm = torch.softmax(v, 0)
+      eff[loc] = sm * v.max() / sm.max()
+    eff[tuple(diag) if isinstance(diag, list) else diag] = args.mpnet_diag_value
+    eff.backward(torch.from_numpy(dc))
+    got = mod.label_context.grad.cpu().numpy()
+    assert np.abs(got - lc.grad.numpy()).max() <= 1e-4 * max(1, np.abs(lc.grad.numpy()).max())
+  # evaluation mode: no indices are kept, same values
+  mod.eval()
+  with torch.no_grad():
+    cost2, _, _, _, _ = mod(torch.from_numpy(unary).cuda(), torch.from_numpy(ew).cuda())
+  assert torch.equal(cost2, cost.detach())
+  # without edge weights the third gradient is None (MP_module.py:80-81)
+  mod.train()
+  u2 = torch.from_numpy(unary).cuda().requires_grad_(True)
+  cost3, _, _, _, _ = mod(u2)
+  cost3.sum().backward()
+  assert u2.grad is not None
+
+
+def test_operator_error_behaviour(gpu):
+  import torch
+  from mplayers_amd import lib_stereo
+  dev = "cuda:0"
+  e = torch.empty(0, dtype=torch.uint8)
+
+  def call(L=5, contiguous=True):
+    u = torch.zeros(1, 1, 3, 4, L, device=dev)
+    if not contiguous:
+      u = torch.zeros(1, 1, 3, L, 4, device=dev).transpose(3, 4)
+    msg = torch.zeros(4, 1, 1, 3, 4, L, device=dev)
+    lib_stereo.TRWP.forward(0.5, 1, 0, u, torch.zeros(L, device=dev),
+                            torch.ones(4, 1, 1, 3, 4, device=dev), msg, torch.zeros(1, 1, 3, 4, L, device=dev),
+                            e, e, torch.zeros(1, 1, 3, 4, L, device=dev), e)
+
+  call()
+  with pytest.raises(RuntimeError, match="contiguous"):
+    call(contiguous=False)
+  # the reference prints and returns zero-filled outputs above MAX_DISPARITY (TRWP.cpp:269-273)
+  with pytest.raises(RuntimeError, match="n_disp"):
+    call(L=300)
+
+
+def test_runs_are_deterministic_and_batch_items_independent(gpu):
+  from mplayers_amd import synthetic
+  cfg = synthetic.make_config("C4", seed=3, scale=0.25, mode="TRWP")
+  unary, ctx, ew = cfg["unary"].numpy(), cfg["context"].numpy(), cfg["edge_weights"].numpy()
+  a = gpu.gpu_forward("TRWP", unary, ctx, ew, 4, 3, 0.5)
+  b = gpu.gpu_forward("TRWP", unary, ctx, ew, 4, 3, 0.5)
+  for k in ("msg", "cost_final", "msg_min_index", "msg_norm_index"):
+    assert np.array_equal(a[k], b[k]), k
+  one = gpu.gpu_forward("TRWP", unary[2:3], ctx, ew[:, 2:3], 4, 3, 0.5)
+  assert np.array_equal(a["cost_final"][2:3], one["cost_final"])
+  assert np.array_equal(a["msg_min_index"][:, :, 2:3], one["msg_min_index"])
+  # twelve identical samples give identical per-sample results (pytorch/test_multi_batch.py:61-63)
+  rep = np.repeat(unary[:1], 12, axis=0)
+  rew = np.repeat(ew[:, :1], 12, axis=1)
+  r = gpu.gpu_forward("ISGMR", rep, ctx, rew, 4, 2, 1.0)
+  assert all(np.array_equal(r["cost_final"][0], r["cost_final"][i]) for i in range(12))
+
+
+@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
+def test_large_config_properties_at_full_size(gpu, mode):
+  """1500 x 2000, 192 labels, 8 directions, training mode: too large for the CPU oracle, so the
+  full-size run is checked through what must hold at any size."""
+  import torch
+  from mplayers_amd import lib_stereo, synthetic
+  cfg = synthetic.make_config("C5", seed=0, mode=mode)
+  B, H, W, L, n_dir = cfg["B"], cfg["H"], cfg["W"], cfg["L"], cfg["n_dir"]
+  n_iter, rho = 2, cfg["rho"]
+  dev = "cuda:0"
+  unary = cfg["unary"].to(dev)
+  ctx = cfg["context"].to(dev)
+  ew = cfg["edge_weights"].to(dev)
+  msg = torch.zeros(n_dir, B, 1, H, W, L, device=dev)
+  cost = torch.zeros(B, 1, H, W, L, device=dev)
+  scratch = torch.zeros(B, 1, H, W, L, device=dev)
+  imin = torch.zeros(n_iter, n_dir, B, 1, H, W, L, dtype=torch.uint8, device=dev)
+  inorm = torch.zeros(n_iter, n_dir, B, 1, H, W, dtype=torch.uint8, device=dev)
+  labels = torch.zeros(n_iter, B, 1, H, W, dtype=torch.uint8, device=dev)
+  print("full size", mode, flush=True)
+  if mode == "TRWP":
+    lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch, labels)
+  else:
+    msg_tmp = torch.zeros_like(msg)
+    lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch,
+                             msg_tmp, labels)
+    del msg_tmp
+  torch.cuda.synchronize()
+  # every message vector is normalised: min exactly 0 (all-zero where the chain starts)
+  assert float(msg.min()) == 0.0
+  mins = msg.amin(dim=-1)
+  assert float(mins.abs().max()) == 0.0
+  assert float(msg[0, 0, 0, :, 0].abs().max()) == 0.0   # direction 0 starts at the left column
+  assert float(msg[3, 0, 0, -1].abs().max()) == 0.0     # direction 3 starts at the bottom row
+  assert float(msg[4, 0, 0, 0].abs().max()) == 0.0      # direction 4 (down-right) at the top row
+  assert float(msg[0, 0, 0, :, 1:].amax(dim=-1).min()) > 0.0
+  # cost_final = unary + sum_k msg_k, summed in direction order (bitwise)
+  acc = unary.clone()
+  for k in range(n_dir):
+    acc += msg[k]
+  assert torch.equal(acc, cost)
+  del acc
+  # labels = argmin of the cost (smallest label on ties); indices are valid labels
+  assert torch.equal(cost.argmin(dim=-1).to(torch.uint8), labels[-1])
+  assert int(imin.max()) < L and int(inorm.max()) < L
+  # the argmin of a message's own argmin index row is where it is zero
+  sel = msg[1, 0, 0].gather(-1, inorm[-1, 1, 0, 0].long().unsqueeze(-1)).squeeze(-1)
+  assert float(sel[:, :-1].abs().max()) == 0.0
+  # backward: gradient mass is conserved (every normalised message has zero net gradient)
+  dcost = torch.randn(B, 1, H, W, L, device=dev, generator=torch.Generator(dev).manual_seed(1))
+  dunary = torch.zeros_like(dcost)
+  dmsg = msg  # reuse as scratch
+  dedge = torch.zeros(n_dir, B, 1, H, W, device=dev)
+  dctx = torch.zeros(L, device=dev)
+  if mode == "TRWP":
+    lib_stereo.TRWP.backward(rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, dmsg, scratch)
+  else:
+    lib_stereo.ISGMR.backward(0, rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, scratch,
+                              scratch, dmsg)
+  torch.cuda.synchronize()
+  total = float(dcost.double().sum())
+  assert abs(float(dunary.double().sum()) - total) <= 1e-6 * float(dcost.double().abs().sum())
+  assert float(dctx[0]) == 0.0 and bool(torch.isfinite(dctx).all()) and bool(torch.isfinite(dedge).all())
+  # edge-weight gradients exist only where a pixel has a front neighbour
+  assert float(dedge[0, 0, 0, :, 0].abs().max()) == 0.0
+  assert float(dedge[0, 0, 0, :, 1:].abs().max()) > 0.0

@@ -100,7 +100,7 @@ def test_forward_matches_oracle(gpu, oracle, mode, n_dir, B, H, W, L, kind, n_it
                        saving_label=True, want_gaps=training)
   got = gpu.gpu_forward(mode, unary, ctx, ew, n_dir, n_iter, rho, training=training,
                         saving_label=True)
-  gpu.assert_values_close(got["msg"], ref["msg"], what="msg")
+  gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=ref["cost_final"])
   gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
   if training:
     tol = 2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max()))
@@ -210,4 +210,4 @@ def test_min_a_dir_and_initial_messages(gpu, oracle):
   first = oracle.forward("TRWP", unary, ctx, None, n_dir, 1, 0.5)
   ref = oracle.forward("TRWP", unary, ctx, None, n_dir, 2, 0.5)
   got = gpu.gpu_forward("TRWP", unary, ctx, None, n_dir, 1, 0.5, msg_init=first["msg"])
-  gpu.assert_values_close(got["msg"], ref["msg"], what="continued msg")
+  gpu.assert_values_close(got["msg"], ref["msg"], what="continued msg", belief=ref["cost_final"])
