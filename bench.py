@@ -22,6 +22,15 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch of the scan kernels at the full-size large configuration, measured with
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (one counter per run) and scaled by what the
+# same counters read for a plain device copy of one plane (FETCH_SIZE x2.0, WRITE_SIZE x1.0); the
+# summary of those runs is kept under profiles/.  Counters cannot be read from inside this script.
+MEASURED_TRAFFIC_BYTES = {
+    ("C5", 1.0, True): {"fwd_sweep": 12.35e9, "bwd_sweep": 14.75e9,
+                        "fwd_sweep_all": 81.29e9, "bwd_sweep_all": 48.25e9},
+}
+
 
 def parse():
   ap = argparse.ArgumentParser()
@@ -33,6 +42,9 @@ def parse():
   ap.add_argument("--alg", default="both", choices=["both", "TRWP", "ISGMR"])
   ap.add_argument("--fwd-only", action="store_true", help="inference forward only (C2/C3 style)")
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--copy-probe", action="store_true",
+                  help="also run one plain device copy of one fp32 plane (reference point for "
+                       "hardware byte counters)")
   return ap.parse_args()
 
 
@@ -81,7 +93,7 @@ def main():
   a = parse()
   if a.gpus != 1:
     print("bench.py: this build drives one GPU only (the path shards by batch item or by "
-          "direction, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+          "direction without any exchange inside the operators); run with --gpus 1", file=sys.stderr)
     return 2
   import torch
   from mplayers_amd import _lib, lib_stereo, synthetic
@@ -136,6 +148,10 @@ def main():
           lib_stereo.ISGMR.backward(0, rho, context, edge, dcost, imin, inorm, dunary, dctx,
                                     dedge, dmsg, dscratch, dmsg_tmp)
 
+  if a.copy_probe:
+    probe = torch.empty_like(cost)
+    probe.copy_(unary)  # reads N*4 bytes, writes N*4 bytes
+    del probe
   for _ in range(a.warmup):
     step()
   torch.cuda.synchronize()
@@ -170,9 +186,11 @@ def main():
                      "achieved_GBs": per_launch / (ms / n * 1e-3) / 1e9,
                      "bytes_per_label_sweep": bpl}
   dominant = max(kernels, key=lambda k: kernels[k]["total_ms"])
+  traffic = MEASURED_TRAFFIC_BYTES.get((cfg["name"], a.scale, training), {}).get(dominant)
   roofline = {"bound": "hbm", "kernel": dominant, "achieved": kernels[dominant]["achieved_GBs"],
               "peak": HBM_PEAK_GBS, "unit": "GB/s",
-              "frac": kernels[dominant]["achieved_GBs"] / HBM_PEAK_GBS, "traffic": None,
+              "frac": kernels[dominant]["achieved_GBs"] / HBM_PEAK_GBS, "traffic": traffic,
+              "algorithmic_bytes_per_launch": kernels[dominant]["bytes_per_launch"],
               "avg_launch_ms": kernels[dominant]["avg_ms"]}
   # whole-step roofline fraction against the contract bytes per unit (n_dir * (fwd + bwd))
   contract = n_dir * (fwd_b + (bwd_b if training else 0.0))
