@@ -42,7 +42,10 @@ constexpr int kPrefetch = MPL_PREFETCH;  // upper limit of pixels in flight per 
 // The hardware counter of outstanding vector-memory operations of a wave has 6 bits; runs with more
 // than 63 loads and stores in flight per wave returned corrupted data.  The prefetch ring is
 // therefore sized from the number of memory instructions a step issues, to stay below kMaxInFlight.
-constexpr int kMaxInFlight = 52;
+#ifndef MPL_MAX_INFLIGHT
+#define MPL_MAX_INFLIGHT 52
+#endif
+constexpr int kMaxInFlight = MPL_MAX_INFLIGHT;
 constexpr int ring_depth(int ops_per_step) {
   int d = kMaxInFlight / (ops_per_step > 0 ? ops_per_step : 1);
   return d < 1 ? 1 : (d > kPrefetch ? kPrefetch : d);
