@@ -51,47 +51,111 @@ __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __r
 }
 
 // ------------------------------------------------------------------------------------------------
-// elementwise kernels
+// elementwise kernels.  V floats per lane and access (4 when every plane is 16-byte aligned and the
+// plane size is a multiple of 4, else 1); ND: number of directions when it is one of the usual ones
+// (loads of all planes are then issued back to back), 0: run-time loop.
 // ------------------------------------------------------------------------------------------------
+template <int V>
+struct Pack {
+  float v[V];
+};
+template <int V>
+__device__ __forceinline__ Pack<V> ld_pack(const float* p) {
+  Pack<V> r;
+  if constexpr (V == 4) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+    r.v[0] = t.x;
+    r.v[1] = t.y;
+    r.v[2] = t.z;
+    r.v[3] = t.w;
+  } else {
+    r.v[0] = *p;
+  }
+  return r;
+}
+template <int V>
+__device__ __forceinline__ void st_pack(float* p, const Pack<V>& r) {
+  if constexpr (V == 4) {
+    f32x4 t;
+    t.x = r.v[0];
+    t.y = r.v[1];
+    t.z = r.v[2];
+    t.w = r.v[3];
+    *reinterpret_cast<f32x4*>(p) = t;
+  } else {
+    *p = r.v[0];
+  }
+}
+
 // S = unary + sum_k m_k  (k ascending, as UpdateUnaryKernel sums, TRWP_forward.cu:70-73)
+template <int V, int ND>
 __global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ unary,
-                                                     const float* __restrict__ msg, int n_dir,
+                                                     const float* __restrict__ msg, int n_dir_rt,
                                                      int64_t N, float* __restrict__ S) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    float v = unary[i];
-    for (int k = 0; k < n_dir; ++k) v += msg[(int64_t)k * N + i];
-    S[i] = v;
+  const int n_dir = ND > 0 ? ND : n_dir_rt;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
+       i += (int64_t)gridDim.x * blockDim.x * V) {
+    Pack<V> v = ld_pack<V>(unary + i);
+    if constexpr (ND > 0) {
+      Pack<V> m[ND];
+#pragma unroll
+      for (int k = 0; k < ND; ++k) m[k] = ld_pack<V>(msg + (int64_t)k * N + i);
+#pragma unroll
+      for (int k = 0; k < ND; ++k)
+#pragma unroll
+        for (int j = 0; j < V; ++j) v.v[j] += m[k].v[j];
+    } else {
+      for (int k = 0; k < n_dir; ++k) {
+        const Pack<V> m = ld_pack<V>(msg + (int64_t)k * N + i);
+#pragma unroll
+        for (int j = 0; j < V; ++j) v.v[j] += m.v[j];
+      }
+    }
+    st_pack<V>(S + i, v);
   }
 }
 
 // cost = factor*unary + sum_k m_k  (or + min_k m_k): CostAggregateKernel, TRWP_forward.cu:31-58,
 // ISGMR_forward.cu:69-99.  copy_to != null: also mirror the message planes there.
+template <int V, int ND>
 __global__ void __launch_bounds__(256) aggregate_kernel(const float* __restrict__ unary,
-                                                        const float* __restrict__ msg, int n_dir,
+                                                        const float* __restrict__ msg, int n_dir_rt,
                                                         int64_t N, float factor, int min_a_dir,
                                                         float* __restrict__ cost,
                                                         float* __restrict__ copy_to) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    float v = unary[i] * factor;
-    if (min_a_dir) {
-      float mn = msg[i];
-      if (copy_to) copy_to[i] = mn;
-      for (int k = 1; k < n_dir; ++k) {
-        float m = msg[(int64_t)k * N + i];
-        if (copy_to) copy_to[(int64_t)k * N + i] = m;
-        if (m < mn) mn = m;
+  const int n_dir = ND > 0 ? ND : n_dir_rt;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
+       i += (int64_t)gridDim.x * blockDim.x * V) {
+    Pack<V> v = ld_pack<V>(unary + i);
+#pragma unroll
+    for (int j = 0; j < V; ++j) v.v[j] *= factor;
+    Pack<V> mn;  // min_a_dir only
+    auto fold = [&](int k, const Pack<V>& m) {
+      if (copy_to) st_pack<V>(copy_to + (int64_t)k * N + i, m);
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        if (!min_a_dir)
+          v.v[j] += m.v[j];  // ((unary + m_0) + m_1) + ... as the reference adds
+        else if (k == 0)
+          mn.v[j] = m.v[j];
+        else
+          mn.v[j] = (m.v[j] < mn.v[j]) ? m.v[j] : mn.v[j];
       }
-      v += mn;
+    };
+    if constexpr (ND > 0) {
+      Pack<V> m[ND];
+#pragma unroll
+      for (int k = 0; k < ND; ++k) m[k] = ld_pack<V>(msg + (int64_t)k * N + i);
+#pragma unroll
+      for (int k = 0; k < ND; ++k) fold(k, m[k]);
     } else {
-      for (int k = 0; k < n_dir; ++k) {
-        float m = msg[(int64_t)k * N + i];
-        if (copy_to) copy_to[(int64_t)k * N + i] = m;
-        v += m;
-      }
+      for (int k = 0; k < n_dir; ++k) fold(k, ld_pack<V>(msg + (int64_t)k * N + i));
     }
-    cost[i] = v;
+    if (min_a_dir) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) v.v[j] += mn.v[j];
+    }
+    st_pack<V>(cost + i, v);
   }
 }
 
@@ -137,27 +201,49 @@ __global__ void __launch_bounds__(256) label_kernel(const float* __restrict__ un
 // ISGMR: after all directions of an iteration have been scanned back (X_k = dU_k):
 //   dunary += rho * sum_k X_k ;  gu_k = rho * (sum - X_k) - X_{k^1}
 // (UpdateUnaryKernelBack summed over directions + SumMsgKernel, ISGMR_backward.cu:39-60, 482-483)
-__global__ void __launch_bounds__(256) isgmr_combine_kernel(float* __restrict__ X, int n_dir,
+template <int V, int ND>
+__global__ void __launch_bounds__(256) isgmr_combine_kernel(float* __restrict__ X, int n_dir_rt,
                                                             int64_t N, float rho,
                                                             const float* __restrict__ dcost,
                                                             float factor, int init_dunary,
                                                             int write_gu,
                                                             float* __restrict__ dunary) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < N;
-       i += (int64_t)gridDim.x * blockDim.x) {
-    float x[kMaxDirs];
-    float sum = 0.f;
+  constexpr int KD = ND > 0 ? ND : kMaxDirs;
+  const int n_dir = ND > 0 ? ND : n_dir_rt;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
+       i += (int64_t)gridDim.x * blockDim.x * V) {
+    Pack<V> x[KD];
 #pragma unroll
-    for (int k = 0; k < kMaxDirs; ++k) {
-      x[k] = (k < n_dir) ? X[(int64_t)k * N + i] : 0.f;
+    for (int k = 0; k < KD; ++k) {
+      if (k < n_dir) {
+        x[k] = ld_pack<V>(X + (int64_t)k * N + i);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) x[k].v[j] = 0.f;
+      }
     }
-    for (int k = n_dir - 1; k >= 0; --k) sum += x[k];
-    float du = init_dunary ? factor * dcost[i] : dunary[i];
-    dunary[i] = fmaf(rho, sum, du);
+    Pack<V> du = init_dunary ? ld_pack<V>(dcost + i) : ld_pack<V>(dunary + i);
+    Pack<V> sum;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      sum.v[j] = 0.f;
+#pragma unroll
+      for (int k = KD - 1; k >= 0; --k)
+        if (k < n_dir) sum.v[j] += x[k].v[j];
+      if (init_dunary) du.v[j] *= factor;
+      du.v[j] = fmaf(rho, sum.v[j], du.v[j]);
+    }
+    st_pack<V>(dunary + i, du);
     if (write_gu) {
 #pragma unroll
-      for (int k = 0; k < kMaxDirs; ++k)
-        if (k < n_dir) X[(int64_t)k * N + i] = fmaf(rho, sum - x[k], -x[k ^ 1]);
+      for (int k = 0; k < KD; ++k) {
+        if (k < n_dir) {
+          Pack<V> g;
+#pragma unroll
+          for (int j = 0; j < V; ++j) g.v[j] = fmaf(rho, sum.v[j] - x[k].v[j], -x[k ^ 1].v[j]);
+          st_pack<V>(X + (int64_t)k * N + i, g);
+        }
+      }
     }
   }
 }
@@ -288,6 +374,25 @@ int elementwise_blocks(int64_t n) {
   if (b > 256 * 32) b = 256 * 32;
   return (int)b;
 }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// Picks the instantiation of an element-wise kernel: 4 floats per access when the planes allow it,
+// the direction count as a compile-time constant when it is 4, 8 or 16.
+#define MPL_EW_LAUNCH(KERNEL, VEC4, NDIR, N, ST, ...)                                            \
+  do {                                                                                           \
+    const int blocks_ = elementwise_blocks((VEC4) ? (N) / 4 : (N));                              \
+    if (VEC4) {                                                                                  \
+      switch (NDIR) {                                                                            \
+        case 4: KERNEL<4, 4><<<blocks_, 256, 0, ST>>>(__VA_ARGS__); break;                       \
+        case 8: KERNEL<4, 8><<<blocks_, 256, 0, ST>>>(__VA_ARGS__); break;                       \
+        case 16: KERNEL<4, 16><<<blocks_, 256, 0, ST>>>(__VA_ARGS__); break;                     \
+        default: KERNEL<4, 0><<<blocks_, 256, 0, ST>>>(__VA_ARGS__); break;                      \
+      }                                                                                          \
+    } else {                                                                                     \
+      KERNEL<1, 0><<<blocks_, 256, 0, ST>>>(__VA_ARGS__);                                        \
+    }                                                                                            \
+  } while (0)
 
 void fill_dirs(const mpl_shape* s, int first, int count, int* dirs, int* prefix, int* n_dirs) {
   *n_dirs = count;
@@ -429,7 +534,8 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   const CtxDesc* desc = make_desc(s, context, cost_final, st);
   {
     Timed timed(MPL_KERNEL_BELIEF, st);
-    belief_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, msg, s->n_dir, N, unary_update);
+    const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
+    MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update);
   }
 
   SweepParams p = base_fwd_params(s, rho, edge_weights, context, desc);
@@ -455,8 +561,9 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   }
   {
     Timed timed(MPL_KERNEL_AGGREGATE, st);
-    aggregate_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, msg, s->n_dir, N, 1.f,
-                                                            enable_min_a_dir, cost_final, nullptr);
+    const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(cost_final);
+    MPL_EW_LAUNCH(aggregate_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, 1.f,
+                  enable_min_a_dir, cost_final, (float*)nullptr);
   }
   return launch_ok("trwp_forward");
 }
@@ -491,7 +598,8 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
     float* nxt = buf[(it + 1) & 1];
     {
       Timed timed(MPL_KERNEL_BELIEF, st);
-      belief_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, cur, s->n_dir, N, unary_update);
+      const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(cur) && aligned16(unary_update);
+      MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, cur, s->n_dir, N, unary_update);
     }
     p.msg_in = cur;
     p.msg_out = nxt;
@@ -511,9 +619,10 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   const float* fin = buf[n_iter & 1];
   {
     Timed timed(MPL_KERNEL_AGGREGATE, st);
-    aggregate_kernel<<<elementwise_blocks(N), 256, 0, st>>>(unary, fin, s->n_dir, N, factor,
-                                                            enable_min_a_dir, cost_final,
-                                                            (n_iter & 1) ? msg : nullptr);
+    const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update) &&
+                    aligned16(cost_final);
+    MPL_EW_LAUNCH(aggregate_kernel, v4, s->n_dir, N, st, unary, fin, s->n_dir, N, factor,
+                  enable_min_a_dir, cost_final, (n_iter & 1) ? msg : (float*)nullptr);
   }
   return launch_ok("isgmr_forward");
 }
@@ -601,8 +710,10 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
     p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
     launch_bwd(p, true, st);
     Timed timed(MPL_KERNEL_COMBINE, st);
-    isgmr_combine_kernel<<<elementwise_blocks(N), 256, 0, st>>>(
-        dmsg_update, s->n_dir, N, rho, dcost_final, factor, first ? 1 : 0, it > 0 ? 1 : 0, dunary);
+    const bool v4 = (N % 4 == 0) && aligned16(dmsg_update) && aligned16(dcost_final) &&
+                    aligned16(dunary);
+    MPL_EW_LAUNCH(isgmr_combine_kernel, v4, s->n_dir, N, st, dmsg_update, s->n_dir, N, rho,
+                  dcost_final, factor, first ? 1 : 0, it > 0 ? 1 : 0, dunary);
   }
   return launch_ok("isgmr_backward");
 }
