@@ -55,6 +55,9 @@ __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __r
 // plane size is a multiple of 4, else 1); ND: number of directions when it is one of the usual ones
 // (loads of all planes are then issued back to back), 0: run-time loop.
 // ------------------------------------------------------------------------------------------------
+#ifndef MPL_EW_NT
+#define MPL_EW_NT 1  // planes are streamed once: non-temporal loads and stores
+#endif
 template <int V>
 struct Pack {
   float v[V];
@@ -63,13 +66,14 @@ template <int V>
 __device__ __forceinline__ Pack<V> ld_pack(const float* p) {
   Pack<V> r;
   if constexpr (V == 4) {
-    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+    const f32x4 t = MPL_EW_NT ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p))
+                              : *reinterpret_cast<const f32x4*>(p);
     r.v[0] = t.x;
     r.v[1] = t.y;
     r.v[2] = t.z;
     r.v[3] = t.w;
   } else {
-    r.v[0] = *p;
+    r.v[0] = MPL_EW_NT ? __builtin_nontemporal_load(p) : *p;
   }
   return r;
 }
@@ -81,9 +85,15 @@ __device__ __forceinline__ void st_pack(float* p, const Pack<V>& r) {
     t.y = r.v[1];
     t.z = r.v[2];
     t.w = r.v[3];
-    *reinterpret_cast<f32x4*>(p) = t;
+    if (MPL_EW_NT)
+      __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
+    else
+      *reinterpret_cast<f32x4*>(p) = t;
   } else {
-    *p = r.v[0];
+    if (MPL_EW_NT)
+      __builtin_nontemporal_store(r.v[0], p);
+    else
+      *p = r.v[0];
   }
 }
 

@@ -144,6 +144,16 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, int bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
 }
 
+// Cache-policy bits of the label-vector accesses (gfx94x/95x: 1 = sc0, 2 = nt, 16 = sc1).  Every
+// plane is streamed once per sweep and is far larger than the caches, so loads and stores carry the
+// non-temporal hint; measured on the 1500x2000x192 forward sweep: 2.98 ms without, 2.54 ms with.
+#ifndef MPL_LD_AUX
+#define MPL_LD_AUX 2
+#endif
+#ifndef MPL_ST_AUX
+#define MPL_ST_AUX 2
+#endif
+
 constexpr int kDeadOffset = 0x7ffffff0;  // a vector offset no descriptor covers: access suppressed
 
 // R consecutive floats at vector byte offset `off` (range-checked) + scalar byte offset `so`.
@@ -152,16 +162,16 @@ constexpr int kDeadOffset = 0x7ffffff0;  // a vector offset no descriptor covers
 template <int R, bool VEC>
 __device__ __forceinline__ void buf_load(rsrc_t r, int off, unsigned so, float (&x)[R]) {
   if constexpr (VEC && R == 2) {
-    f32x2 t = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)((unsigned)off + so), 0, 0));
+    f32x2 t = __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)((unsigned)off + so), 0, MPL_LD_AUX));
     x[0] = t[0];
     x[1] = t[1];
   } else if constexpr (VEC && R == 3) {
-    f32x3 t = __builtin_bit_cast(f32x3, __builtin_amdgcn_raw_buffer_load_b96(r, (int)((unsigned)off + so), 0, 0));
+    f32x3 t = __builtin_bit_cast(f32x3, __builtin_amdgcn_raw_buffer_load_b96(r, (int)((unsigned)off + so), 0, MPL_LD_AUX));
     x[0] = t[0];
     x[1] = t[1];
     x[2] = t[2];
   } else if constexpr (VEC && R == 4) {
-    f32x4 t = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)((unsigned)off + so), 0, 0));
+    f32x4 t = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)((unsigned)off + so), 0, MPL_LD_AUX));
     x[0] = t[0];
     x[1] = t[1];
     x[2] = t[2];
@@ -169,7 +179,7 @@ __device__ __forceinline__ void buf_load(rsrc_t r, int off, unsigned so, float (
   } else {
 #pragma unroll
     for (int j = 0; j < R; ++j)
-      x[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)((unsigned)(off + 4 * j) + so), 0, 0));
+      x[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)((unsigned)(off + 4 * j) + so), 0, MPL_LD_AUX));
   }
 }
 
@@ -177,17 +187,17 @@ template <int R, bool VEC>
 __device__ __forceinline__ void buf_store(rsrc_t r, int off, unsigned so, const float (&x)[R]) {
   if constexpr (VEC && R == 2) {
     f32x2 t = {x[0], x[1]};
-    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, t), r, (int)((unsigned)off + so), 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, t), r, (int)((unsigned)off + so), 0, MPL_ST_AUX);
   } else if constexpr (VEC && R == 3) {
     f32x3 t = {x[0], x[1], x[2]};
-    __builtin_amdgcn_raw_buffer_store_b96(__builtin_bit_cast(u32x3, t), r, (int)((unsigned)off + so), 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b96(__builtin_bit_cast(u32x3, t), r, (int)((unsigned)off + so), 0, MPL_ST_AUX);
   } else if constexpr (VEC && R == 4) {
     f32x4 t = {x[0], x[1], x[2], x[3]};
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, t), r, (int)((unsigned)off + so), 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, t), r, (int)((unsigned)off + so), 0, MPL_ST_AUX);
   } else {
 #pragma unroll
     for (int j = 0; j < R; ++j)
-      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[j]), r, (int)((unsigned)(off + 4 * j) + so), 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[j]), r, (int)((unsigned)(off + 4 * j) + so), 0, MPL_ST_AUX);
   }
 }
 
@@ -195,18 +205,18 @@ __device__ __forceinline__ void buf_store(rsrc_t r, int off, unsigned so, const 
 template <int R, bool VEC>
 __device__ __forceinline__ void buf_load_u8(rsrc_t r, int off, unsigned so, int (&x)[R]) {
   if constexpr (VEC && R == 4) {
-    unsigned t = __builtin_amdgcn_raw_buffer_load_b32(r, (int)((unsigned)off + so), 0, 0);
+    unsigned t = __builtin_amdgcn_raw_buffer_load_b32(r, (int)((unsigned)off + so), 0, MPL_LD_AUX);
     x[0] = t & 0xff;
     x[1] = (t >> 8) & 0xff;
     x[2] = (t >> 16) & 0xff;
     x[3] = t >> 24;
   } else if constexpr (VEC && R == 2) {
-    unsigned t = __builtin_amdgcn_raw_buffer_load_b16(r, (int)((unsigned)off + so), 0, 0);
+    unsigned t = __builtin_amdgcn_raw_buffer_load_b16(r, (int)((unsigned)off + so), 0, MPL_LD_AUX);
     x[0] = t & 0xff;
     x[1] = (t >> 8) & 0xff;
   } else {
 #pragma unroll
-    for (int j = 0; j < R; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b8(r, (int)((unsigned)(off + j) + so), 0, 0);
+    for (int j = 0; j < R; ++j) x[j] = __builtin_amdgcn_raw_buffer_load_b8(r, (int)((unsigned)(off + j) + so), 0, MPL_LD_AUX);
   }
 }
 
@@ -214,14 +224,14 @@ template <int R, bool VEC>
 __device__ __forceinline__ void buf_store_u8(rsrc_t r, int off, unsigned so, const int (&x)[R]) {
   if constexpr (VEC && R == 4) {
     unsigned t = (unsigned)x[0] | ((unsigned)x[1] << 8) | ((unsigned)x[2] << 16) | ((unsigned)x[3] << 24);
-    __builtin_amdgcn_raw_buffer_store_b32(t, r, (int)((unsigned)off + so), 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b32(t, r, (int)((unsigned)off + so), 0, MPL_ST_AUX);
   } else if constexpr (VEC && R == 2) {
     unsigned short t = (unsigned short)((unsigned)x[0] | ((unsigned)x[1] << 8));
-    __builtin_amdgcn_raw_buffer_store_b16(t, r, (int)((unsigned)off + so), 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b16(t, r, (int)((unsigned)off + so), 0, MPL_ST_AUX);
   } else {
 #pragma unroll
     for (int j = 0; j < R; ++j)
-      __builtin_amdgcn_raw_buffer_store_b8((unsigned char)x[j], r, (int)((unsigned)(off + j) + so), 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b8((unsigned char)x[j], r, (int)((unsigned)(off + j) + so), 0, MPL_ST_AUX);
   }
 }
 
@@ -371,8 +381,9 @@ void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t
 template <int R>
 void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 
+// a_s (kMaxL floats) + the context: (L,L) for 2-D tables and for the one-label-per-lane dense path
 inline size_t fwd_lds_bytes(int L, int ctx2d) {
-  return sizeof(float) * (kMaxL + (ctx2d ? L * L : L));
+  return sizeof(float) * (kMaxL + ((ctx2d || L <= kWave) ? L * L : L));
 }
 
 }  // namespace mpl

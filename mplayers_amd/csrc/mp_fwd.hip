@@ -55,6 +55,27 @@ __device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&val
   __syncthreads();
 }
 
+// Dense step for L <= 64 (one label per lane): a[fd] is broadcast with v_readlane and the context
+// comes from a full table tab[fd * L + cd] in LDS, which consecutive lanes read without bank
+// conflicts.  Same scan order as dense_step.
+template <bool TRAIN>
+__device__ __forceinline__ void dense_step_r1(float a, int L, float w, int lane, const float* tab,
+                                              float& v, int& fd_idx) {
+  const float* col = tab + (lane < L ? lane : L - 1);
+  float best = INFINITY;
+  int arg = L - 1;
+#pragma unroll 4
+  for (int fd = L - 1; fd >= 0; --fd) {
+    const float af = readlane_f(a, fd);
+    const float val = fmaf(w, col[fd * L], af);
+    const bool take = (fd == L - 1) || (val < best);
+    best = take ? val : best;
+    if (TRAIN) arg = take ? fd : arg;
+  }
+  v = best;
+  fd_idx = arg;
+}
+
 // Band O(L*K) step for 1-D contexts with a constant tail (c[k] == cmax for k >= K, c[k] <= cmax
 // below), exact for w >= 0:
 //   v[cd] = min( min_{|k|<K} a[cd+k] + w*c[|k|],  min_fd a[fd] + w*cmax )
@@ -258,6 +279,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
           nmin = fmaf(w, KT > 0 ? c_reg[0] : ctx_s[0], amin);
           need_nmin = false;
         }
+      } else if (R == 1 && KT < 0) {
+        dense_step_r1<TRAIN>(a[0], L, w, lane, ctx_s, v[0], fd_idx[0]);
       } else if (live) {
         dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
       } else {
@@ -321,8 +344,17 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
     desc.pad = 0;
   }
   // context table into LDS (dense path, run-time band taps, negative-weight fallback)
-  const int n_ctx = p.ctx2d ? L * L : L;
-  for (int i = lane; i < n_ctx; i += kWave) ctx_s[i] = p.ctx[i];
+  if (R == 1 && desc.band_k == 0) {
+    // full symmetric table for dense_step_r1: tab[fd * L + cd] = ctx(cd, fd), TRWP_forward.cu:101-113
+    for (int i = lane; i < L * L; i += kWave) {
+      const int fd = i / L, cd = i - fd * L;
+      const int lo = cd < fd ? cd : fd, hi = cd < fd ? fd : cd;
+      ctx_s[i] = p.ctx[p.ctx2d ? lo * L + hi : hi - lo];
+    }
+  } else {
+    const int n_ctx = p.ctx2d ? L * L : L;
+    for (int i = lane; i < n_ctx; i += kWave) ctx_s[i] = p.ctx[i];
+  }
   __syncthreads();
 
   switch (desc.band_k) {
