@@ -413,9 +413,11 @@ void fill_dirs(const mpl_shape* s, int first, int count, int* dirs, int* prefix,
   }
 }
 
+int labels_per_lane(int L) { return (L + kWave - 1) / kWave; }
+
 void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st);
-  switch ((p.L + kWave - 1) / kWave) {
+  switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_fwd<1>(p, train, jacobi, st); break;
     case 2: launch_sweep_fwd<2>(p, train, jacobi, st); break;
     case 3: launch_sweep_fwd<3>(p, train, jacobi, st); break;
@@ -425,7 +427,7 @@ void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
 
 void launch_bwd(const BackParams& p, bool jacobi, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st);
-  switch ((p.L + kWave - 1) / kWave) {
+  switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_bwd<1>(p, jacobi, st); break;
     case 2: launch_sweep_bwd<2>(p, jacobi, st); break;
     case 3: launch_sweep_bwd<3>(p, jacobi, st); break;

@@ -272,6 +272,10 @@ __device__ __forceinline__ void chain_start(const DirGeom& g, int H, int W, int 
   if (c < g.count_a) {
     int r = c / W;
     ww = c - r * W;
+    // enumerate so that chain lengths first grow, then (second branch) shrink, whatever the sign of
+    // the column step: with the lengths of a diagonal sweep ordered long-first the SIMDs that drew
+    // several long chains finished 15 % later than the rest
+    if (g.ws > 0) ww = W - 1 - ww;
     hh = g.hs > 0 ? r : H - 1 - r;
   } else {
     int cc = c - g.count_a;
