@@ -125,14 +125,54 @@ __global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ u
   }
 }
 
+// ISGMR: every direction of an iteration reads the old messages only through
+//   U_d = rho * (unary + sum_k m_k - m_d) - m_{d^1}      (UpdateUnaryKernel, ISGMR_forward.cu:101-121)
+// so U_d is stored once per iteration (in place of m_d, or into the other message buffer) before
+// the sweeps: a sweep then reads one plane per pixel, not three.
+template <int V, int ND>
+__global__ void __launch_bounds__(256) isgmr_unary_kernel(const float* __restrict__ unary,
+                                                          const float* msg, float* out,
+                                                          int n_dir_rt, int64_t N, float rho) {
+  constexpr int KD = ND > 0 ? ND : kMaxDirs;
+  const int n_dir = ND > 0 ? ND : n_dir_rt;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
+       i += (int64_t)gridDim.x * blockDim.x * V) {
+    Pack<V> S = ld_pack<V>(unary + i);
+    Pack<V> m[KD];
+#pragma unroll
+    for (int k = 0; k < KD; ++k) {
+      if (k < n_dir) {
+        m[k] = ld_pack<V>(msg + (int64_t)k * N + i);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) m[k].v[j] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < KD; ++k)
+      if (k < n_dir) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) S.v[j] += m[k].v[j];  // k ascending, as the reference sums
+      }
+#pragma unroll
+    for (int k = 0; k < KD; ++k) {
+      if (k < n_dir) {
+        Pack<V> u;
+#pragma unroll
+        for (int j = 0; j < V; ++j) u.v[j] = fmaf(S.v[j] - m[k].v[j], rho, -m[k ^ 1].v[j]);
+        st_pack<V>(out + (int64_t)k * N + i, u);  // out == msg: in place
+      }
+    }
+  }
+}
+
 // cost = factor*unary + sum_k m_k  (or + min_k m_k): CostAggregateKernel, TRWP_forward.cu:31-58,
-// ISGMR_forward.cu:69-99.  copy_to != null: also mirror the message planes there.
+// ISGMR_forward.cu:69-99.
 template <int V, int ND>
 __global__ void __launch_bounds__(256) aggregate_kernel(const float* __restrict__ unary,
                                                         const float* __restrict__ msg, int n_dir_rt,
                                                         int64_t N, float factor, int min_a_dir,
-                                                        float* __restrict__ cost,
-                                                        float* __restrict__ copy_to) {
+                                                        float* __restrict__ cost) {
   const int n_dir = ND > 0 ? ND : n_dir_rt;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
        i += (int64_t)gridDim.x * blockDim.x * V) {
@@ -141,7 +181,6 @@ __global__ void __launch_bounds__(256) aggregate_kernel(const float* __restrict_
     for (int j = 0; j < V; ++j) v.v[j] *= factor;
     Pack<V> mn;  // min_a_dir only
     auto fold = [&](int k, const Pack<V>& m) {
-      if (copy_to) st_pack<V>(copy_to + (int64_t)k * N + i, m);
 #pragma unroll
       for (int j = 0; j < V; ++j) {
         if (!min_a_dir)
@@ -575,7 +614,7 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
     Timed timed(MPL_KERNEL_AGGREGATE, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(cost_final);
     MPL_EW_LAUNCH(aggregate_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, 1.f,
-                  enable_min_a_dir, cost_final, (float*)nullptr);
+                  enable_min_a_dir, cost_final);
   }
   return launch_ok("trwp_forward");
 }
@@ -602,18 +641,23 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   p.belief = unary_update;
   p.belief_out = nullptr;
   fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
-  float* buf[2] = {msg, msg_update};
+  float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {
-    // Jacobi over directions (ISGMR_forward.cu:506-622): every direction reads the old messages;
-    // the two buffers alternate instead of being copied.
-    const float* cur = buf[it & 1];
-    float* nxt = buf[(it + 1) & 1];
+    // Jacobi over directions (ISGMR_forward.cu:506-622): every direction reads the old messages,
+    // through U; the two buffers alternate instead of being copied.  U normally overwrites the
+    // old messages and the new ones go to the other buffer; with an odd number of iterations the
+    // first one stores U in the other buffer and the new messages in `msg`, so that the final
+    // messages always end up in `msg` as in the reference.
+    float* other = (have == msg) ? msg_update : msg;
+    const bool out_of_place = (it == 0) && (n_iter & 1);
+    float* ubuf = out_of_place ? other : have;
+    float* nxt = out_of_place ? have : other;
     {
       Timed timed(MPL_KERNEL_BELIEF, st);
-      const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(cur) && aligned16(unary_update);
-      MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, cur, s->n_dir, N, unary_update);
+      const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update);
+      MPL_EW_LAUNCH(isgmr_unary_kernel, v4, s->n_dir, N, st, unary, have, ubuf, s->n_dir, N, rho);
     }
-    p.msg_in = cur;
+    p.msg_in = ubuf;
     p.msg_out = nxt;
     if (train) {
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
@@ -627,14 +671,13 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
                                                            factor, enable_min_a_dir,
                                                            label_all + it * P);
     }
+    have = nxt;
   }
-  const float* fin = buf[n_iter & 1];
   {
     Timed timed(MPL_KERNEL_AGGREGATE, st);
-    const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update) &&
-                    aligned16(cost_final);
-    MPL_EW_LAUNCH(aggregate_kernel, v4, s->n_dir, N, st, unary, fin, s->n_dir, N, factor,
-                  enable_min_a_dir, cost_final, (n_iter & 1) ? msg : (float*)nullptr);
+    const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(cost_final);
+    MPL_EW_LAUNCH(aggregate_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, factor,
+                  enable_min_a_dir, cost_final);
   }
   return launch_ok("isgmr_forward");
 }

@@ -7,7 +7,9 @@
 //     v[cd]  = min_fd a[fd] + w[p] * ctx(cd, fd)          (largest fd on ties)
 //     m[p,:] = v - min_cd v                               (largest cd on ties)
 // with U = rho * (S - m_dir_old) - m_inv_old taken from the belief plane S = unary + sum_k m_k
-// instead of re-summing all messages (UpdateUnaryKernel, TRWP_forward.cu:60-80).
+// instead of re-summing all messages (UpdateUnaryKernel, TRWP_forward.cu:60-80).  TRWP (Gauss-Seidel
+// over directions) forms U on the fly from S, m_dir, m_inv and keeps S up to date; ISGMR (Jacobi)
+// finds U of every direction precomputed in place of the old messages.
 //
 // Compiled once per R (labels per lane) with -DMPL_INST_R=<R>.
 
@@ -159,7 +161,9 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   const int64_t img_e = img_p * L;
   const int vbytes = L * 4;
   // plane bases of this batch item and direction; descriptors are formed per access
-  const float* __restrict__ bS = p.belief + img_e;
+  // Jacobi: the plane of this direction in msg_in holds U itself (written by the host's
+  // element-wise pass before the sweeps), so one plane is read per pixel instead of three
+  const float* __restrict__ bS = (JACOBI ? p.msg_in + (int64_t)dir * N : p.belief) + img_e;
   const float* __restrict__ bMd = p.msg_in + (int64_t)dir * N + img_e;
   const float* __restrict__ bMi = p.msg_in + (int64_t)(dir ^ 1) * N + img_e;
   float* __restrict__ bMo = p.msg_out + (int64_t)dir * N + img_e;
@@ -199,8 +203,10 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     const unsigned so = pp * (unsigned)vbytes;
     const int nrec = (int)(so + (unsigned)vbytes);
     buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
-    buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
-    buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
+    if (!JACOBI) {
+      buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
+      buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
+    }
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
     ld_p += ch.pstep;
     ld_t += 1;
@@ -215,8 +221,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
 #pragma unroll
     for (int j = 0; j < R; ++j) {
       prev[j] = 0.f;
-      float tt = p0.s[j] - p0.md[j];
-      float un = fmaf(tt, rho, -p0.mi[j]);
+      float un = p0.s[j];
+      if (!JACOBI) un = fmaf(p0.s[j] - p0.md[j], rho, -p0.mi[j]);
       uf[j] = valid[j] ? un : inf;
     }
     if (JACOBI) {
@@ -228,8 +234,9 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     }
   }
 
-  // memory instructions per step: 3 label vectors + the weight in, 1-2 label vectors (+ indices) out
-  constexpr int kOps = 3 * vec_ops(R, VEC) + 1 + (JACOBI ? 1 : 2) * vec_ops(R, VEC) +
+  // memory instructions per step: 1 or 3 label vectors + the weight in, 1-2 label vectors
+  // (+ indices) out
+  constexpr int kOps = (JACOBI ? 1 : 3) * vec_ops(R, VEC) + 1 + (JACOBI ? 1 : 2) * vec_ops(R, VEC) +
                        (TRAIN ? byte_ops(R, VEC) + 1 : 0);
   constexpr int D = ring_depth(kOps);
   PixF<R> ring[D];
@@ -249,8 +256,13 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       float tt[R], un[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) {
-        tt[j] = px.s[j] - px.md[j];             // unary + the other directions' messages
-        float x = fmaf(tt[j], rho, -px.mi[j]);  // UpdateUnaryKernel, TRWP_forward.cu:70-78
+        float x = px.s[j];
+        if (!JACOBI) {
+          tt[j] = px.s[j] - px.md[j];       // unary + the other directions' messages
+          x = fmaf(tt[j], rho, -px.mi[j]);  // UpdateUnaryKernel, TRWP_forward.cu:70-78
+        } else {
+          tt[j] = 0.f;
+        }
         un[j] = valid[j] ? x : inf;
       }
       const float w = uniform_f(px.w);
