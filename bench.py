@@ -27,8 +27,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # same counters read for a plain device copy of one plane (FETCH_SIZE x2.0, WRITE_SIZE x1.0); the
 # summary of those runs is kept under profiles/.  Counters cannot be read from inside this script.
 MEASURED_TRAFFIC_BYTES = {
-    ("C5", 1.0, True): {"fwd_sweep": 12.35e9, "bwd_sweep": 14.75e9,
-                        "fwd_sweep_all": 81.29e9, "bwd_sweep_all": 48.25e9},
+    ("C5", 1.0, True): {"fwd_sweep": 12.24e9, "bwd_sweep": 14.44e9,
+                        "fwd_sweep_all": 43.95e9, "bwd_sweep_all": 47.09e9},
 }
 
 
