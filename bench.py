@@ -28,15 +28,16 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # summary of those runs is kept under profiles/.  Counters cannot be read from inside this script.
 MEASURED_TRAFFIC_BYTES = {
     ("C5", 1.0, True): {"fwd_sweep": 12.24e9, "bwd_sweep": 14.44e9,
-                        "fwd_sweep_all": 43.95e9, "bwd_sweep_all": 47.09e9},
+                        # ISGMR: scan + its element-wise companion pass
+                        "fwd_sweep_all": 43.95e9 + 39.17e9, "bwd_sweep_all": 47.09e9 + 37.79e9},
 }
 
 
 def parse():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
-  ap.add_argument("--steps", type=int, default=3)
-  ap.add_argument("--warmup", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=10)
+  ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--config", default="C5")
   ap.add_argument("--scale", type=float, default=1.0, help="shrink H and W (debugging only)")
   ap.add_argument("--alg", default="both", choices=["both", "TRWP", "ISGMR"])
@@ -45,6 +46,9 @@ def parse():
   ap.add_argument("--copy-probe", action="store_true",
                   help="also run one plain device copy of one fp32 plane (reference point for "
                        "hardware byte counters)")
+  ap.add_argument("--edge-probe", action="store_true",
+                  help="also time the edge-weight producer on an image of the workload's size "
+                       "(reported under \"edge_weights\")")
   return ap.parse_args()
 
 
@@ -87,6 +91,25 @@ def cpu_baseline(cfg, budget_s=15.0):
           "sample": "%s forward only (the reference has no CPU backward), first %d rows x %d "
                     "columns of %s, %d labels, %d directions, 1 iteration, unit edge weights, "
                     "%.1f s" % (mode, rows, W, cfg["name"], L, n_dir, dt)}
+
+
+def edge_probe(B, H, W, n_dir, dev, channels=3, reps=20):
+  """exp(-|I(p) - I(q)|) weights of a (B, 3, H, W) image for n_dir directions: reads one image,
+  writes n_dir maps of its size."""
+  import torch
+  from mplayers_amd import edge_weights
+  img = torch.rand(B, channels, H, W, device=dev)
+  edge_weights.getEdgeShift("edge_net", img, n_dir)
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(reps):
+    edge_weights.getEdgeShift("edge_net", img, n_dir)
+  torch.cuda.synchronize()
+  ms = (time.perf_counter() - t0) / reps * 1e3
+  nbytes = B * channels * H * W * 4 * (1 + n_dir)
+  return {"mode": "edge_net", "image": [B, channels, H, W], "n_dirs": n_dir, "ms": ms,
+          "algorithmic_GBs": nbytes / (ms * 1e-3) / 1e9,
+          "note": "wall time per call including the allocation of the result"}
 
 
 def main():
@@ -172,26 +195,33 @@ def main():
   # One launch handles N labels of one direction (TRWP) or of all n_dir directions (ISGMR).
   fwd_b = (21.0 + 1.0 / L) if training else 20.0
   bwd_b = 25.0 + 1.0 / L
-  # kind -> (bytes per label and direction sweep, direction sweeps per launch)
-  model = {"fwd_sweep": (fwd_b, 1), "bwd_sweep": (bwd_b, 1),
-           "fwd_sweep_all": (fwd_b, n_dir), "bwd_sweep_all": (bwd_b, n_dir)}
+  # kind -> (bytes per label and direction sweep, direction sweeps per launch, companion pass)
+  # ISGMR splits the work of a sweep between the scan kernel and one element-wise pass per
+  # iteration (forward: U of every direction; backward: gradient recombination); its rate is
+  # computed over both, so that it stays comparable with the algorithmic byte count.
+  model = {"fwd_sweep": (fwd_b, 1, None), "bwd_sweep": (bwd_b, 1, None),
+           "fwd_sweep_all": (fwd_b, n_dir, "unary_all"), "bwd_sweep_all": (bwd_b, n_dir, "combine")}
   kernels = {}
-  for kind, (bpl, dirs_per_launch) in model.items():
+  for kind, (bpl, dirs_per_launch, companion) in model.items():
     n, ms = stats[kind]
     if n == 0:
       continue
     per_launch = bpl * N * dirs_per_launch  # algorithmic bytes one launch moves
-    kernels[kind] = {"launches": n, "avg_ms": ms / n, "total_ms": ms,
+    both_ms = ms + (stats[companion][1] if companion else 0.0)
+    kernels[kind] = {"launches": n, "avg_ms": ms / n, "total_ms": both_ms,
                      "bytes_per_launch": per_launch,
-                     "achieved_GBs": per_launch / (ms / n * 1e-3) / 1e9,
+                     "achieved_GBs": per_launch / (both_ms / n * 1e-3) / 1e9,
                      "bytes_per_label_sweep": bpl}
+    if companion:
+      kernels[kind]["companion_pass"] = companion
+      kernels[kind]["companion_avg_ms"] = stats[companion][1] / n
   dominant = max(kernels, key=lambda k: kernels[k]["total_ms"])
   traffic = MEASURED_TRAFFIC_BYTES.get((cfg["name"], a.scale, training), {}).get(dominant)
   roofline = {"bound": "hbm", "kernel": dominant, "achieved": kernels[dominant]["achieved_GBs"],
               "peak": HBM_PEAK_GBS, "unit": "GB/s",
               "frac": kernels[dominant]["achieved_GBs"] / HBM_PEAK_GBS, "traffic": traffic,
               "algorithmic_bytes_per_launch": kernels[dominant]["bytes_per_launch"],
-              "avg_launch_ms": kernels[dominant]["avg_ms"]}
+              "avg_launch_ms": kernels[dominant]["total_ms"] / kernels[dominant]["launches"]}
   # whole-step roofline fraction against the contract bytes per unit (n_dir * (fwd + bwd))
   contract = n_dir * (fwd_b + (bwd_b if training else 0.0))
   whole = contract * value / 1e9 / HBM_PEAK_GBS
@@ -212,7 +242,10 @@ def main():
       "kernels": {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in v.items()}
                   for k, v in kernels.items()},
       "other_kernels_ms": {k: round(stats[k][1], 3) for k in stats if k not in kernels},
+
   }
+  if a.edge_probe:
+    out["edge_weights"] = edge_probe(B, H, W, n_dir, dev)
   if not a.no_cpu_baseline:
     out["cpu_baseline"] = cpu_baseline(cfg)
   print(json.dumps(out))

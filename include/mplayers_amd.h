@@ -64,7 +64,8 @@ int mpl_trwp_backward(const mpl_shape* shape, float rho, int n_iter, const float
                       void* stream);
 
 /* Replaces lib_*.ISGMR.forward: MPLayers/ISGMR/ISGMR.cpp:300-342 -> ISGMR_forward.cu:433-665.
- * msg_update: second message buffer (zero-filled); on return msg holds the final messages. */
+ * msg_update: second message buffer (any contents); on return msg holds the final messages,
+ * msg_update intermediate values; unary_update is accepted and unused. */
 int mpl_isgmr_forward(const mpl_shape* shape, int enable_sgm, float rho, int n_iter,
                       int enable_min_a_dir, const float* unary, const float* context,
                       const float* edge_weights, float* msg, float* cost_final,
@@ -90,14 +91,15 @@ int mpl_selftest_wave_ops(int* out_host);
  * launch; nothing is recorded outside such a bracket.  One bracket at a time per process. */
 #define MPL_KERNEL_FWD_SWEEP 0      /* forward scan of one direction (TRWP) */
 #define MPL_KERNEL_BWD_SWEEP 1      /* reverse scan of one direction (TRWP) */
-#define MPL_KERNEL_BELIEF 2         /* S = unary + sum of messages */
+#define MPL_KERNEL_BELIEF 2         /* S = unary + sum of messages (TRWP, once per call) */
 #define MPL_KERNEL_AGGREGATE 3      /* cost_final */
 #define MPL_KERNEL_LABEL 4          /* per-iteration labels */
 #define MPL_KERNEL_COMBINE 5        /* ISGMR backward: per-iteration gradient recombination */
 #define MPL_KERNEL_OTHER 6
 #define MPL_KERNEL_FWD_SWEEP_ALL 7  /* forward scan of all directions in one launch (ISGMR) */
 #define MPL_KERNEL_BWD_SWEEP_ALL 8  /* reverse scan of all directions in one launch (ISGMR) */
-#define MPL_KERNEL_KINDS 9
+#define MPL_KERNEL_UNARY_ALL 9     /* ISGMR forward: per-iteration U of every direction */
+#define MPL_KERNEL_KINDS 10
 typedef struct mpl_kernel_stat {
   int launches;
   double total_ms;
@@ -110,6 +112,28 @@ int mpl_profile_end(mpl_kernel_stat* stats, int n_stats);
  * counts trees of the two-pixel steps that never enter the image).  Host-only helper; -1 for a
  * direction outside the table. */
 int mpl_n_chains(int dir, int height, int width);
+
+/* Edge-weight producer, the layer's immediate upstream: replaces getEdgeShift of
+ * utils/edge_weights.py:45-111.  image (batch, channels, H, W) fp32 -> out (n_dirs, batch, channels,
+ * H, W) fp32, fully written: for direction d with step r_d and every pixel p whose front neighbour
+ * q = p - r_d is inside the image, out[d, p] = f_mode(|I(p) - I(q)|); 0 where q is outside.
+ * The channel-reducing modes (SUPERPIXEL, CUE_REAL, CUE_BINARY, THRESHOLD) take batch == 1 and
+ * write their per-pixel value to every channel plane, as the reference's broadcasting assignment
+ * does for one image.  dir_sums: 16 doubles of device scratch, used by CUE_BINARY only (may be
+ * NULL otherwise).  Modes are the reference's edge_mode strings: */
+#define MPL_EDGE_GT 0          /* 'gt_edge': 1 where equal and the pixel is not 255, else 0 */
+#define MPL_EDGE_SUPERPIXEL 1  /* 'superpixel_edge': 1 where all channels are equal */
+#define MPL_EDGE_LINEAR 2      /* 'sobel', 'edge_net_sigmoid': 1 - diff */
+#define MPL_EDGE_CANNY 3       /* 'canny': 1 - diff, diff forced to 1 on edge pixels (value 1) */
+#define MPL_EDGE_EXP 4         /* 'edge_net': exp(-diff) */
+#define MPL_EDGE_CUE_REAL 5    /* 'kernel_cue_real': exp(-mean_c(diff^2) / (2 sigma^2)) */
+#define MPL_EDGE_CUE_BINARY 6  /* 'kernel_cue_binary': CUE_REAL >= 0.8 * its mean over valid pixels */
+#define MPL_EDGE_THRESHOLD 7   /* 'threshold': penalty where mean_c(diff^2) < threshold, else 0 */
+#define MPL_EDGE_SHIFT 8       /* any other string: the front neighbour's value I(q) */
+#define MPL_EDGE_MODES 9
+int mpl_edge_shift(int mode, const float* image, int batch, int channels, int height, int width,
+                   int n_dirs, float sigma, float threshold, float penalty, float* out,
+                   double* dir_sums, void* stream);
 
 /* Message of the last failed call on this thread ("" if none). */
 const char* mpl_last_error(void);

@@ -7,10 +7,10 @@ LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hi
 
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
            "mpl_selftest_wave_ops", "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
-           "mpl_last_error", "mpl_version")
+           "mpl_last_error", "mpl_version", "mpl_edge_shift")
 
 KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combine", "other",
-                "fwd_sweep_all", "bwd_sweep_all")
+                "fwd_sweep_all", "bwd_sweep_all", "unary_all")
 
 
 class Shape(ctypes.Structure):

@@ -332,15 +332,6 @@ __global__ void __launch_bounds__(kWave) selftest_kernel(int* out) {
 // ------------------------------------------------------------------------------------------------
 thread_local char g_err[512] = "";
 
-int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
-int fail(int code, const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_err, sizeof(g_err), fmt, ap);
-  va_end(ap);
-  return code;
-}
-
 // Optional per-kernel timing with HIP events on the launch stream (off unless mpl_profile_begin
 // was called): lets a benchmark read each kernel's average duration without an external profiler.
 struct ProfRec {
@@ -503,6 +494,16 @@ const CtxDesc* make_desc(const mpl_shape* s, const float* ctx, float* cost_final
 
 }  // namespace
 
+namespace mpl {
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+}  // namespace mpl
+
 // ------------------------------------------------------------------------------------------------
 // C ABI
 // ------------------------------------------------------------------------------------------------
@@ -653,7 +654,7 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
     float* ubuf = out_of_place ? other : have;
     float* nxt = out_of_place ? have : other;
     {
-      Timed timed(MPL_KERNEL_BELIEF, st);
+      Timed timed(MPL_KERNEL_UNARY_ALL, st);
       const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update);
       MPL_EW_LAUNCH(isgmr_unary_kernel, v4, s->n_dir, N, st, unary, have, ubuf, s->n_dir, N, rho);
     }
