@@ -46,6 +46,10 @@ def parse():
   ap.add_argument("--copy-probe", action="store_true",
                   help="also run one plain device copy of one fp32 plane (reference point for "
                        "hardware byte counters)")
+  ap.add_argument("--module-probe", action="store_true",
+                  help="also time forward+backward through the nn.Module surface, which allocates "
+                       "its buffers on every call as the reference's does (reported under "
+                       "\"module_surface\")")
   ap.add_argument("--edge-probe", action="store_true",
                   help="also time the edge-weight producer on an image of the workload's size "
                        "(reported under \"edge_weights\")")
@@ -91,6 +95,38 @@ def cpu_baseline(cfg, budget_s=15.0):
           "sample": "%s forward only (the reference has no CPU backward), first %d rows x %d "
                     "columns of %s, %d labels, %d directions, 1 iteration, unit edge weights, "
                     "%.1f s" % (mode, rows, W, cfg["name"], L, n_dir, dt)}
+
+
+def module_probe(cfg, algs, unary, edge, dcost, reps=3):
+  """forward + backward of MPModule (buffers allocated inside every call, as the reference's
+  autograd functions do), per algorithm: wall ms per call."""
+  import torch
+  from mplayers_amd import MPModule
+  res = {}
+  u = unary.permute(0, 1, 4, 2, 3).contiguous().requires_grad_(True)        # (B, cv, L, H, W)
+  e = edge[:, :, 0].permute(1, 0, 2, 3).contiguous().requires_grad_(True)   # (B, n_dir, H, W)
+  g = dcost.permute(0, 1, 4, 2, 3).contiguous()
+  for alg in algs:
+    ns = argparse.Namespace(mpnet_mrf_mode=alg, mpnet_max_iter=cfg["n_iter"],
+                            mpnet_n_dirs=cfg["n_dir"], n_classes=cfg["L"], mpnet_term_weight=1.0,
+                            mpnet_smoothness_train="", mpnet_smoothness_mode="TL",
+                            mpnet_smoothness_trunct_value=3, mpnet_smoothness_trunct_loc=-1,
+                            mpnet_diag_value=0.0, enable_symmetric=True, enable_cuda=True)
+    mod = MPModule(ns, enable_create_label_context=True).cuda().train()
+    times = []
+    for r in range(reps + 1):
+      u.grad = e.grad = None
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      cost = mod(u, e)[0]
+      cost.backward(g)
+      torch.cuda.synchronize()
+      times.append((time.perf_counter() - t0) * 1e3)
+      del cost
+    res[alg] = {"ms_per_call": sum(times[1:]) / reps}
+  res["note"] = ("includes the per-call allocation of messages, indices and gradients, the two "
+                 "layout permutes of the module and autograd's bookkeeping")
+  return res
 
 
 def edge_probe(B, H, W, n_dir, dev, channels=3, reps=20):
@@ -244,6 +280,8 @@ def main():
       "other_kernels_ms": {k: round(stats[k][1], 3) for k in stats if k not in kernels},
 
   }
+  if a.module_probe and training:
+    out["module_surface"] = module_probe(cfg, algs, unary, edge, dcost)
   if a.edge_probe:
     out["edge_weights"] = edge_probe(B, H, W, n_dir, dev)
   if not a.no_cpu_baseline:

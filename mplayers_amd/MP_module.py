@@ -27,37 +27,43 @@ _EMPTY_U8 = dict(dtype=torch.uint8)
 
 
 def _forward_buffers(unary, args, n_dir, n_iter, with_message_tmp):
-  """Allocates what the operators fill in place (MP_module.py:26-45, 97-118)."""
+  """Allocates what the operators fill in place (MP_module.py:26-45, 97-118).  Only the initial
+  messages have to be zero: the library writes every element of the other tensors that is ever
+  read (index bytes of chain-start pixels stay unwritten and are never used), so they are
+  allocated without the memset the reference pays for."""
   batch, cv, h, w, n_disp = unary.size()
   buf = dict(
       message=unary.new_zeros(n_dir, batch, cv, h, w, n_disp),
-      cost_final=unary.new_zeros(batch, cv, h, w, n_disp),
-      unary_update=unary.new_zeros(batch, cv, h, w, n_disp))
+      cost_final=unary.new_empty(batch, cv, h, w, n_disp),
+      unary_update=unary.new_empty(batch, cv, h, w, n_disp))
   if with_message_tmp:
-    buf["message_tmp"] = unary.new_zeros(n_dir, batch, cv, h, w, n_disp)
+    buf["message_tmp"] = unary.new_empty(n_dir, batch, cv, h, w, n_disp)
   if args.training:
-    buf["message_index"] = unary.new_zeros(n_iter, n_dir, batch, cv, h, w, n_disp, **_EMPTY_U8)
-    buf["cost_index"] = unary.new_zeros(n_iter, n_dir, batch, cv, h, w, **_EMPTY_U8)
+    buf["message_index"] = unary.new_empty(n_iter, n_dir, batch, cv, h, w, n_disp, **_EMPTY_U8)
+    buf["cost_index"] = unary.new_empty(n_iter, n_dir, batch, cv, h, w, **_EMPTY_U8)
   else:
     buf["message_index"] = torch.empty(0, **_EMPTY_U8)
     buf["cost_index"] = torch.empty(0, **_EMPTY_U8)
   if args.enable_saving_label:
-    buf["label_all"] = unary.new_zeros(n_iter, batch, cv, h, w, **_EMPTY_U8)
+    buf["label_all"] = unary.new_empty(n_iter, batch, cv, h, w, **_EMPTY_U8)
   else:
     buf["label_all"] = torch.empty(0, **_EMPTY_U8)
   return buf
 
 
 def _backward_buffers(dcost_final, message_index, with_message_tmp):
-  """Allocates the gradient tensors (MP_module.py:65-74, 139-150)."""
+  """Allocates the gradient tensors (MP_module.py:65-74, 139-150).  dedge_weights and
+  dlabel_context accumulate and start at zero; dunary is written everywhere and the scratch
+  tensors are written before they are read."""
   n_iter, n_dir, batch, cv, h, w, n_disp = message_index.size()
   buf = dict(
-      dunary=dcost_final.new_zeros(batch, cv, h, w, n_disp),
-      dmessage=dcost_final.new_zeros(n_dir, batch, cv, h, w, n_disp),
-      dunary_update=dcost_final.new_zeros(batch, cv, h, w, n_disp),
+      dunary=dcost_final.new_empty(batch, cv, h, w, n_disp),
+      dmessage=dcost_final.new_empty(n_dir, batch, cv, h, w, n_disp),
+      dunary_update=dcost_final.new_empty(0),
       dedge_weights=dcost_final.new_zeros(n_dir, batch, cv, h, w))
   if with_message_tmp:
-    buf["dmessage_tmp"] = dcost_final.new_zeros(n_dir, batch, cv, h, w, n_disp)
+    buf["dmessage_tmp"] = dcost_final.new_empty(n_dir, batch, cv, h, w, n_disp)
+    buf["dmessage"] = dcost_final.new_empty(0)  # ISGMR's backward keeps everything in dmessage_tmp
   if n_disp == 21:
     buf["dlabel_context"] = dcost_final.new_zeros(n_disp, n_disp)
   else:

@@ -39,9 +39,10 @@ constexpr int kMaxBandK = 32;   // widest band handled by the O(L*K) path
 #endif
 constexpr int kPrefetch = MPL_PREFETCH;  // upper limit of pixels in flight per wave
 
-// The hardware counter of outstanding vector-memory operations of a wave has 6 bits; runs with more
-// than 63 loads and stores in flight per wave returned corrupted data.  The prefetch ring is
-// therefore sized from the number of memory instructions a step issues, to stay below kMaxInFlight.
+// The hardware counter of outstanding vector-memory operations of a wave has 6 bits (63 at most).
+// The prefetch ring is sized from the number of memory instructions a step issues so that a wave
+// never has more than kMaxInFlight of them outstanding: the explicit waits of the scan loops then
+// stay exact, and a deeper ring buys nothing (2 to 8 pixels ahead measure the same).
 #ifndef MPL_MAX_INFLIGHT
 #define MPL_MAX_INFLIGHT 52
 #endif
