@@ -174,3 +174,54 @@ def refcpu_forward(mode, unary, context, n_dir, n_iter, rho, n_threads=16, ctx2d
                                    _ptr(unary), _ptr(context), ctypes.c_int64(stride), _ptr(msg),
                                    _ptr(msg_update), _ptr(cost), int(n_threads))
   return dict(msg=msg, cost_final=cost)
+
+
+def forward_soft(unary, context, edge_weights, n_dir, n_iter, rho, training=True,
+                 saving_label=False, ctx2d=None):
+  """Restated ForwardCUDASoft (TRWP_hard_soft/TRWP_forward_soft.cu:378-559).
+
+  Returns a dict with msg, cost_final, msg_edge_label (n_iter, n_dir, B, cv, H, W, L, L),
+  msg_norm_index and label_all (None where switched off)."""
+  unary = np.ascontiguousarray(unary)
+  sfx, creal = _real(unary.dtype)
+  dt = unary.dtype
+  b, cv, h, w, L = unary.shape
+  g = _geom(n_dir, unary.shape, ctx2d)
+  context = np.ascontiguousarray(context, dtype=dt)
+  if edge_weights is None:
+    edge_weights = np.ones((n_dir, b, cv, h, w), dtype=dt)
+  edge_weights = np.ascontiguousarray(edge_weights, dtype=dt)
+  msg = np.zeros((n_dir, b, cv, h, w, L), dtype=dt)
+  cost = np.zeros((b, cv, h, w, L), dtype=dt)
+  mel = np.zeros((n_iter, n_dir, b, cv, h, w, L, L), dtype=dt) if training else None
+  inorm = np.zeros((n_iter, n_dir, b, cv, h, w), dtype=np.uint8) if training else None
+  label = np.zeros((n_iter, b, cv, h, w), dtype=np.uint8) if saving_label else None
+  fn = getattr(lib(), "mpo_trwp_soft_forward_" + sfx)
+  fn(ctypes.byref(g), creal(rho), int(n_iter), _ptr(unary), _ptr(context), _ptr(edge_weights),
+     _ptr(msg), _ptr(cost), _ptr(mel), _ptr(inorm), _ptr(label))
+  return dict(msg=msg, cost_final=cost, msg_edge_label=mel, msg_norm_index=inorm, label_all=label)
+
+
+def backward_soft(context, edge_weights, dcost_final, msg_edge_label, msg_norm_index, rho,
+                  ctx2d=None):
+  """Restated BackwardCUDASoft (TRWP_hard_soft/TRWP_backward_soft.cu:422-548).
+  Returns (dunary, dcontext, dedge_weights)."""
+  dcost_final = np.ascontiguousarray(dcost_final)
+  sfx, creal = _real(dcost_final.dtype)
+  dt = dcost_final.dtype
+  n_iter, n_dir, b, cv, h, w, L, _ = msg_edge_label.shape
+  g = _geom(n_dir, (b, cv, h, w, L), ctx2d)
+  context = np.ascontiguousarray(context, dtype=dt)
+  if edge_weights is None:
+    edge_weights = np.ones((n_dir, b, cv, h, w), dtype=dt)
+  edge_weights = np.ascontiguousarray(edge_weights, dtype=dt)
+  msg_edge_label = np.ascontiguousarray(msg_edge_label, dtype=dt)
+  msg_norm_index = np.ascontiguousarray(msg_norm_index)
+  dunary = np.zeros((b, cv, h, w, L), dtype=dt)
+  dcontext = np.zeros((L, L) if g.ctx2d else (L,), dtype=dt)
+  dedge = np.zeros((n_dir, b, cv, h, w), dtype=dt)
+  fn = getattr(lib(), "mpo_trwp_soft_backward_" + sfx)
+  fn(ctypes.byref(g), creal(rho), int(n_iter), _ptr(context), _ptr(edge_weights),
+     _ptr(dcost_final), _ptr(msg_edge_label), _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
+     _ptr(dedge))
+  return dunary, dcontext, dedge

@@ -345,3 +345,197 @@ int FN(mpo_isgmr_backward)(const mpo_geom* g, int enable_sgm, REAL rho, int n_it
   free(dU);
   return 0;
 }
+
+/* =========================================================================================== */
+/* Soft-weighted TRWP (MPLayers/TRWP_hard_soft): the min over front labels is replaced by the     */
+/* expectation of the dual under softmin weights.                                                 */
+/* =========================================================================================== */
+
+/* offset of (cd, fd) inside a pixel's (L, L) block of msg_edge_label: even directions store      */
+/* [fd][cd], odd ones [cd][fd] (is_pass_l2r = dir % 2 == 0, common.cpp:20;                        */
+/* TRWP_forward_soft.cu:64)                                                                        */
+static inline int64_t FN(soft_loc)(int L, int dir, int cd, int fd) {
+  return (dir % 2 == 0) ? (int64_t)fd * L + cd : (int64_t)cd * L + fd;
+}
+
+/* softmin statistics of one row dual[0..L-1] (front labels): TRWP_forward_soft.cu:74-97.         */
+/* prob may be NULL.  Returns the soft message sum_fd prob*dual.                                  */
+static REAL FN(soft_row)(int L, const REAL* dual, REAL* prob) {
+  REAL mn = dual[0];
+  for (int fd = 1; fd < L; ++fd)
+    if (dual[fd] < mn) mn = dual[fd];
+  REAL s = 0;
+  for (int fd = 0; fd < L; ++fd) s += (REAL)exp((double)(-dual[fd] + mn));
+  REAL soft = 0;
+  for (int fd = 0; fd < L; ++fd) {
+    REAL e = (REAL)exp((double)(-dual[fd] + mn));
+    if (prob) prob[fd] = e / s;
+    soft += e * dual[fd] / s;
+  }
+  return soft;
+}
+
+/* one pixel of DynamicProgramming: TRWP_forward_soft.cu:9-117.  edge_label: the pixel's (L,L)     */
+/* block or NULL.  Norm index: largest label on ties (TRWP_soft.cuh:104-108, torch >= 1).          */
+static void FN(pixel_step_soft)(int L, int ctx2d, int dir, REAL rho, const REAL* Ufront,
+                                const REAL* context, REAL w, REAL* prev, REAL* tmp, REAL* row,
+                                REAL* m_out, REAL* edge_label, uint8_t* idx_norm) {
+  for (int cd = 0; cd < L; ++cd) {
+    for (int fd = 0; fd < L; ++fd) {
+      REAL cv = context[FN(ctx_offset)(L, ctx2d, cd, fd)];
+      row[fd] = Ufront[fd] + rho * prev[fd] + w * cv; /* :69 */
+      if (edge_label) edge_label[FN(soft_loc)(L, dir, cd, fd)] = row[fd];
+    }
+    tmp[cd] = FN(soft_row)(L, row, NULL);
+  }
+  REAL nmin = tmp[0];
+  int narg = 0;
+  for (int cd = 1; cd < L; ++cd)
+    if (tmp[cd] <= nmin) { /* equal: the larger index wins */
+      nmin = tmp[cd];
+      narg = cd;
+    }
+  for (int cd = 0; cd < L; ++cd) {
+    prev[cd] = tmp[cd] - nmin;
+    m_out[cd] = prev[cd];
+  }
+  if (idx_norm) *idx_norm = (uint8_t)narg;
+}
+
+/* Horizontal/DiagonalWide/DiagonalNarrow KernelSoft: TRWP_forward_soft.cu:183-376 (same chain     */
+/* geometry as the hard kernels)                                                                   */
+static void FN(sweep_soft)(const mpo_geom* g, int dir, REAL rho, const REAL* U, const REAL* context,
+                           const REAL* w_dir, REAL* m_out, REAL* edge_label, uint8_t* idx_norm) {
+  int L = g->L, H = g->H, W = g->W;
+  int hs, ws;
+  mpo_dir_step(dir, &hs, &ws);
+  int n_trees = mpo_n_trees(dir, H, W);
+  REAL* prev = (REAL*)malloc(sizeof(REAL) * L);
+  REAL* tmp = (REAL*)malloc(sizeof(REAL) * L);
+  REAL* row = (REAL*)malloc(sizeof(REAL) * L);
+  for (int bv = 0; bv < g->B; ++bv) {
+    int64_t pix_base = (int64_t)bv * H * W;
+    for (int tree = 0; tree < n_trees; ++tree) {
+      int h0, w0, n_roll;
+      mpo_tree_start(dir, hs, ws, H, W, tree, &h0, &w0, &n_roll);
+      for (int l = 0; l < L; ++l) prev[l] = 0;
+      for (int i = 0; i <= n_roll; ++i) {
+        int ch = h0 + i * hs, cw = w0 + i * ws;
+        int fh = ch - hs, fw = cw - ws;
+        if (ch < 0 || ch >= H || cw < 0 || cw >= W || fh < 0 || fh >= H || fw < 0 || fw >= W)
+          continue;
+        int64_t pc = pix_base + (int64_t)ch * W + cw;
+        int64_t pf = pix_base + (int64_t)fh * W + fw;
+        FN(pixel_step_soft)(L, g->ctx2d, dir, rho, U + pf * L, context, w_dir[pc], prev, tmp, row,
+                            m_out + pc * L, edge_label ? edge_label + pc * L * L : NULL,
+                            idx_norm ? idx_norm + pc : NULL);
+      }
+    }
+  }
+  free(prev);
+  free(tmp);
+  free(row);
+}
+
+/* ForwardCUDASoft: TRWP_forward_soft.cu:378-559.  msg_edge_label (n_iter,n_dir,B,H,W,L,L) and      */
+/* msg_norm_index (n_iter,n_dir,B,H,W) may both be NULL (inference).                               */
+int FN(mpo_trwp_soft_forward)(const mpo_geom* g, REAL rho, int n_iter, const REAL* unary,
+                              const REAL* context, const REAL* edge_weights, REAL* msg,
+                              REAL* cost_final, REAL* msg_edge_label, uint8_t* msg_norm_index,
+                              uint8_t* label_all) {
+  int64_t N = mpo_plane(g), P = mpo_pixels(g);
+  REAL* U = (REAL*)malloc(sizeof(REAL) * N);
+  for (int it = 0; it < n_iter; ++it) {
+    for (int d = 0; d < g->n_dir; ++d) {
+      int64_t io = ((int64_t)it * g->n_dir + d);
+      FN(update_unary)(g, d, rho, unary, msg, U); /* UpdateUnaryKernelSoft :161-181, same formula */
+      FN(sweep_soft)(g, d, rho, U, context, edge_weights + (int64_t)d * P, msg + (int64_t)d * N,
+                     msg_edge_label ? msg_edge_label + io * N * g->L : NULL,
+                     msg_norm_index ? msg_norm_index + io * P : NULL);
+    }
+    if (label_all) {
+      FN(cost_aggregate)(g, 0, 1, unary, msg, cost_final); /* CostAggregateKernelSoft :142-159 */
+      FN(cal_label)(g, cost_final, label_all + (int64_t)it * P); /* CalLabelKernelSoft :119-140 */
+    }
+  }
+  FN(cost_aggregate)(g, 0, 1, unary, msg, cost_final);
+  free(U);
+  return 0;
+}
+
+/* DynamicProgrammingBack over one direction: TRWP_backward_soft.cu:9-129, 170-420                  */
+static void FN(sweep_back_soft)(const mpo_geom* g, int dir, REAL rho, const REAL* context,
+                                const REAL* w_dir, const REAL* edge_label, const uint8_t* idx_norm,
+                                REAL* dmsg_dir, REAL* dU, REAL* dcontext, REAL* dedge_dir) {
+  int L = g->L, H = g->H, W = g->W;
+  int hs, ws;
+  mpo_dir_step(dir, &hs, &ws);
+  hs = -hs;
+  ws = -ws;
+  int n_trees = mpo_n_trees(dir, H, W);
+  REAL* gv = (REAL*)malloc(sizeof(REAL) * L);
+  REAL* row = (REAL*)malloc(sizeof(REAL) * L);
+  REAL* prob = (REAL*)malloc(sizeof(REAL) * L);
+  for (int bv = 0; bv < g->B; ++bv) {
+    int64_t pix_base = (int64_t)bv * H * W;
+    for (int tree = 0; tree < n_trees; ++tree) {
+      int h0, w0, n_roll;
+      mpo_tree_start(dir, hs, ws, H, W, tree, &h0, &w0, &n_roll);
+      for (int i = 0; i <= n_roll; ++i) {
+        int ch = h0 + i * hs, cw = w0 + i * ws;
+        int fh = ch + hs, fw = cw + ws;
+        if (ch < 0 || ch >= H || cw < 0 || cw >= W || fh < 0 || fh >= H || fw < 0 || fw >= W)
+          continue;
+        int64_t pc = pix_base + (int64_t)ch * W + cw;
+        int64_t pf = pix_base + (int64_t)fh * W + fw;
+        for (int l = 0; l < L; ++l) gv[l] = dmsg_dir[pc * L + l];
+        REAL s = 0; /* back norm :52-63 */
+        for (int l = 0; l < L; ++l) s += gv[l];
+        gv[idx_norm[pc]] -= s;
+        for (int cd = 0; cd < L; ++cd) {
+          for (int fd = 0; fd < L; ++fd) row[fd] = edge_label[pc * L * L + FN(soft_loc)(L, dir, cd, fd)];
+          REAL soft = FN(soft_row)(L, row, prob); /* :83-105 */
+          for (int fd = 0; fd < L; ++fd) {
+            REAL dd = gv[cd] * prob[fd] * (1 - row[fd] + soft); /* :110-113 */
+            int64_t co = FN(ctx_offset)(L, g->ctx2d, cd, fd);
+            dU[pf * L + fd] += dd;
+            dmsg_dir[pf * L + fd] += rho * dd;
+            dedge_dir[pc] += context[co] * dd;
+            dcontext[co] += w_dir[pc] * dd; /* every pair, the diagonal included :126 */
+          }
+        }
+      }
+    }
+  }
+  free(gv);
+  free(row);
+  free(prob);
+}
+
+/* BackwardCUDASoft: TRWP_backward_soft.cu:422-548 */
+int FN(mpo_trwp_soft_backward)(const mpo_geom* g, REAL rho, int n_iter, const REAL* context,
+                               const REAL* edge_weights, const REAL* dcost_final,
+                               const REAL* msg_edge_label, const uint8_t* msg_norm_index,
+                               REAL* dunary, REAL* dcontext, REAL* dedge_weights) {
+  int64_t N = mpo_plane(g), P = mpo_pixels(g);
+  REAL* dmsg = (REAL*)malloc(sizeof(REAL) * N * g->n_dir);
+  REAL* dU = (REAL*)calloc(N, sizeof(REAL));
+  for (int64_t i = 0; i < N; ++i) { /* CostAggregateKernelSoftBack :131-147 */
+    dunary[i] = dcost_final[i];
+    for (int k = 0; k < g->n_dir; ++k) dmsg[(int64_t)k * N + i] = dcost_final[i];
+  }
+  for (int it = n_iter - 1; it >= 0; --it) {
+    for (int d = g->n_dir - 1; d >= 0; --d) {
+      int64_t io = ((int64_t)it * g->n_dir + d);
+      FN(sweep_back_soft)(g, d, rho, context, edge_weights + (int64_t)d * P,
+                          msg_edge_label + io * N * g->L, msg_norm_index + io * P,
+                          dmsg + (int64_t)d * N, dU, dcontext, dedge_weights + (int64_t)d * P);
+      FN(update_unary_back)(g, d, rho, dU, dunary, dmsg); /* UpdateUnaryKernelSoftBack :149-168 */
+      memset(dU, 0, sizeof(REAL) * N);                    /* :535 */
+      memset(dmsg + (int64_t)d * N, 0, sizeof(REAL) * N); /* :536 */
+    }
+  }
+  free(dmsg);
+  free(dU);
+  return 0;
+}
