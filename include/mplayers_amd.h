@@ -80,6 +80,26 @@ int mpl_isgmr_backward(const mpl_shape* shape, int enable_sgm, float rho, int n_
                        float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
                        float* dmsg_update, void* stream);
 
+/* Soft-weighted TRWP: replaces lib_*.TRWP_hard_soft.forward_soft, MPLayers/TRWP_hard_soft/TRWP.cpp:
+ * 313-349 (ForwardSoft) -> TRWP_forward_soft.cu:378-559.  The min over front labels becomes the
+ * expectation of the dual under softmin weights.  n_disp <= 64.
+ *   msg_edge_label (n_iter, n_dir, B, H, W, L, L) fp32: every dual of every pixel, kept for the
+ *   backward pass (even directions [fd][cd], odd ones [cd][fd]); blocks of chain-start pixels are
+ *   not written.  NULL together with msg_norm_index => inference. */
+int mpl_trwp_soft_forward(const mpl_shape* shape, float rho, int n_iter, const float* unary,
+                          const float* context, const float* edge_weights, float* msg,
+                          float* msg_edge_label, uint8_t* msg_norm_index, float* cost_final,
+                          float* unary_update, uint8_t* label_all, void* stream);
+
+/* Replaces lib_*.TRWP_hard_soft.backward_soft, TRWP.cpp:351-383 (BackwardSoft) ->
+ * TRWP_backward_soft.cu:422-548.  dcontext also receives the zero-offset / diagonal terms here
+ * (the hard operator skips them).  dmsg is scratch (n_dir planes, any contents). */
+int mpl_trwp_soft_backward(const mpl_shape* shape, float rho, int n_iter, const float* dcost_final,
+                           const float* context, const float* edge_weights,
+                           const float* msg_edge_label, const uint8_t* msg_norm_index,
+                           float* dunary, float* dcontext, float* dedge_weights, float* dmsg,
+                           float* dunary_update, void* stream);
+
 /* Device check of the wavefront primitives the kernels are built on (cross-lane shifts, min/sum
  * reductions, ballots).  out: 8 host ints, out[0] == 1 when every check passed.  Synchronises. */
 int mpl_selftest_wave_ops(int* out_host);

@@ -774,4 +774,105 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
   return launch_ok("isgmr_backward");
 }
 
+// ---- soft-weighted TRWP ------------------------------------------------------------------------
+int mpl_trwp_soft_forward(const mpl_shape* s, float rho, int n_iter, const float* unary,
+                          const float* context, const float* edge_weights, float* msg,
+                          float* msg_edge_label, uint8_t* msg_norm_index, float* cost_final,
+                          float* unary_update, uint8_t* label_all, void* stream) {
+  int rc = check_shape(s, n_iter);
+  if (rc) return rc;
+  if (s->n_disp > kWave)
+    return fail(MPL_EINVAL, "trwp_soft_forward: at most %d labels (one per lane; the stored "
+                "duals take n_disp^2 floats per pixel, direction and iteration), got %d", kWave,
+                s->n_disp);
+  if (!unary || !context || !edge_weights || !msg || !cost_final || !unary_update)
+    return fail(MPL_EINVAL, "trwp_soft_forward: null tensor pointer");
+  if ((msg_edge_label == nullptr) != (msg_norm_index == nullptr))
+    return fail(MPL_EINVAL, "trwp_soft_forward: msg_edge_label and msg_norm_index go together");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t P = (int64_t)s->batch * s->height * s->width;
+  const int64_t N = P * s->n_disp;
+  const bool train = msg_edge_label != nullptr;
+  {
+    Timed timed(MPL_KERNEL_BELIEF, st);
+    const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
+    MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update);
+  }
+  SweepParams p = base_fwd_params(s, rho, edge_weights, context, nullptr);
+  p.belief = unary_update;
+  p.belief_out = unary_update;
+  p.msg_in = msg;
+  p.msg_out = msg;
+  for (int it = 0; it < n_iter; ++it) {
+    for (int d = 0; d < s->n_dir; ++d) {  // TRWP_forward_soft.cu:441-520
+      fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
+      if (train) {
+        p.edge_label = msg_edge_label + (int64_t)it * s->n_dir * N * s->n_disp;
+        p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
+      }
+      Timed timed(MPL_KERNEL_FWD_SWEEP, st);
+      launch_soft_fwd(p, train, st);
+    }
+    if (label_all) {
+      int64_t waves = (P < 256 * 64) ? P : 256 * 64;
+      Timed timed(MPL_KERNEL_LABEL, st);
+      label_kernel<<<(int)((waves + 3) / 4), 256, 0, st>>>(unary, msg, s->n_dir, P, s->n_disp, 1.f,
+                                                           0, label_all + it * P);
+    }
+  }
+  {
+    Timed timed(MPL_KERNEL_AGGREGATE, st);
+    const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(cost_final);
+    MPL_EW_LAUNCH(aggregate_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, 1.f, 0,
+                  cost_final);
+  }
+  return launch_ok("trwp_soft_forward");
+}
+
+int mpl_trwp_soft_backward(const mpl_shape* s, float rho, int n_iter, const float* dcost_final,
+                           const float* context, const float* edge_weights,
+                           const float* msg_edge_label, const uint8_t* msg_norm_index,
+                           float* dunary, float* dcontext, float* dedge_weights, float* dmsg,
+                           float* dunary_update, void* stream) {
+  (void)dunary_update;
+  int rc = check_shape(s, n_iter);
+  if (rc) return rc;
+  if (s->n_disp > kWave)
+    return fail(MPL_EINVAL, "trwp_soft_backward: at most %d labels, got %d", kWave, s->n_disp);
+  if (!context || !edge_weights || !dcost_final || !msg_edge_label || !msg_norm_index || !dunary ||
+      !dcontext || !dedge_weights || !dmsg)
+    return fail(MPL_EINVAL, "trwp_soft_backward: null tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t P = (int64_t)s->batch * s->height * s->width;
+  const int64_t N = P * s->n_disp;
+  BackParams p;
+  memset(&p, 0, sizeof(p));
+  p.B = s->batch;
+  p.H = s->height;
+  p.W = s->width;
+  p.L = s->n_disp;
+  p.ctx2d = s->ctx2d ? 1 : 0;
+  p.rho = rho;
+  p.a_out = dunary;
+  p.h = dmsg;
+  p.edge = edge_weights;
+  p.ctx = context;
+  p.dedge = dedge_weights;
+  p.dctx = dcontext;
+  bool first = true;
+  for (int it = n_iter - 1; it >= 0; --it) {
+    for (int d = s->n_dir - 1; d >= 0; --d) {  // TRWP_backward_soft.cu:454-538
+      fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
+      p.a_in = first ? dcost_final : dunary;
+      p.first_touch = (it == n_iter - 1) && (d & 1);
+      p.edge_label = msg_edge_label + (int64_t)it * s->n_dir * N * s->n_disp;
+      p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
+      Timed timed(MPL_KERNEL_BWD_SWEEP, st);
+      launch_soft_bwd(p, st);
+      first = false;
+    }
+  }
+  return launch_ok("trwp_soft_backward");
+}
+
 }  // extern "C"

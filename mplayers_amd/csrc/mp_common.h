@@ -353,6 +353,7 @@ struct SweepParams {
   const CtxDesc* desc;             // may be null: dense path
   uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
+  float* edge_label;               // soft TRWP: (n_dir_total, P, L, L) duals of this iteration, or null
 };
 
 struct BackParams {
@@ -378,6 +379,7 @@ struct BackParams {
   const uint8_t* idx_norm;  // (n_dir_total, P)
   float* dedge;             // (n_dir_total, P) accumulates
   float* dctx;              // accumulates
+  const float* edge_label;  // soft TRWP: (n_dir_total, P, L, L) duals of this iteration
 };
 
 // records the message mpl_last_error() returns on this thread and returns `code`
@@ -390,6 +392,10 @@ template <int R>
 void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 
 // a_s (kMaxL floats) + the context: (L,L) for 2-D tables and for the one-label-per-lane dense path
+// soft-weighted TRWP (mp_soft.hip): one direction per launch, L <= 64
+void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st);
+void launch_soft_bwd(const BackParams& p, hipStream_t st);
+
 inline size_t fwd_lds_bytes(int L, int ctx2d) {
   return sizeof(float) * (kMaxL + ((ctx2d || L <= kWave) ? L * L : L));
 }

@@ -163,3 +163,76 @@ class ISGMR(object):
                                   _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),
                                   _ptr(dmsg_update), _Op._stream(dcost_final))
     _lib.check(rc, "ISGMR.backward")
+
+
+class TRWP_hard_soft(object):
+  """Drop-in for the reference's `lib_stereo.TRWP_hard_soft` / `lib_seg.TRWP_hard_soft` extension
+  modules (MPLayers/TRWP_hard_soft/TRWP.cpp:428-445): the hard operators under the same names as
+  in `TRWP`, plus `forward_soft` / `backward_soft`.  `soft_weighted_message(_back)`, the stand-alone
+  softmin of a stored tensor, is not part of this build and raises."""
+
+  forward = TRWP.forward
+  backward = TRWP.backward
+
+  @staticmethod
+  def forward_soft(rho, n_iter, unary, context, edge_weights, msg, msg_edge_label, msg_norm_index,
+                   cost_final, unary_update, label_all):
+    lib = _lib.load()
+    shape, P, L, ctx2d = _Op._shape_from_msg(msg)
+    N = P * L
+    f32, u8 = torch.float32, torch.uint8
+    _check("unary", unary, f32, N)
+    _check("context", context, f32, _context_numel(L, ctx2d))
+    _check("edge_weights", edge_weights, f32, shape.n_dir * P)
+    _check("msg", msg, f32, shape.n_dir * N)
+    _check("cost_final", cost_final, f32, N)
+    _check("unary_update", unary_update, f32, N)
+    if msg_edge_label.numel() > 0:
+      _check("msg_edge_label", msg_edge_label, f32, n_iter * shape.n_dir * N * L)
+      _check("msg_norm_index", msg_norm_index, u8, n_iter * shape.n_dir * P)
+    if label_all.numel() > 0:
+      _check("label_all", label_all, u8, n_iter * P)
+    with torch.cuda.device(unary.device):
+      rc = lib.mpl_trwp_soft_forward(shape, float(rho), int(n_iter), _ptr(unary), _ptr(context),
+                                     _ptr(edge_weights), _ptr(msg), _ptr(msg_edge_label),
+                                     _ptr(msg_norm_index), _ptr(cost_final), _ptr(unary_update),
+                                     _ptr(label_all), _Op._stream(unary))
+    _lib.check(rc, "TRWP_hard_soft.forward_soft")
+
+  @staticmethod
+  def backward_soft(rho, dcost_final, context, edge_weights, msg_edge_label, msg_norm_index,
+                    dunary, dcontext, dedge_weights, dmsg, dunary_update):
+    lib = _lib.load()
+    if msg_norm_index.dim() != 6:
+      raise RuntimeError("msg_norm_index must be (n_iter, n_dir, batch, cv, h, w)")
+    n_iter, n_dir, b, cv, h, w = msg_norm_index.shape
+    L = dcost_final.size(-1)
+    ctx2d = (L == 21)
+    shape = _lib.Shape(n_dir, b * cv, h, w, L, int(ctx2d))
+    P = b * cv * h * w
+    N = P * L
+    f32, u8 = torch.float32, torch.uint8
+    _check("dcost_final", dcost_final, f32, N)
+    _check("context", context, f32, _context_numel(L, ctx2d))
+    _check("edge_weights", edge_weights, f32, n_dir * P)
+    _check("msg_edge_label", msg_edge_label, f32, n_iter * n_dir * N * L)
+    _check("msg_norm_index", msg_norm_index, u8, n_iter * n_dir * P)
+    _check("dunary", dunary, f32, N)
+    _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
+    _check("dedge_weights", dedge_weights, f32, n_dir * P)
+    _check("dmsg", dmsg, f32, n_dir * N)
+    with torch.cuda.device(dcost_final.device):
+      rc = lib.mpl_trwp_soft_backward(shape, float(rho), int(n_iter), _ptr(dcost_final),
+                                      _ptr(context), _ptr(edge_weights), _ptr(msg_edge_label),
+                                      _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
+                                      _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),
+                                      _Op._stream(dcost_final))
+    _lib.check(rc, "TRWP_hard_soft.backward_soft")
+
+  @staticmethod
+  def soft_weighted_message(*args):
+    raise RuntimeError("soft_weighted_message is not part of this build")
+
+  @staticmethod
+  def soft_weighted_message_back(*args):
+    raise RuntimeError("soft_weighted_message_back is not part of this build")

@@ -17,3 +17,14 @@ def oracle():
   from oracle import mp_oracle
   mp_oracle.build()
   return mp_oracle
+
+
+@pytest.fixture(scope="session")
+def gpu():
+  """Helpers of the GPU parity tests; fails (not skips) without a GPU or without the HIP library."""
+  import torch
+  assert torch.cuda.is_available(), "these tests need the MI355X"
+  from mplayers_amd import _lib
+  _lib.load()
+  from tests import _gpu_util
+  return _gpu_util

@@ -12,16 +12,6 @@ pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
-@pytest.fixture(scope="module")
-def gpu():
-  import torch
-  assert torch.cuda.is_available(), "these tests need the MI355X"
-  from mplayers_amd import _lib
-  _lib.load()
-  from tests import _gpu_util
-  return _gpu_util
-
-
 CONFIG_CASES = [
     # config, mode, scale, n_iter override
     ("C1", "ISGMR", 1.0, None),

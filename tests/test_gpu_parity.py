@@ -11,16 +11,6 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module")
-def gpu():
-  import torch
-  assert torch.cuda.is_available(), "these tests need the MI355X"
-  from mplayers_amd import _lib
-  _lib.load()
-  from tests import _gpu_util
-  return _gpu_util
-
-
 def test_wave_primitives(gpu):
   import ctypes
   from mplayers_amd import _lib
