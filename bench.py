@@ -40,7 +40,9 @@ def parse():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--config", default="C5")
   ap.add_argument("--scale", type=float, default=1.0, help="shrink H and W (debugging only)")
-  ap.add_argument("--alg", default="both", choices=["both", "TRWP", "ISGMR"])
+  ap.add_argument("--alg", default="both", choices=["both", "TRWP", "ISGMR", "SOFT"],
+                  help="SOFT: soft-weighted TRWP (at most 64 labels; stores n_disp^2 floats per "
+                       "pixel, direction and iteration)")
   ap.add_argument("--fwd-only", action="store_true", help="inference forward only (C2/C3 style)")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--copy-probe", action="store_true",
@@ -175,6 +177,8 @@ def main():
   u8 = dict(dtype=torch.uint8, device=dev)
   msg = torch.zeros(n_dir, B, 1, H, W, L, **f32)
   msg_tmp = torch.zeros(n_dir, B, 1, H, W, L, **f32) if "ISGMR" in algs else None
+  soft_blocks = (torch.zeros(n_iter, n_dir, B, 1, H, W, L, L, **f32)
+                 if ("SOFT" in algs and training) else torch.empty(0))
   cost = torch.zeros(B, 1, H, W, L, **f32)
   belief = torch.zeros(B, 1, H, W, L, **f32)
   empty = torch.empty(0, dtype=torch.uint8)
@@ -192,9 +196,15 @@ def main():
 
   def step():
     for alg in algs:
-      rho = 0.5 if alg == "TRWP" else 1.0
+      rho = 1.0 if alg == "ISGMR" else 0.5
       msg.zero_()
-      if alg == "TRWP":
+      if alg == "SOFT":
+        lib_stereo.TRWP_hard_soft.forward_soft(rho, n_iter, unary, context, edge, msg, soft_blocks,
+                                               inorm, cost, belief, empty)
+        if training:
+          lib_stereo.TRWP_hard_soft.backward_soft(rho, dcost, context, edge, soft_blocks, inorm,
+                                                  dunary, dctx, dedge, dmsg, dscratch)
+      elif alg == "TRWP":
         lib_stereo.TRWP.forward(rho, n_iter, 0, unary, context, edge, msg, cost, imin, inorm,
                                 belief, empty)
         if training:
@@ -231,6 +241,11 @@ def main():
   # One launch handles N labels of one direction (TRWP) or of all n_dir directions (ISGMR).
   fwd_b = (21.0 + 1.0 / L) if training else 20.0
   bwd_b = 25.0 + 1.0 / L
+  if a.alg == "SOFT":
+    # the stored duals replace the argmin index: 4*L bytes per label written forward (training)
+    # and read back
+    fwd_b = (20.0 + 4.0 * L + 1.0 / L) if training else 20.0
+    bwd_b = 24.0 + 4.0 * L + 1.0 / L
   # kind -> (bytes per label and direction sweep, direction sweeps per launch, companion pass)
   # ISGMR splits the work of a sweep between the scan kernel and one element-wise pass per
   # iteration (forward: U of every direction; backward: gradient recombination); its rate is

@@ -147,7 +147,8 @@ __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, c
   }
 }
 
-// One chain.  KT: > 0 band with compile-time K, 0 band with run-time K, -1 dense.
+// One chain.  KT: > 0 band with compile-time K, 0 band with run-time K, -1 dense, -21 dense with
+// exactly 21 labels.
 // VEC: L % R == 0 (vector accesses).  MASK: some lanes own labels >= L.
 template <int R, bool VEC, bool MASK, bool TRAIN, bool JACOBI, int KT>
 __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
@@ -188,6 +189,13 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   if (KT > 0) {
 #pragma unroll
     for (int k = 0; k < KT; ++k) c_reg[k] = p.ctx[k];
+  }
+  // KT == -21: dense path with the label count fixed at 21 (the segmentation case)
+  constexpr int LT = (KT == -21) ? 21 : 0;
+  float tcol[LT > 0 ? LT : 1];
+  if (LT > 0) {
+#pragma unroll
+    for (int fd = 0; fd < LT; ++fd) tcol[fd] = ctx_s[fd * LT + (lane < LT ? lane : LT - 1)];
   }
   const int K = desc.band_k;
   const float cmax = desc.cmax;
@@ -292,7 +300,22 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
           need_nmin = false;
         }
       } else if (R == 1 && KT < 0) {
-        dense_step_r1<TRAIN>(a[0], L, w, lane, ctx_s, v[0], fd_idx[0]);
+        if constexpr (LT > 0) {
+          // 21 labels: the scan over front labels fully unrolled, context column in registers
+          float best = inf;
+          int arg = LT - 1;
+#pragma unroll
+          for (int fd = LT - 1; fd >= 0; --fd) {
+            const float val = fmaf(w, tcol[fd], readlane_f(a[0], fd));
+            const bool take = (fd == LT - 1) || (val < best);
+            best = take ? val : best;
+            if (TRAIN) arg = take ? fd : arg;
+          }
+          v[0] = best;
+          fd_idx[0] = arg;
+        } else {
+          dense_step_r1<TRAIN>(a[0], L, w, lane, ctx_s, v[0], fd_idx[0]);
+        }
       } else if (live) {
         dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
       } else {
@@ -370,7 +393,12 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
   __syncthreads();
 
   switch (desc.band_k) {
-    case 0: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -1>(p, desc, ch, a_s, ctx_s); break;
+    case 0:
+      if (R == 1 && L == 21)
+        run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, (R == 1 ? -21 : -1)>(p, desc, ch, a_s, ctx_s);
+      else
+        run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -1>(p, desc, ch, a_s, ctx_s);
+      break;
     case 2: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 2>(p, desc, ch, a_s, ctx_s); break;
     case 3: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 3>(p, desc, ch, a_s, ctx_s); break;
     case 4: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 4>(p, desc, ch, a_s, ctx_s); break;

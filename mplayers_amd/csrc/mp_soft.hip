@@ -36,10 +36,12 @@ __device__ __forceinline__ void fill_table(const float* ctx, int L, int ctx2d, i
   }
 }
 
-template <bool TRAIN, int T>
+// LT > 0: the label count is known at compile time (the segmentation case, 21 labels): the loops
+// over front labels are unrolled and the lane's column of the context table lives in registers.
+template <bool TRAIN, int T, int LT>
 __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
   extern __shared__ float smem[];
-  const int L = p.L, LL = L * L;
+  const int L = LT > 0 ? LT : p.L, LL = L * L;
   float* tab = smem;        // LL floats
   float* tile = smem + LL;  // max(LL, 64 * T) floats: the pixel's block of duals
   const int lane = threadIdx.x;
@@ -72,6 +74,13 @@ __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
   const bool valid = lane < L;
   const int col = valid ? lane : L - 1;  // keeps the table reads of idle lanes in range
   const bool even = (dir & 1) == 0;
+  float tcol[LT > 0 ? LT : 1];  // ctx(cd = lane, fd)
+  if (LT > 0) {
+#pragma unroll
+    for (int fd = 0; fd < LT; ++fd) tcol[fd] = tab[fd * L + col];
+  }
+  const int wstep = even ? L : 1;             // address step of the front label inside the block
+  const int wbase = even ? lane : lane * L;   // address of (cd = lane, fd = 0)
 
   const int last_p = ch.pix0 + (n - 1) * ch.pstep;
   int ld_p = ch.pix0;
@@ -122,20 +131,36 @@ __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
       const float a = fmaf(rho, prev, uf);  // lane = front label
       // pass 1: minimum of the duals of this lane's label; the block goes to LDS
       float mn = inf;
-#pragma unroll 4
-      for (int fd = 0; fd < L; ++fd) {
-        const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
-        mn = fminf(mn, dual);
-        if (TRAIN && valid) tile[even ? fd * L + lane : lane * L + fd] = dual;
-      }
-      // pass 2: softmin weights and the expected dual
       float se = 0.f, sd = 0.f;
+      if constexpr (LT > 0) {
+        float dual[LT];
+#pragma unroll
+        for (int fd = 0; fd < LT; ++fd) {
+          dual[fd] = fmaf(w, tcol[fd], readlane_f(a, fd));
+          mn = fminf(mn, dual[fd]);
+          if (TRAIN && valid) tile[wbase + fd * wstep] = dual[fd];
+        }
+        // pass 2: softmin weights and the expected dual
+#pragma unroll
+        for (int fd = 0; fd < LT; ++fd) {
+          const float e = fast_exp(mn - dual[fd]);
+          se += e;
+          sd = fmaf(e, dual[fd], sd);
+        }
+      } else {
 #pragma unroll 4
-      for (int fd = 0; fd < L; ++fd) {
-        const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
-        const float e = fast_exp(mn - dual);
-        se += e;
-        sd = fmaf(e, dual, sd);
+        for (int fd = 0; fd < L; ++fd) {
+          const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
+          mn = fminf(mn, dual);
+          if (TRAIN && valid) tile[wbase + fd * wstep] = dual;
+        }
+#pragma unroll 4
+        for (int fd = 0; fd < L; ++fd) {
+          const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
+          const float e = fast_exp(mn - dual);
+          se += e;
+          sd = fmaf(e, dual, sd);
+        }
       }
       const float soft = sd / se;
       const float nmin = wave_min(valid ? soft : inf);
@@ -176,10 +201,10 @@ struct PixSB {
   float blk[T];
 };
 
-template <int T>
+template <int T, int LT>
 __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
   extern __shared__ float smem[];
-  const int L = p.L, LL = L * L;
+  const int L = LT > 0 ? LT : p.L, LL = L * L;
   const int Lp = L | 1;  // odd row stride of the transposed gradient block: conflict-free reads
   constexpr int kTile = kWave * T;
   float* tab = smem;            // LL
@@ -218,6 +243,14 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
   const bool even = (dir & 1) == 0;
   const int dstep = even ? L : 1;             // address step of the front label inside the block
   const int dbase = even ? col : col * L;     // address of (cd = lane, fd = 0)
+  float tcol[LT > 0 ? LT : 1], hreg[LT > 0 ? LT : 1];  // ctx(lane, fd); dcontext partial sums
+  if (LT > 0) {
+#pragma unroll
+    for (int fd = 0; fd < LT; ++fd) {
+      tcol[fd] = tab[fd * L + col];
+      hreg[fd] = 0.f;
+    }
+  }
 
   int ld_t = n - 1;
   int ld_p = ch.pix0 + (n - 1) * ch.pstep;
@@ -272,28 +305,52 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
         for (int k = 0; k < T; ++k) tile[lane + kWave * k] = px.blk[k];
         // softmin statistics of this lane's label, :83-105
         float mn = INFINITY;
+        float se = 0.f, sd = 0.f, de = 0.f;
+        if constexpr (LT > 0) {
+          float dual[LT], ex[LT];
+#pragma unroll
+          for (int fd = 0; fd < LT; ++fd) {
+            dual[fd] = tile[dbase + fd * dstep];
+            mn = fminf(mn, dual[fd]);
+          }
+#pragma unroll
+          for (int fd = 0; fd < LT; ++fd) {
+            ex[fd] = fast_exp(mn - dual[fd]);
+            se += ex[fd];
+            sd = fmaf(ex[fd], dual[fd], sd);
+          }
+          const float inv = 1.f / se;
+          const float soft1 = fmaf(sd, inv, 1.f);
+          const float gs = gv * inv;
+#pragma unroll
+          for (int fd = 0; fd < LT; ++fd) {
+            const float dd = gs * ex[fd] * (soft1 - dual[fd]);  // :110-113
+            de = fmaf(tcol[fd], dd, de);
+            hreg[fd] = fmaf(w, dd, hreg[fd]);
+            if (valid) grad[fd * Lp + lane] = dd;
+          }
+        } else {
 #pragma unroll 4
-        for (int fd = 0; fd < L; ++fd) mn = fminf(mn, tile[dbase + fd * dstep]);
-        float se = 0.f, sd = 0.f;
+          for (int fd = 0; fd < L; ++fd) mn = fminf(mn, tile[dbase + fd * dstep]);
 #pragma unroll 4
-        for (int fd = 0; fd < L; ++fd) {
-          const float dual = tile[dbase + fd * dstep];
-          const float e = fast_exp(mn - dual);
-          se += e;
-          sd = fmaf(e, dual, sd);
-        }
-        const float inv = 1.f / se;
-        const float soft = sd * inv;
-        const float gs = gv * inv;
-        float de = 0.f;
+          for (int fd = 0; fd < L; ++fd) {
+            const float dual = tile[dbase + fd * dstep];
+            const float e = fast_exp(mn - dual);
+            se += e;
+            sd = fmaf(e, dual, sd);
+          }
+          const float inv = 1.f / se;
+          const float soft1 = fmaf(sd, inv, 1.f);
+          const float gs = gv * inv;
 #pragma unroll 4
-        for (int fd = 0; fd < L; ++fd) {
-          const float dual = tile[dbase + fd * dstep];
-          const float dd = gs * fast_exp(mn - dual) * (1.f - dual + soft);  // :110-113
-          de = fmaf(tab[fd * L + col], dd, de);
-          if (valid) {
-            hist[fd * L + lane] = fmaf(w, dd, hist[fd * L + lane]);  // this lane's own entries
-            grad[fd * Lp + lane] = dd;
+          for (int fd = 0; fd < L; ++fd) {
+            const float dual = tile[dbase + fd * dstep];
+            const float dd = gs * fast_exp(mn - dual) * (soft1 - dual);  // :110-113
+            de = fmaf(tab[fd * L + col], dd, de);
+            if (valid) {
+              hist[fd * L + lane] = fmaf(w, dd, hist[fd * L + lane]);  // this lane's own entries
+              grad[fd * Lp + lane] = dd;
+            }
           }
         }
         // dU[q, fd] = sum_cd ddual[cd, fd]: lane fd adds up its row of the transposed block
@@ -316,6 +373,10 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
       sc = scn;
       st_p -= ch.pstep;
     }
+  }
+  if (LT > 0 && valid) {
+#pragma unroll
+    for (int fd = 0; fd < LT; ++fd) hist[fd * L + lane] = hreg[fd];
   }
   __syncthreads();
   // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D), the diagonal
@@ -353,14 +414,21 @@ void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st) {
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (LL + (train ? (LL > kWave * T ? LL : kWave * T) : 0));
   if (!train) {
-    soft_fwd_kernel<false, 0><<<blocks, kWave, lds, st>>>(p);
+    if (p.L == 21)
+      soft_fwd_kernel<false, 0, 21><<<blocks, kWave, lds, st>>>(p);
+    else
+      soft_fwd_kernel<false, 0, 0><<<blocks, kWave, lds, st>>>(p);
+    return;
+  }
+  if (p.L == 21) {
+    soft_fwd_kernel<true, 7, 21><<<blocks, kWave, lds, st>>>(p);
     return;
   }
   switch (T) {
-    case 4: soft_fwd_kernel<true, 4><<<blocks, kWave, lds, st>>>(p); break;
-    case 7: soft_fwd_kernel<true, 7><<<blocks, kWave, lds, st>>>(p); break;
-    case 16: soft_fwd_kernel<true, 16><<<blocks, kWave, lds, st>>>(p); break;
-    default: soft_fwd_kernel<true, 64><<<blocks, kWave, lds, st>>>(p); break;
+    case 4: soft_fwd_kernel<true, 4, 0><<<blocks, kWave, lds, st>>>(p); break;
+    case 7: soft_fwd_kernel<true, 7, 0><<<blocks, kWave, lds, st>>>(p); break;
+    case 16: soft_fwd_kernel<true, 16, 0><<<blocks, kWave, lds, st>>>(p); break;
+    default: soft_fwd_kernel<true, 64, 0><<<blocks, kWave, lds, st>>>(p); break;
   }
 }
 
@@ -370,15 +438,19 @@ void launch_soft_bwd(const BackParams& p, hipStream_t st) {
   const int LL = p.L * p.L;
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (2 * LL + kWave * T + p.L * (p.L | 1));
+  if (p.L == 21) {
+    soft_bwd_kernel<7, 21><<<blocks, kWave, lds, st>>>(p);
+    return;
+  }
   switch (T) {
-    case 4: soft_bwd_kernel<4><<<blocks, kWave, lds, st>>>(p); break;
-    case 7: soft_bwd_kernel<7><<<blocks, kWave, lds, st>>>(p); break;
-    case 16: soft_bwd_kernel<16><<<blocks, kWave, lds, st>>>(p); break;
+    case 4: soft_bwd_kernel<4, 0><<<blocks, kWave, lds, st>>>(p); break;
+    case 7: soft_bwd_kernel<7, 0><<<blocks, kWave, lds, st>>>(p); break;
+    case 16: soft_bwd_kernel<16, 0><<<blocks, kWave, lds, st>>>(p); break;
     default:
       // up to 66 KB of LDS at 64 labels: above the default limit of a workgroup
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&soft_bwd_kernel<64>),
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&soft_bwd_kernel<64, 0>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      soft_bwd_kernel<64><<<blocks, kWave, lds, st>>>(p);
+      soft_bwd_kernel<64, 0><<<blocks, kWave, lds, st>>>(p);
       break;
   }
 }
