@@ -100,6 +100,18 @@ int mpl_trwp_soft_backward(const mpl_shape* shape, float rho, int n_iter, const 
                            float* dunary, float* dcontext, float* dedge_weights, float* dmsg,
                            float* dunary_update, void* stream);
 
+/* Stand-alone softmin of stored blocks: replaces lib_*.TRWP_hard_soft.soft_weighted_message and
+ * soft_weighted_message_back, TRWP.cpp:385-417 -> TRWP_swbp.cu:131-321.  message (n_trees, L, L)
+ * laid out [fd][cd]; message_soft_sum_norm (n_trees, L) = sum_fd softmax_fd(-message) * message,
+ * minus its minimum over cd; message_soft_sum_min_ind (n_trees) uint8: the label of that minimum
+ * (largest on ties).  The backward call fills dmessage (n_trees, L, L). */
+int mpl_soft_weighted_message(int n_trees, int n_disp, const float* message,
+                              float* message_soft_sum_norm, uint8_t* message_soft_sum_min_ind,
+                              void* stream);
+int mpl_soft_weighted_message_back(int n_trees, int n_disp, const float* dmessage_soft_sum_norm,
+                                   const float* message, const uint8_t* message_soft_sum_min_ind,
+                                   float* dmessage, void* stream);
+
 /* Device check of the wavefront primitives the kernels are built on (cross-lane shifts, min/sum
  * reductions, ballots).  out: 8 host ints, out[0] == 1 when every check passed.  Synchronises. */
 int mpl_selftest_wave_ops(int* out_host);

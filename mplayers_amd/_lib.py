@@ -8,7 +8,7 @@ LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hi
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
            "mpl_selftest_wave_ops", "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
            "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_trwp_soft_forward",
-           "mpl_trwp_soft_backward")
+           "mpl_trwp_soft_backward", "mpl_soft_weighted_message", "mpl_soft_weighted_message_back")
 
 KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combine", "other",
                 "fwd_sweep_all", "bwd_sweep_all", "unary_all")
@@ -46,6 +46,8 @@ def load():
   lib.mpl_isgmr_backward.argtypes = [sp, ci, cf, ci] + [vp] * 12
   lib.mpl_trwp_soft_forward.argtypes = [sp, cf, ci] + [vp] * 10
   lib.mpl_trwp_soft_backward.argtypes = [sp, cf, ci] + [vp] * 11
+  lib.mpl_soft_weighted_message.argtypes = [ci, ci, vp, vp, vp, vp]
+  lib.mpl_soft_weighted_message_back.argtypes = [ci, ci, vp, vp, vp, vp, vp]
   lib.mpl_edge_shift.argtypes = [ci, vp, ci, ci, ci, ci, ci, cf, cf, cf, vp, vp, vp]
   lib.mpl_selftest_wave_ops.argtypes = [ctypes.POINTER(ci)]
   lib.mpl_n_chains.argtypes = [ci, ci, ci]

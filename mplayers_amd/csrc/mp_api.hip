@@ -875,4 +875,29 @@ int mpl_trwp_soft_backward(const mpl_shape* s, float rho, int n_iter, const floa
   return launch_ok("trwp_soft_backward");
 }
 
+int mpl_soft_weighted_message(int n_trees, int n_disp, const float* message,
+                              float* message_soft_sum_norm, uint8_t* message_soft_sum_min_ind,
+                              void* stream) {
+  if (n_trees < 0 || n_disp < 1 || n_disp > kMaxL)
+    return fail(MPL_EINVAL, "soft_weighted_message: n_trees >= 0 and 1 <= n_disp <= %d needed", kMaxL);
+  if (!message || !message_soft_sum_norm || !message_soft_sum_min_ind)
+    return fail(MPL_EINVAL, "soft_weighted_message: null tensor pointer");
+  launch_swm_fwd(message, n_trees, n_disp, message_soft_sum_norm, message_soft_sum_min_ind,
+                 (hipStream_t)stream);
+  return launch_ok("soft_weighted_message");
+}
+
+int mpl_soft_weighted_message_back(int n_trees, int n_disp, const float* dmessage_soft_sum_norm,
+                                   const float* message, const uint8_t* message_soft_sum_min_ind,
+                                   float* dmessage, void* stream) {
+  if (n_trees < 0 || n_disp < 1 || n_disp > kMaxL)
+    return fail(MPL_EINVAL, "soft_weighted_message_back: n_trees >= 0 and 1 <= n_disp <= %d needed",
+                kMaxL);
+  if (!dmessage_soft_sum_norm || !message || !message_soft_sum_min_ind || !dmessage)
+    return fail(MPL_EINVAL, "soft_weighted_message_back: null tensor pointer");
+  launch_swm_bwd(dmessage_soft_sum_norm, message, message_soft_sum_min_ind, n_trees, n_disp,
+                 dmessage, (hipStream_t)stream);
+  return launch_ok("soft_weighted_message_back");
+}
+
 }  // extern "C"

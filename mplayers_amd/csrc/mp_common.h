@@ -395,6 +395,10 @@ void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 // soft-weighted TRWP (mp_soft.hip): one direction per launch, L <= 64
 void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st);
 void launch_soft_bwd(const BackParams& p, hipStream_t st);
+void launch_swm_fwd(const float* msg, int n_trees, int L, float* out, uint8_t* min_ind,
+                    hipStream_t st);
+void launch_swm_bwd(const float* dout, const float* msg, const uint8_t* min_ind, int n_trees, int L,
+                    float* dmsg, hipStream_t st);
 
 inline size_t fwd_lds_bytes(int L, int ctx2d) {
   return sizeof(float) * (kMaxL + ((ctx2d || L <= kWave) ? L * L : L));

@@ -400,6 +400,96 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
   }
 }
 
+// Stand-alone softmin of stored blocks (SoftWeightedMessageKernel / ...BackKernel,
+// TRWP_hard_soft/TRWP_swbp.cu:131-254): message (n_trees, L, L) laid out [fd][cd];
+//   out[tree, cd] = sum_fd prob * message - min_cd(...),  prob = softmax_fd(-message[:, cd])
+// One wavefront per tree, lane i owns labels i, i + 64, ... (consecutive lanes read consecutive
+// floats of a row).
+constexpr int kSwmR = kMaxL / kWave;
+
+__device__ __forceinline__ void swm_stats(const float* __restrict__ blk, int L, int lane,
+                                          float (&mn)[kSwmR], float (&inv)[kSwmR],
+                                          float (&soft)[kSwmR]) {
+#pragma unroll
+  for (int j = 0; j < kSwmR; ++j) {
+    const int cd = lane + kWave * j;
+    mn[j] = INFINITY;
+    inv[j] = 0.f;
+    soft[j] = 0.f;
+    if (cd < L) {
+      for (int fd = 0; fd < L; ++fd) mn[j] = fminf(mn[j], blk[fd * L + cd]);
+      float se = 0.f, sd = 0.f;
+      for (int fd = 0; fd < L; ++fd) {
+        const float v = blk[fd * L + cd];
+        const float e = expf(-(v - mn[j]));
+        se += e;
+        sd = fmaf(e, v, sd);
+      }
+      inv[j] = 1.f / se;
+      soft[j] = sd * inv[j];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(kWave) swm_fwd_kernel(const float* __restrict__ msg, int n_trees,
+                                                        int L, float* __restrict__ out,
+                                                        uint8_t* __restrict__ min_ind) {
+  const int lane = threadIdx.x;
+  for (int tree = blockIdx.x; tree < n_trees; tree += gridDim.x) {
+    float mn[kSwmR], inv[kSwmR], soft[kSwmR];
+    swm_stats(msg + (int64_t)tree * L * L, L, lane, mn, inv, soft);
+    float lo = INFINITY;
+#pragma unroll
+    for (int j = 0; j < kSwmR; ++j) lo = fminf(lo, (lane + kWave * j < L) ? soft[j] : INFINITY);
+    const float nmin = wave_min(lo);
+    int arg = -1;  // largest label that attains the minimum (TRWP_swbp.cu:95-101)
+#pragma unroll
+    for (int j = 0; j < kSwmR; ++j) {
+      const int cd = lane + kWave * j;
+      if (cd < L) {
+        out[(int64_t)tree * L + cd] = soft[j] - nmin;
+        if (soft[j] == nmin) arg = cd;
+      }
+    }
+    const float best = -wave_min(-(float)arg);
+    if (lane == 0) min_ind[tree] = (uint8_t)(int)best;
+  }
+}
+
+__global__ void __launch_bounds__(kWave) swm_bwd_kernel(const float* __restrict__ dout,
+                                                        const float* __restrict__ msg,
+                                                        const uint8_t* __restrict__ min_ind,
+                                                        int n_trees, int L,
+                                                        float* __restrict__ dmsg) {
+  const int lane = threadIdx.x;
+  for (int tree = blockIdx.x; tree < n_trees; tree += gridDim.x) {
+    const float* blk = msg + (int64_t)tree * L * L;
+    float mn[kSwmR], inv[kSwmR], soft[kSwmR], g[kSwmR];
+    swm_stats(blk, L, lane, mn, inv, soft);
+    float part = 0.f;
+#pragma unroll
+    for (int j = 0; j < kSwmR; ++j) {
+      const int cd = lane + kWave * j;
+      g[j] = cd < L ? dout[(int64_t)tree * L + cd] : 0.f;
+      part += g[j];
+    }
+    const float tot = wave_sum(part);
+    const int ind = min_ind[tree];
+#pragma unroll
+    for (int j = 0; j < kSwmR; ++j) {
+      const int cd = lane + kWave * j;
+      if (cd == ind) g[j] -= tot;
+      if (cd < L) {
+        for (int fd = 0; fd < L; ++fd) {
+          const float v = blk[fd * L + cd];
+          const float prob = expf(-(v - mn[j])) * inv[j];
+          dmsg[(int64_t)tree * L * L + fd * L + cd] = g[j] * prob * (1.f - v + soft[j]);
+        }
+      }
+    }
+  }
+}
+
 int tile_bucket(int L) {
   const int need = (L * L + kWave - 1) / kWave;
   return need <= 4 ? 4 : (need <= 7 ? 7 : (need <= 16 ? 16 : 64));
@@ -453,6 +543,19 @@ void launch_soft_bwd(const BackParams& p, hipStream_t st) {
       soft_bwd_kernel<64, 0><<<blocks, kWave, lds, st>>>(p);
       break;
   }
+}
+
+void launch_swm_fwd(const float* msg, int n_trees, int L, float* out, uint8_t* min_ind,
+                    hipStream_t st) {
+  if (n_trees <= 0) return;
+  swm_fwd_kernel<<<n_trees < 65536 ? n_trees : 65536, kWave, 0, st>>>(msg, n_trees, L, out, min_ind);
+}
+
+void launch_swm_bwd(const float* dout, const float* msg, const uint8_t* min_ind, int n_trees, int L,
+                    float* dmsg, hipStream_t st) {
+  if (n_trees <= 0) return;
+  swm_bwd_kernel<<<n_trees < 65536 ? n_trees : 65536, kWave, 0, st>>>(dout, msg, min_ind, n_trees, L,
+                                                                     dmsg);
 }
 
 }  // namespace mpl

@@ -168,8 +168,8 @@ class ISGMR(object):
 class TRWP_hard_soft(object):
   """Drop-in for the reference's `lib_stereo.TRWP_hard_soft` / `lib_seg.TRWP_hard_soft` extension
   modules (MPLayers/TRWP_hard_soft/TRWP.cpp:428-445): the hard operators under the same names as
-  in `TRWP`, plus `forward_soft` / `backward_soft`.  `soft_weighted_message(_back)`, the stand-alone
-  softmin of a stored tensor, is not part of this build and raises."""
+  in `TRWP`, plus `forward_soft` / `backward_soft` and the stand-alone softmin of stored blocks,
+  `soft_weighted_message` / `soft_weighted_message_back`."""
 
   forward = TRWP.forward
   backward = TRWP.backward
@@ -230,9 +230,35 @@ class TRWP_hard_soft(object):
     _lib.check(rc, "TRWP_hard_soft.backward_soft")
 
   @staticmethod
-  def soft_weighted_message(*args):
-    raise RuntimeError("soft_weighted_message is not part of this build")
+  def soft_weighted_message(message, message_soft_sum_norm, message_soft_sum_min_ind):
+    """message (n_trees, L, L) [fd][cd] -> normalised soft message sums (n_trees, L) and the label
+    of their minimum (n_trees) uint8; TRWP.cpp:385-400."""
+    lib = _lib.load()
+    if message.dim() != 3 or message.size(1) != message.size(2):
+      raise RuntimeError("message must be (n_trees, n_disp, n_disp)")
+    n_trees, L, _ = message.shape
+    _check("message", message, torch.float32)
+    _check("message_soft_sum_norm", message_soft_sum_norm, torch.float32, n_trees * L)
+    _check("message_soft_sum_min_ind", message_soft_sum_min_ind, torch.uint8, n_trees)
+    with torch.cuda.device(message.device):
+      rc = lib.mpl_soft_weighted_message(n_trees, L, _ptr(message), _ptr(message_soft_sum_norm),
+                                         _ptr(message_soft_sum_min_ind), _Op._stream(message))
+    _lib.check(rc, "TRWP_hard_soft.soft_weighted_message")
 
   @staticmethod
-  def soft_weighted_message_back(*args):
-    raise RuntimeError("soft_weighted_message_back is not part of this build")
+  def soft_weighted_message_back(dmessage_soft_sum_norm, message, message_soft_sum_min_ind,
+                                 dmessage):
+    """Gradient of soft_weighted_message with respect to message; TRWP.cpp:402-417."""
+    lib = _lib.load()
+    if message.dim() != 3 or message.size(1) != message.size(2):
+      raise RuntimeError("message must be (n_trees, n_disp, n_disp)")
+    n_trees, L, _ = message.shape
+    _check("dmessage_soft_sum_norm", dmessage_soft_sum_norm, torch.float32, n_trees * L)
+    _check("message", message, torch.float32)
+    _check("message_soft_sum_min_ind", message_soft_sum_min_ind, torch.uint8, n_trees)
+    _check("dmessage", dmessage, torch.float32, n_trees * L * L)
+    with torch.cuda.device(message.device):
+      rc = lib.mpl_soft_weighted_message_back(n_trees, L, _ptr(dmessage_soft_sum_norm),
+                                              _ptr(message), _ptr(message_soft_sum_min_ind),
+                                              _ptr(dmessage), _Op._stream(message))
+    _lib.check(rc, "TRWP_hard_soft.soft_weighted_message_back")

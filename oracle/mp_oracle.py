@@ -225,3 +225,28 @@ def backward_soft(context, edge_weights, dcost_final, msg_edge_label, msg_norm_i
      _ptr(dcost_final), _ptr(msg_edge_label), _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
      _ptr(dedge))
   return dunary, dcontext, dedge
+
+
+def soft_weighted_message(message):
+  """Restated SoftWeightedMessageKernel (TRWP_hard_soft/TRWP_swbp.cu:131-200): message
+  (n_trees, L, L) laid out [fd][cd].  Returns (message_soft_sum_norm (n_trees, L),
+  message_soft_sum_min_ind (n_trees,) uint8, largest label on ties)."""
+  m = np.asarray(message)
+  e = np.exp(-(m - m.min(axis=1, keepdims=True)))       # :170-172
+  prob = e / e.sum(axis=1, keepdims=True)               # :175
+  soft = (m * prob).sum(axis=1)                         # :176-180
+  L = m.shape[1]
+  ind = (L - 1 - np.argmin(soft[:, ::-1], axis=1)).astype(np.uint8)  # :95-101
+  return soft - soft.min(axis=1, keepdims=True), ind
+
+
+def soft_weighted_message_back(dnorm, message, min_ind):
+  """Restated SoftWeightedMessageBackKernel (TRWP_swbp.cu:203-254): gradient w.r.t. message."""
+  m = np.asarray(message)
+  g = np.array(dnorm, dtype=m.dtype, copy=True)
+  rows = np.arange(m.shape[0])
+  g[rows, min_ind] -= g.sum(axis=1)                     # :224-231
+  e = np.exp(-(m - m.min(axis=1, keepdims=True)))
+  prob = e / e.sum(axis=1, keepdims=True)
+  soft = (m * prob).sum(axis=1, keepdims=True)
+  return g[:, None, :] * prob * (1 - m + soft)          # :250

@@ -184,5 +184,24 @@ def test_soft_refuses_more_than_64_labels(gpu):
         0.5, 1, u, torch.zeros(L, device="cuda"), torch.ones(4, 1, 1, 2, 2, device="cuda"),
         torch.zeros(4, 1, 1, 2, 2, L, device="cuda"), torch.empty(0), torch.empty(0, dtype=torch.uint8),
         torch.zeros_like(u), torch.zeros_like(u), torch.empty(0, dtype=torch.uint8))
-  with pytest.raises(RuntimeError):
-    lib_stereo.TRWP_hard_soft.soft_weighted_message()
+
+
+@pytest.mark.parametrize("T,L", [(5, 6), (3, 21), (2, 64), (2, 100), (1, 255)])
+def test_soft_weighted_message(gpu, oracle, T, L):
+  import torch
+  from mplayers_amd import lib_seg
+  rng = np.random.default_rng(L)
+  m = (rng.random((T, L, L)) * 4).astype(np.float32)
+  R = rng.standard_normal((T, L)).astype(np.float32)
+  ref_norm, ref_ind = oracle.soft_weighted_message(m.astype(np.float64))
+  ref_dm = oracle.soft_weighted_message_back(R.astype(np.float64), m.astype(np.float64), ref_ind)
+  msg = t(m)
+  norm = msg.new_zeros(T, L)
+  ind = torch.zeros(T, dtype=torch.uint8, device="cuda")
+  lib_seg.TRWP_hard_soft.soft_weighted_message(msg, norm, ind)
+  dm = torch.zeros_like(msg)
+  lib_seg.TRWP_hard_soft.soft_weighted_message_back(t(R), msg, t(ref_ind), dm)
+  torch.cuda.synchronize()
+  assert np.abs(norm.cpu().numpy() - ref_norm).max() <= 1e-5 * max(1.0, np.abs(m).max())
+  np.testing.assert_array_equal(ind.cpu().numpy(), ref_ind)
+  assert np.abs(dm.cpu().numpy() - ref_dm).max() <= 1e-4 * max(1.0, np.abs(ref_dm).max())

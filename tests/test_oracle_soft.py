@@ -151,3 +151,33 @@ def test_backward_matches_finite_differences(oracle, n_dir, ctx2d):
   du1, _, _ = oracle.backward_soft(ctx, ew, ones, fwd["msg_edge_label"], fwd["msg_norm_index"], rho,
                                    ctx2d=ctx2d)
   np.testing.assert_allclose(du1.sum(), ones.sum(), rtol=1e-9)
+
+
+def test_soft_weighted_message_oracle():
+  """Stand-alone softmin of stored blocks: forward against the logsumexp derivative, backward
+  against central finite differences."""
+  rng = np.random.default_rng(5)
+  T, L = 4, 6
+  m = rng.random((T, L, L)) * 3
+  norm, ind = soft_oracle().soft_weighted_message(m)
+  soft = soft_expect(np.swapaxes(m, 1, 2))                 # [cd][fd] rows
+  np.testing.assert_allclose(norm, soft - soft.min(axis=1, keepdims=True), atol=2e-9)
+  np.testing.assert_array_equal(ind, soft.argmin(axis=1))
+  # ties pick the largest label
+  m2 = np.tile(m[:1, :, :1], (1, 1, L))
+  assert soft_oracle().soft_weighted_message(m2)[1][0] == L - 1
+  R = rng.standard_normal((T, L))
+  dm = soft_oracle().soft_weighted_message_back(R, m, ind)
+  h = 1e-6
+  for _ in range(20):
+    idx = tuple(rng.integers(0, s) for s in m.shape)
+    p, q = m.copy(), m.copy()
+    p[idx] += h
+    q[idx] -= h
+    fd = ((soft_oracle().soft_weighted_message(p)[0] - soft_oracle().soft_weighted_message(q)[0]) * R).sum() / (2 * h)
+    assert abs(fd - dm[idx]) < 1e-6
+
+
+def soft_oracle():
+  from oracle import mp_oracle
+  return mp_oracle
