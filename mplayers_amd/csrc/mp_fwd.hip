@@ -129,7 +129,19 @@ __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, c
 #pragma unroll
     for (int k = 1; k < KT; ++k) tap(k, c_reg[k]);
   } else {
-    for (int k = 1; k < K; ++k) tap(k, ctx_s[k]);
+    // R taps per trip: the R one-label rotations of up[] / dn[] then cancel, so the loop carries
+    // no register moves, and the R coefficients are fetched from LDS together
+    int k = 1;
+    for (; k + R <= K; k += R) {
+      float cc[R];
+#pragma unroll
+      for (int u = 0; u < R; ++u) cc[u] = ctx_s[k + u];
+#pragma unroll
+      for (int u = 0; u < R; ++u) tap(k + u, cc[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < R - 1; ++u)
+      if (k + u < K) tap(k + u, ctx_s[k + u]);
   }
   const float far = fmaf(w, cmax, amin);
 #pragma unroll

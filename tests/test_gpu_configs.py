@@ -253,3 +253,58 @@ def test_large_config_properties_at_full_size(gpu, mode):
   # edge-weight gradients exist only where a pixel has a front neighbour
   assert float(dedge[0, 0, 0, :, 0].abs().max()) == 0.0
   assert float(dedge[0, 0, 0, :, 1:].abs().max()) > 0.0
+
+
+@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
+def test_full_size_rows_match_oracle(gpu, oracle, mode):
+  """With only the two horizontal directions the rows of an image do not interact, so the oracle
+  can check a few rows of a full-size (1500 x 2000 x 192) run exactly as it checks small images:
+  first rows, a middle row and the last rows, whose byte offsets lie beyond 2^31."""
+  import torch
+  from mplayers_amd import lib_stereo, synthetic
+  cfg = synthetic.make_config("C5", seed=0, mode=mode)
+  B, H, W, L = cfg["B"], cfg["H"], cfg["W"], cfg["L"]
+  n_dir, n_iter, rho = 2, 2, cfg["rho"]
+  dev = "cuda:0"
+  unary = cfg["unary"].to(dev)
+  ctx = cfg["context"].to(dev)
+  ew = cfg["edge_weights"][:n_dir].contiguous().to(dev)
+  dcost = synthetic.upstream_grad(cfg).to(dev)
+  msg = torch.zeros(n_dir, B, 1, H, W, L, device=dev)
+  cost = torch.zeros(B, 1, H, W, L, device=dev)
+  scratch = torch.zeros(B, 1, H, W, L, device=dev)
+  imin = torch.zeros(n_iter, n_dir, B, 1, H, W, L, dtype=torch.uint8, device=dev)
+  inorm = torch.zeros(n_iter, n_dir, B, 1, H, W, dtype=torch.uint8, device=dev)
+  empty = torch.empty(0, dtype=torch.uint8)
+  dunary = torch.zeros_like(cost)
+  dedge = torch.zeros(n_dir, B, 1, H, W, device=dev)
+  dctx = torch.zeros(L, device=dev)
+  dmsg = torch.empty_like(msg)
+  print("full-size rows", mode, flush=True)
+  if mode == "TRWP":
+    lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch, empty)
+    lib_stereo.TRWP.backward(rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, dmsg, scratch)
+  else:
+    msg_tmp = torch.zeros_like(msg)
+    lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch,
+                             msg_tmp, empty)
+    lib_stereo.ISGMR.backward(0, rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, scratch,
+                              scratch, dmsg)
+  torch.cuda.synchronize()
+  rows = [0, 1, H // 2, H - 2, H - 1]
+  sub = lambda t, ax: t.index_select(ax, torch.tensor(rows, device=t.device)).cpu().numpy()
+  un, en, dn = sub(unary, 2), sub(ew, 3), sub(dcost, 2)
+  ref = oracle.forward(mode, un, ctx.cpu().numpy(), en, n_dir, n_iter, rho, want_gaps=True)
+  belief = ref["cost_final"]
+  tol = 1e-5 * max(1.0, float(np.abs(belief).max()))
+  gpu.assert_values_close(sub(msg, 3), ref["msg"], what="msg rows", belief=belief)
+  gpu.assert_values_close(sub(cost, 2), ref["cost_final"], what="cost rows")
+  gpu.assert_indices_match_off_ties(sub(imin, 4), ref["msg_min_index"], ref["gap_min"], 4 * tol,
+                                    "min index rows")
+  gpu.assert_indices_match_off_ties(sub(inorm, 4), ref["msg_norm_index"], ref["gap_norm"], 4 * tol,
+                                    "norm index rows")
+  # backward on the GPU's own indices of those rows
+  du, _, de = oracle.backward(mode, ctx.cpu().numpy().astype(np.float64), en.astype(np.float64),
+                              dn.astype(np.float64), sub(imin, 4), sub(inorm, 4), rho)
+  assert np.abs(sub(dunary, 2) - du).max() <= 1e-4 * max(1.0, np.abs(du).max())
+  assert np.abs(sub(dedge, 3) - de).max() <= 1e-4 * max(1.0, np.abs(de).max())
