@@ -308,3 +308,86 @@ def test_full_size_rows_match_oracle(gpu, oracle, mode):
                               dn.astype(np.float64), sub(imin, 4), sub(inorm, 4), rho)
   assert np.abs(sub(dunary, 2) - du).max() <= 1e-4 * max(1.0, np.abs(du).max())
   assert np.abs(sub(dedge, 3) - de).max() <= 1e-4 * max(1.0, np.abs(de).max())
+
+
+@pytest.mark.parametrize("mode,pair", [("TRWP", 2), ("ISGMR", 2), ("TRWP", 4), ("ISGMR", 6)])
+def test_full_size_chains_match_oracle(gpu, oracle, mode, pair):
+  """Zero edge weights make a direction's messages vanish, so with every direction but one
+  opposite pair switched off the chains of that pair do not interact: single columns (pair 2/3)
+  or diagonals (4/5, 6/7) of a full-size run are then two-direction problems on a 1 x n image,
+  which the oracle checks exactly, forward and backward."""
+  import torch
+  from mplayers_amd import lib_stereo, synthetic
+  cfg = synthetic.make_config("C5", seed=0, mode=mode)
+  B, H, W, L = cfg["B"], cfg["H"], cfg["W"], cfg["L"]
+  n_dir = 4 if pair < 4 else 8
+  n_iter, rho = 2, cfg["rho"]
+  dev = "cuda:0"
+  unary = cfg["unary"].to(dev)
+  ctx = cfg["context"].to(dev)
+  ew = cfg["edge_weights"][:n_dir].clone()
+  for d in range(n_dir):
+    if d not in (pair, pair + 1):
+      ew[d] = 0
+  ew = ew.contiguous().to(dev)
+  dcost = synthetic.upstream_grad(cfg).to(dev)
+  msg = torch.zeros(n_dir, B, 1, H, W, L, device=dev)
+  cost = torch.zeros(B, 1, H, W, L, device=dev)
+  scratch = torch.zeros(B, 1, H, W, L, device=dev)
+  imin = torch.zeros(n_iter, n_dir, B, 1, H, W, L, dtype=torch.uint8, device=dev)
+  inorm = torch.zeros(n_iter, n_dir, B, 1, H, W, dtype=torch.uint8, device=dev)
+  empty = torch.empty(0, dtype=torch.uint8)
+  dunary = torch.zeros_like(cost)
+  dedge = torch.zeros(n_dir, B, 1, H, W, device=dev)
+  dctx = torch.zeros(L, device=dev)
+  dmsg = torch.empty_like(msg)
+  print("full-size chains", mode, pair, flush=True)
+  if mode == "TRWP":
+    lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch, empty)
+    lib_stereo.TRWP.backward(rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, dmsg, scratch)
+  else:
+    msg_tmp = torch.zeros_like(msg)
+    lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch,
+                             msg_tmp, empty)
+    lib_stereo.ISGMR.backward(0, rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, scratch,
+                              scratch, dmsg)
+    del msg_tmp
+  torch.cuda.synchronize()
+  # messages of the switched-off directions vanish
+  for d in range(n_dir):
+    if d not in (pair, pair + 1):
+      assert float(msg[d].abs().max()) == 0.0
+  hs, ws = oracle.dir_step(pair)
+  if pair == 2:
+    starts = [(0, 0), (0, 1), (0, W // 2), (0, W - 1)]
+  elif pair == 4:   # down-right: chains start on the top row and on the left column
+    starts = [(0, 0), (0, 700), (0, W - 3), (H - 5, 0), (600, 0)]
+  else:             # pair 6, down-left: top row and right column
+    starts = [(0, W - 1), (0, 900), (0, 2), (H - 4, W - 1), (400, W - 1)]
+  ctx_np = ctx.cpu().numpy()
+  for (h0, w0) in starts:
+    n = 1 + min((H - 1 - h0) // hs if hs else 10**9,
+                ((W - 1 - w0) // ws if ws > 0 else (w0 // -ws if ws < 0 else 10**9)))
+    hh = torch.arange(n, device=dev) * hs + h0
+    ww = torch.arange(n, device=dev) * ws + w0
+    pick = lambda t: t[..., hh, ww, :] if t.shape[-1] == L else t[..., hh, ww]
+    un = unary[:, :, hh, ww, :].cpu().numpy()[:, :, None]                 # (1, 1, 1, n, L)
+    en = ew[[pair, pair + 1]][:, :, :, hh, ww].cpu().numpy()[:, :, :, None]  # (2, 1, 1, 1, n)
+    dn = dcost[:, :, hh, ww, :].cpu().numpy()[:, :, None]
+    ref = oracle.forward(mode, un, ctx_np, en, 2, n_iter, rho, want_gaps=True)
+    belief = ref["cost_final"]
+    tol = 1e-5 * max(1.0, float(np.abs(belief).max()))
+    got_msg = msg[[pair, pair + 1]][:, :, :, hh, ww, :].cpu().numpy()[:, :, :, None]
+    gpu.assert_values_close(got_msg, ref["msg"], what="chain msg", belief=belief)
+    gpu.assert_values_close(cost[:, :, hh, ww, :].cpu().numpy()[:, :, None], ref["cost_final"],
+                            what="chain cost")
+    gi = imin[:, [pair, pair + 1]][:, :, :, :, hh, ww, :].cpu().numpy()[:, :, :, :, None]
+    gn = inorm[:, [pair, pair + 1]][:, :, :, :, hh, ww].cpu().numpy()[:, :, :, :, None]
+    gpu.assert_indices_match_off_ties(gi, ref["msg_min_index"], ref["gap_min"], 4 * tol, "min idx")
+    gpu.assert_indices_match_off_ties(gn, ref["msg_norm_index"], ref["gap_norm"], 4 * tol, "norm idx")
+    du, _, de = oracle.backward(mode, ctx_np.astype(np.float64), en.astype(np.float64),
+                                dn.astype(np.float64), gi, gn, rho)
+    got_du = dunary[:, :, hh, ww, :].cpu().numpy()[:, :, None]
+    got_de = dedge[[pair, pair + 1]][:, :, :, hh, ww].cpu().numpy()[:, :, :, None]
+    assert np.abs(got_du - du).max() <= 1e-4 * max(1.0, np.abs(du).max()), (h0, w0)
+    assert np.abs(got_de - de).max() <= 1e-4 * max(1.0, np.abs(de).max()), (h0, w0)
