@@ -27,6 +27,20 @@ namespace {
 //   * indices within kNear labels of their own label are moved with DPP label shifts,
 //   * only what is left goes through LDS atomics.
 constexpr int kNear = 3;
+constexpr int kSmallL = 16;  // beyond that the register/LDS scatter below is faster (measured at 21)
+
+// sum over the first LS lanes c of g[c] where target[c] == lane
+template <int LS>
+__device__ __forceinline__ float gather_by_target(float g, int target, int lane) {
+  float acc = 0.f;
+#pragma unroll
+  for (int c = 0; c < LS; ++c) {
+    const float gc = readlane_f(g, c);
+    const int fc = __builtin_amdgcn_readlane(target, c);
+    acc += (lane == fc) ? gc : 0.f;
+  }
+  return acc;
+}
 
 template <int R>
 struct PixB {
@@ -36,7 +50,8 @@ struct PixB {
   float w, de;
 };
 
-template <int R, bool VEC, bool MASK, bool JACOBI>
+// SMALL: one label per lane and at most kSmallL labels (see small_l below)
+template <int R, bool VEC, bool MASK, bool JACOBI, bool SMALL>
 __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   extern __shared__ float smem[];
   const int L = p.L;
@@ -46,6 +61,10 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   float* g1_s = g0_s + kMaxL;      // same for class 1
   float* ctx_s = g1_s + kMaxL;     // context table
   float* hist_s = ctx_s + n_ctx;   // dcontext accumulator of the slow path (and of 2-D contexts)
+  // one label per lane and at most kSmallL labels: the scatter is a loop over source labels and
+  // dcontext is accumulated per (cd, fd) pair, each lane owning the row of its label
+  constexpr bool small_l = SMALL;
+  float* pair_s = hist_s + n_ctx;  // L * L floats when small_l
   const int lane = threadIdx.x;
   const int64_t P = (int64_t)p.B * p.H * p.W;
   const int64_t N = P * L;
@@ -58,6 +77,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     hist_s[i] = 0.f;
   }
   for (int i = lane; i < 3 * kMaxL; i += kWave) sc_s[i] = 0.f;  // sc_s, g0_s, g1_s
+  if (small_l)
+    for (int i = lane; i < L * L; i += kWave) pair_s[i] = 0.f;
   __syncthreads();
 
   const int64_t HW = (int64_t)p.H * p.W;
@@ -156,6 +177,24 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           part += gv[j];
         }
         const float tot = wave_sum(part);  // MsgNormNaiveBack, commonCUDA.cuh:131-145
+        if constexpr (R == 1 && SMALL) {
+          const int cd = lane, fd = px.fd[0];
+          float g = gv[0];
+          if (cd == nidx) g -= tot;
+          if (!valid[0]) g = 0.f;
+          // this lane's own pair: dedge and dcontext (TRWP_backward.cu:109-112)
+          const int ao = fd > cd ? fd - cd : cd - fd;
+          const int ci = !valid[0] ? 0 : (p.ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
+          const float de = ctx_s[ci] * g;
+          if (valid[0] && cd != fd) pair_s[cd * L + fd] = fmaf(w, g, pair_s[cd * L + fd]);
+          // dU[q, f] = sum of g[c] over the labels c that point at f: one source label per trip
+          // (fully unrolled for the next size bucket: lanes past L carry g = 0)
+          if (L <= 8)
+            scn[0] = gather_by_target<8>(g, fd, lane);
+          else
+            scn[0] = gather_by_target<16>(g, fd, lane);
+          det = wave_sum(de);
+        } else {
         // the two popular targets: where the first and the last label point
         const int f0 = __builtin_amdgcn_readlane(px.fd[0], 0);
         int f1 = 0;
@@ -274,6 +313,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
             if (valid[j]) scn[j] += atomicExch(&sc_s[lab0 + j], 0.f);  // read and clear
         }
         det = wave_sum(de);
+        }
       }
       // pixel-local part of UpdateUnaryKernelBack with dU[pix] = sc; nothing is stored for t < 0
       const unsigned sp = (unsigned)uniform_i(st_p);
@@ -302,6 +342,26 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     }
   }
   __syncthreads();
+  if (small_l) {
+    // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D)
+    if (!p.ctx2d) {
+      if (lane >= 1 && lane < L) {
+        float acc = 0.f;
+        for (int c = 0; c < L; ++c) {
+          if (c + lane < L) acc += pair_s[c * L + c + lane];
+          if (c - lane >= 0) acc += pair_s[c * L + c - lane];
+        }
+        if (acc != 0.f) atomicAdd(&p.dctx[lane], acc);
+      }
+    } else {
+      for (int i = lane; i < L * L; i += kWave) {
+        const int c = i / L, f = i - c * L;
+        if (c >= f) continue;  // the (f, c) entry is added here; the diagonal never accumulates
+        const float v = pair_s[i] + pair_s[f * L + c];
+        if (v != 0.f) atomicAdd(&p.dctx[i], v);
+      }
+    }
+  }
   for (int i = lane; i < n_ctx; i += kWave) {
     float v = hist_s[i];
     if (v != 0.f) atomicAdd(&p.dctx[i], v);
@@ -321,12 +381,21 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 template <int R, bool VEC, bool MASK>
 void launch_vm(const BackParams& p, bool jacobi, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
-  const size_t lds =
-      sizeof(float) * (3 * kMaxL + 2 * (p.ctx2d ? p.L * p.L : p.L));
+  const size_t lds = sizeof(float) * (3 * kMaxL + 2 * (p.ctx2d ? p.L * p.L : p.L) +
+                                      ((R == 1 && p.L <= kSmallL) ? p.L * p.L : 0));
+  if constexpr (R == 1) {
+    if (p.L <= kSmallL) {
+      if (jacobi)
+        sweep_bwd_kernel<R, VEC, MASK, true, true><<<blocks, kWave, lds, st>>>(p);
+      else
+        sweep_bwd_kernel<R, VEC, MASK, false, true><<<blocks, kWave, lds, st>>>(p);
+      return;
+    }
+  }
   if (jacobi)
-    sweep_bwd_kernel<R, VEC, MASK, true><<<blocks, kWave, lds, st>>>(p);
+    sweep_bwd_kernel<R, VEC, MASK, true, false><<<blocks, kWave, lds, st>>>(p);
   else
-    sweep_bwd_kernel<R, VEC, MASK, false><<<blocks, kWave, lds, st>>>(p);
+    sweep_bwd_kernel<R, VEC, MASK, false, false><<<blocks, kWave, lds, st>>>(p);
 }
 
 }  // namespace
