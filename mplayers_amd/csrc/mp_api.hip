@@ -132,7 +132,8 @@ __global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ u
 template <int V, int ND>
 __global__ void __launch_bounds__(256) isgmr_unary_kernel(const float* __restrict__ unary,
                                                           const float* msg, float* out,
-                                                          int n_dir_rt, int64_t N, float rho) {
+                                                          int n_dir_rt, int64_t N, float rho,
+                                                          int pair_share) {
   constexpr int KD = ND > 0 ? ND : kMaxDirs;
   const int n_dir = ND > 0 ? ND : n_dir_rt;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
@@ -156,7 +157,9 @@ __global__ void __launch_bounds__(256) isgmr_unary_kernel(const float* __restric
       }
 #pragma unroll
     for (int k = 0; k < KD; ++k) {
-      if (k < n_dir) {
+      // pair_share (rho == 1): U_d and U_{d^1} are both S - m_d - m_{d^1}; one plane per pair is
+      // stored (they differ by the order of the two subtractions, at most 2 ulp of S)
+      if (k < n_dir && !(pair_share && (k & 1))) {
         Pack<V> u;
 #pragma unroll
         for (int j = 0; j < V; ++j) u.v[j] = fmaf(S.v[j] - m[k].v[j], rho, -m[k ^ 1].v[j]);
@@ -642,6 +645,7 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   p.belief = unary_update;
   p.belief_out = nullptr;
   fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
+  p.u_pair_share = (rho == 1.f) ? 1 : 0;
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {
     // Jacobi over directions (ISGMR_forward.cu:506-622): every direction reads the old messages,
@@ -656,7 +660,8 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
     {
       Timed timed(MPL_KERNEL_UNARY_ALL, st);
       const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update);
-      MPL_EW_LAUNCH(isgmr_unary_kernel, v4, s->n_dir, N, st, unary, have, ubuf, s->n_dir, N, rho);
+      MPL_EW_LAUNCH(isgmr_unary_kernel, v4, s->n_dir, N, st, unary, have, ubuf, s->n_dir, N, rho,
+                    p.u_pair_share);
     }
     p.msg_in = ubuf;
     p.msg_out = nxt;

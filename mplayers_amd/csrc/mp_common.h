@@ -353,6 +353,7 @@ struct SweepParams {
   const CtxDesc* desc;             // may be null: dense path
   uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
+  int u_pair_share;                // Jacobi: directions d and d^1 read the U plane of the even one
   float* edge_label;               // soft TRWP: (n_dir_total, P, L, L) duals of this iteration, or null
 };
 

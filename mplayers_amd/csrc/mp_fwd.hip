@@ -176,7 +176,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // plane bases of this batch item and direction; descriptors are formed per access
   // Jacobi: the plane of this direction in msg_in holds U itself (written by the host's
   // element-wise pass before the sweeps), so one plane is read per pixel instead of three
-  const float* __restrict__ bS = (JACOBI ? p.msg_in + (int64_t)dir * N : p.belief) + img_e;
+  const float* __restrict__ bS =
+      (JACOBI ? p.msg_in + (int64_t)(p.u_pair_share ? (dir & ~1) : dir) * N : p.belief) + img_e;
   const float* __restrict__ bMd = p.msg_in + (int64_t)dir * N + img_e;
   const float* __restrict__ bMi = p.msg_in + (int64_t)(dir ^ 1) * N + img_e;
   float* __restrict__ bMo = p.msg_out + (int64_t)dir * N + img_e;
