@@ -73,7 +73,8 @@ int mpl_isgmr_forward(const mpl_shape* shape, int enable_sgm, float rho, int n_i
                       float* msg_update, uint8_t* label_all, void* stream);
 
 /* Replaces lib_*.ISGMR.backward: MPLayers/ISGMR/ISGMR.cpp:344-379 -> ISGMR_backward.cu:290-493.
- * dmsg_update is scratch (n_dir planes, any contents); dmsg and dunary_update are unused. */
+ * dmsg_update and dmsg are scratch (n_dir planes each, any contents); dmsg may be NULL (the pass
+ * then works in place in dmsg_update and moves somewhat more data); dunary_update is unused. */
 int mpl_isgmr_backward(const mpl_shape* shape, int enable_sgm, float rho, int n_iter,
                        const float* context, const float* edge_weights, const float* dcost_final,
                        const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,

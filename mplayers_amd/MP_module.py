@@ -63,7 +63,6 @@ def _backward_buffers(dcost_final, message_index, with_message_tmp):
       dedge_weights=dcost_final.new_zeros(n_dir, batch, cv, h, w))
   if with_message_tmp:
     buf["dmessage_tmp"] = dcost_final.new_empty(n_dir, batch, cv, h, w, n_disp)
-    buf["dmessage"] = dcost_final.new_empty(0)  # ISGMR's backward keeps everything in dmessage_tmp
   if n_disp == 21:
     buf["dlabel_context"] = dcost_final.new_zeros(n_disp, n_disp)
   else:

@@ -251,14 +251,14 @@ __global__ void __launch_bounds__(256) label_kernel(const float* __restrict__ un
 }
 
 // ISGMR: after all directions of an iteration have been scanned back (X_k = dU_k):
-//   dunary += rho * sum_k X_k ;  gu_k = rho * (sum - X_k) - X_{k^1}
+//   dunary += rho * sum_k X_k ;  gu_k = rho * (sum - X_k) - X_{k^1}   (written to G)
 // (UpdateUnaryKernelBack summed over directions + SumMsgKernel, ISGMR_backward.cu:39-60, 482-483)
 template <int V, int ND>
-__global__ void __launch_bounds__(256) isgmr_combine_kernel(float* __restrict__ X, int n_dir_rt,
+__global__ void __launch_bounds__(256) isgmr_combine_kernel(const float* X, float* G, int n_dir_rt,
                                                             int64_t N, float rho,
                                                             const float* __restrict__ dcost,
                                                             float factor, int init_dunary,
-                                                            int write_gu,
+                                                            int write_gu, int pair_share,
                                                             float* __restrict__ dunary) {
   constexpr int KD = ND > 0 ? ND : kMaxDirs;
   const int n_dir = ND > 0 ? ND : n_dir_rt;
@@ -289,11 +289,13 @@ __global__ void __launch_bounds__(256) isgmr_combine_kernel(float* __restrict__ 
     if (write_gu) {
 #pragma unroll
       for (int k = 0; k < KD; ++k) {
-        if (k < n_dir) {
+        // pair_share (rho == 1): gu_k and gu_{k^1} are both sum - X_k - X_{k^1}; one plane per
+        // pair is stored (G == X: in place, every plane)
+        if (k < n_dir && !(pair_share && (k & 1))) {
           Pack<V> g;
 #pragma unroll
           for (int j = 0; j < V; ++j) g.v[j] = fmaf(rho, sum.v[j] - x[k].v[j], -x[k ^ 1].v[j]);
-          st_pack<V>(X + (int64_t)k * N + i, g);
+          st_pack<V>(G + (int64_t)k * N + i, g);
         }
       }
     }
@@ -737,13 +739,17 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
                        const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
                        float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
                        float* dmsg_update, void* stream) {
-  (void)dmsg;
   (void)dunary_update;
   int rc = check_shape(s, n_iter);
   if (rc) return rc;
   if (!context || !edge_weights || !dcost_final || !msg_min_index || !msg_norm_index || !dunary ||
       !dcontext || !dedge_weights || !dmsg_update)
     return fail(MPL_EINVAL, "isgmr_backward: null tensor pointer");
+  // The reverse scans write X_k = dU_k into dmsg_update; the recombined gradients gu_k of the next
+  // (earlier) iteration go to dmsg when the caller passes it, so that at rho == 1 one plane per
+  // pair of opposite directions suffices; without dmsg they overwrite X_k in place.
+  float* gu_buf = dmsg != nullptr ? dmsg : dmsg_update;
+  const int pair_share = (dmsg != nullptr && rho == 1.f) ? 1 : 0;
   hipStream_t st = (hipStream_t)stream;
   const int64_t P = (int64_t)s->batch * s->height * s->width;
   const int64_t N = P * s->n_disp;
@@ -765,16 +771,17 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
   fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
   for (int it = n_iter - 1; it >= 0; --it) {
     const bool first = (it == n_iter - 1);
-    p.gu_in = first ? dcost_final : dmsg_update;  // gu_k = dcost_final for every k at the start
+    p.gu_in = first ? dcost_final : gu_buf;  // gu_k = dcost_final for every k at the start
     p.gu_stride = first ? 0 : N;
+    p.gu_pair_share = first ? 0 : pair_share;
     p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
     p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
     launch_bwd(p, true, st);
     Timed timed(MPL_KERNEL_COMBINE, st);
-    const bool v4 = (N % 4 == 0) && aligned16(dmsg_update) && aligned16(dcost_final) &&
-                    aligned16(dunary);
-    MPL_EW_LAUNCH(isgmr_combine_kernel, v4, s->n_dir, N, st, dmsg_update, s->n_dir, N, rho,
-                  dcost_final, factor, first ? 1 : 0, it > 0 ? 1 : 0, dunary);
+    const bool v4 = (N % 4 == 0) && aligned16(dmsg_update) && aligned16(gu_buf) &&
+                    aligned16(dcost_final) && aligned16(dunary);
+    MPL_EW_LAUNCH(isgmr_combine_kernel, v4, s->n_dir, N, st, dmsg_update, gu_buf, s->n_dir, N, rho,
+                  dcost_final, factor, first ? 1 : 0, it > 0 ? 1 : 0, pair_share, dunary);
   }
   return launch_ok("isgmr_backward");
 }

@@ -87,7 +87,9 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const int vbytes = L * 4;
   const bool read_h = !JACOBI && !p.first_touch;
   // plane bases of this batch item and direction; label-vector descriptors are formed per access
-  const float* __restrict__ bA = (JACOBI ? p.gu_in + (int64_t)dir * p.gu_stride : p.a_in) + img_e;
+  const float* __restrict__ bA =
+      (JACOBI ? p.gu_in + (int64_t)(p.gu_pair_share ? (dir & ~1) : dir) * p.gu_stride : p.a_in) +
+      img_e;
   float* __restrict__ bAo = (JACOBI ? p.du_out + (int64_t)dir * N : p.a_out) + img_e;
   float* hbase = JACOBI ? p.du_out : p.h;  // Jacobi never touches these two planes
   float* __restrict__ bHd = hbase + (int64_t)dir * N + img_e;

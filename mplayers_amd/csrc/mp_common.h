@@ -373,6 +373,7 @@ struct BackParams {
   // du_out (n_dir_total, N) receives dU_d in place of gu_d
   const float* gu_in;
   int64_t gu_stride;
+  int gu_pair_share;        // directions d and d^1 read the gu plane of the even one
   float* du_out;
   const float* edge;        // (n_dir_total, P)
   const float* ctx;

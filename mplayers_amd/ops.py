@@ -156,6 +156,10 @@ class ISGMR(object):
     _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
     _check("dedge_weights", dedge_weights, f32, shape.n_dir * P)
     _check("dmsg_update", dmsg_update, f32, shape.n_dir * N)
+    # dmsg is optional scratch: used when it has the reference's full size, ignored otherwise
+    if not (isinstance(dmsg, torch.Tensor) and dmsg.is_cuda and dmsg.is_contiguous() and
+            dmsg.dtype == f32 and dmsg.numel() >= shape.n_dir * N):
+      dmsg = None
     with torch.cuda.device(dcost_final.device):
       rc = lib.mpl_isgmr_backward(shape, int(enable_sgm), float(rho), int(n_iter), _ptr(context),
                                   _ptr(edge_weights), _ptr(dcost_final), _ptr(msg_min_index),
