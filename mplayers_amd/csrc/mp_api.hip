@@ -725,6 +725,8 @@ int mpl_trwp_backward(const mpl_shape* s, float rho, int n_iter, const float* co
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
       p.a_in = first ? dcost_final : dunary;  // CostAggregateKernelBack: every g_k starts as dcost
       p.first_touch = (it == n_iter - 1) && (d & 1);
+      p.inv_from_a = (d & 1) ? 0 : 1;  // the launch before an even direction swept d + 1 = d ^ 1
+      p.skip_hd_store = (d & 1) ? 1 : 0;
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       launch_bwd(p, false, st);

@@ -86,6 +86,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const int64_t img_e = img_p * L;
   const int vbytes = L * 4;
   const bool read_h = !JACOBI && !p.first_touch;
+  const bool inv_from_a = !JACOBI && p.inv_from_a;
   // plane bases of this batch item and direction; label-vector descriptors are formed per access
   const float* __restrict__ bA =
       (JACOBI ? p.gu_in + (int64_t)(p.gu_pair_share ? (dir & ~1) : dir) * p.gu_stride : p.a_in) +
@@ -119,7 +120,13 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     if (!JACOBI) {
       // before the first write of these planes they count as zero: an empty descriptor reads 0
       buf_load<R, VEC>(make_rsrc(bHd, read_h ? nrec : 0), foff, so, r.hd);
-      buf_load<R, VEC>(make_rsrc(bHi, read_h ? nrec : 0), foff, so, r.hi);
+      // the sweep that ran just before this one was the opposite direction's: it left
+      // h_inv = -A everywhere, so the plane need not be read (empty descriptor, no traffic)
+      buf_load<R, VEC>(make_rsrc(bHi, (read_h && !inv_from_a) ? nrec : 0), foff, so, r.hi);
+      if (inv_from_a) {
+#pragma unroll
+        for (int j = 0; j < R; ++j) r.hi[j] = -r.a[j];
+      }
     } else {
 #pragma unroll
       for (int j = 0; j < R; ++j) r.hd[j] = r.hi[j] = 0.f;
@@ -332,7 +339,9 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           hin[j] = px.hi[j] - sc[j];          // g_inv -= dU
         }
         buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, an);
-        buf_store<R, VEC>(make_rsrc(bHd, nrec), foff, so, hdn);
+        // h_dir = -A is only read by the next launch when that one sweeps the opposite
+        // direction, which derives it from A instead: nothing is stored then
+        buf_store<R, VEC>(make_rsrc(bHd, p.skip_hd_store ? 0 : nrec), foff, so, hdn);
         buf_store<R, VEC>(make_rsrc(bHi, nrec), foff, so, hin);
       }
       // each pixel receives over exactly one edge per direction: plain read-modify-write

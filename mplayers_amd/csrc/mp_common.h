@@ -369,6 +369,8 @@ struct BackParams {
   float* a_out;
   float* h;                 // (n_dir_total, N) planes h_k
   int first_touch;          // h_dir and h_inv have not been written yet: read as zero
+  int inv_from_a;           // h_inv == -A (the previous launch swept the opposite direction)
+  int skip_hd_store;        // the next launch sweeps the opposite direction and overwrites h_dir
   // ISGMR: gu_in planes (plane stride gu_stride; 0 on the first iteration where gu_k = dcost_final),
   // du_out (n_dir_total, N) receives dU_d in place of gu_d
   const float* gu_in;
