@@ -28,7 +28,7 @@ __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __r
   r.band_k = 0;
   r.c0_is_min = 0;
   r.cmax = 0.f;
-  r.pad = 0;
+  r.msg_nonzero = 0;
   if (!ctx2d) {
     float tail = ctx[L - 1];
     int k = L - 1;
@@ -101,8 +101,10 @@ __device__ __forceinline__ void st_pack(float* p, const Pack<V>& r) {
 template <int V, int ND>
 __global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ unary,
                                                      const float* __restrict__ msg, int n_dir_rt,
-                                                     int64_t N, float* __restrict__ S) {
+                                                     int64_t N, float* __restrict__ S,
+                                                     int* nonzero_flag) {
   const int n_dir = ND > 0 ? ND : n_dir_rt;
+  bool any = false;  // some message of this thread's elements is not zero
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
        i += (int64_t)gridDim.x * blockDim.x * V) {
     Pack<V> v = ld_pack<V>(unary + i);
@@ -113,16 +115,23 @@ __global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ u
 #pragma unroll
       for (int k = 0; k < ND; ++k)
 #pragma unroll
-        for (int j = 0; j < V; ++j) v.v[j] += m[k].v[j];
+        for (int j = 0; j < V; ++j) {
+          v.v[j] += m[k].v[j];
+          any = any || (m[k].v[j] != 0.f);
+        }
     } else {
       for (int k = 0; k < n_dir; ++k) {
         const Pack<V> m = ld_pack<V>(msg + (int64_t)k * N + i);
 #pragma unroll
-        for (int j = 0; j < V; ++j) v.v[j] += m.v[j];
+        for (int j = 0; j < V; ++j) {
+          v.v[j] += m.v[j];
+          any = any || (m.v[j] != 0.f);
+        }
       }
     }
     st_pack<V>(S + i, v);
   }
+  if (nonzero_flag != nullptr && any) *nonzero_flag = 1;  // every writer stores the same value
 }
 
 // ISGMR: every direction of an iteration reads the old messages only through
@@ -592,7 +601,8 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   {
     Timed timed(MPL_KERNEL_BELIEF, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
-    MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update);
+    int* flag = desc != nullptr ? &const_cast<CtxDesc*>(desc)->msg_nonzero : nullptr;
+    MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update, flag);
   }
 
   SweepParams p = base_fwd_params(s, rho, edge_weights, context, desc);
@@ -603,6 +613,7 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   for (int it = 0; it < n_iter; ++it) {
     for (int d = 0; d < s->n_dir; ++d) {  // Gauss-Seidel over directions: TRWP_forward.cu:440-518
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
+      p.first_iter = (it == 0);
       if (train) {
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
         p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
@@ -810,7 +821,8 @@ int mpl_trwp_soft_forward(const mpl_shape* s, float rho, int n_iter, const float
   {
     Timed timed(MPL_KERNEL_BELIEF, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
-    MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update);
+    MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update,
+                  (int*)nullptr);
   }
   SweepParams p = base_fwd_params(s, rho, edge_weights, context, nullptr);
   p.belief = unary_update;

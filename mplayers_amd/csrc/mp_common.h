@@ -331,7 +331,7 @@ struct CtxDesc {
   int band_k;     // > 0: c[k] == cmax for all k >= band_k and c[k] <= cmax below; 0: dense path
   int c0_is_min;  // c[0] <= c[k] for all k
   float cmax;
-  int pad;
+  int msg_nonzero;  // set by the belief pass when some initial message is not zero
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -353,6 +353,8 @@ struct SweepParams {
   const CtxDesc* desc;             // may be null: dense path
   uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
+  int first_iter;                  // Gauss-Seidel: first iteration (planes not yet swept hold the
+                                   // caller's initial messages, which need not be read when zero)
   int u_pair_share;                // Jacobi: directions d and d^1 read the U plane of the even one
   float* edge_label;               // soft TRWP: (n_dir_total, P, L, L) duals of this iteration, or null
 };

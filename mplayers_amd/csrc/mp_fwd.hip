@@ -214,6 +214,10 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   const float cmax = desc.cmax;
   const bool c0min = desc.c0_is_min != 0;
 
+  // first Gauss-Seidel iteration over all-zero initial messages: the plane of this direction has
+  // not been swept yet, and neither has the opposite one when this direction is the even one
+  const bool md_zero = !JACOBI && p.first_iter && desc.msg_nonzero == 0;
+  const bool mi_zero = md_zero && (dir & 1) == 0;
   // loads of the next pixel; past the end of the chain the last pixel is fetched again
   const int last_p = ch.pix0 + (n - 1) * ch.pstep;
   int ld_p = ch.pix0;
@@ -225,8 +229,9 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     const int nrec = (int)(so + (unsigned)vbytes);
     buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
     if (!JACOBI) {
-      buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
-      buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
+      // planes that still hold all-zero initial messages are read through an empty descriptor
+      buf_load<R, VEC>(make_rsrc(bMd, md_zero ? 0 : nrec), foff, so, r.md);
+      buf_load<R, VEC>(make_rsrc(bMi, mi_zero ? 0 : nrec), foff, so, r.mi);
     }
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
     ld_p += ch.pstep;
@@ -389,7 +394,7 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
     desc.band_k = 0;
     desc.c0_is_min = 0;
     desc.cmax = 0.f;
-    desc.pad = 0;
+    desc.msg_nonzero = 1;
   }
   // context table into LDS (dense path, run-time band taps, negative-weight fallback)
   if (R == 1 && desc.band_k == 0) {
