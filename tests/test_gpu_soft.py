@@ -205,3 +205,43 @@ def test_soft_weighted_message(gpu, oracle, T, L):
   assert np.abs(norm.cpu().numpy() - ref_norm).max() <= 1e-5 * max(1.0, np.abs(m).max())
   np.testing.assert_array_equal(ind.cpu().numpy(), ref_ind)
   assert np.abs(dm.cpu().numpy() - ref_dm).max() <= 1e-4 * max(1.0, np.abs(ref_dm).max())
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_soft_case(gpu, oracle, seed):
+  """Seeded random shapes: every block bucket, partial lanes, 2 to 16 directions, tiny grids."""
+  import torch
+  from mplayers_amd import lib_stereo
+  rng = np.random.default_rng(500 + seed)
+  n_dir = int(rng.choice([2, 4, 8, 16]))
+  B, H, W = int(rng.integers(1, 3)), int(rng.integers(1, 8)), int(rng.integers(1, 8))
+  L = int(rng.choice([1, 2, 7, 8, 9, 15, 16, 17, 21, 22, 31, 32, 33, 47, 63, 64]))
+  n_iter = int(rng.integers(1, 3))
+  ctx = make_ctx("dense2d" if L == 21 else ["tl2", "dense1d"][seed % 2], L, rng)
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ew = (0.2 + rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  dcost = rng.standard_normal((B, 1, H, W, L)).astype(np.float32)
+  print("case", seed, n_dir, B, H, W, L, n_iter, flush=True)
+  ref = oracle.forward_soft(unary, ctx, ew, n_dir, n_iter, 0.5)
+  got = gpu_forward_soft(unary, ctx, ew, n_dir, n_iter, 0.5)
+  belief = ref["cost_final"]
+  gpu.assert_values_close(got["msg"], ref["msg"], rel=2e-5, what="msg", belief=belief)
+  gpu.assert_values_close(got["cost_final"], ref["cost_final"], rel=2e-5, what="cost")
+  gpu.assert_values_close(got["msg_edge_label"], ref["msg_edge_label"], rel=2e-5, what="duals",
+                          belief=belief)
+  du, dc, de = oracle.backward_soft(ctx.astype(np.float64), ew.astype(np.float64),
+                                    dcost.astype(np.float64),
+                                    ref["msg_edge_label"].astype(np.float64),
+                                    ref["msg_norm_index"], 0.5)
+  g = t(dcost)
+  dunary = g.new_zeros(B, 1, H, W, L)
+  dmsg = torch.full((n_dir, B, 1, H, W, L), -2.5, device="cuda")
+  dctx = g.new_zeros(L, L) if L == 21 else g.new_zeros(L)
+  dedge = g.new_zeros(n_dir, B, 1, H, W)
+  lib_stereo.TRWP_hard_soft.backward_soft(0.5, g, t(ctx), t(ew), t(ref["msg_edge_label"]),
+                                          t(ref["msg_norm_index"]), dunary, dctx, dedge, dmsg,
+                                          g.new_empty(0))
+  torch.cuda.synchronize()
+  for name, a, r in (("dunary", dunary, du), ("dcontext", dctx, dc), ("dedge", dedge, de)):
+    err = np.abs(a.cpu().numpy().astype(np.float64) - r).max()
+    assert err <= 1e-4 * max(1.0, np.abs(r).max()), (name, err)
