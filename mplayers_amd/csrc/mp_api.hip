@@ -761,6 +761,11 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
   // The reverse scans write X_k = dU_k into dmsg_update; the recombined gradients gu_k of the next
   // (earlier) iteration go to dmsg when the caller passes it, so that at rho == 1 one plane per
   // pair of opposite directions suffices; without dmsg they overwrite X_k in place.
+  {
+    const int64_t planes = (int64_t)s->n_dir * s->batch * s->height * s->width * s->n_disp;
+    if (dmsg != nullptr && dmsg < dmsg_update + planes && dmsg_update < dmsg + planes)
+      dmsg = nullptr;  // overlaps dmsg_update: not usable as a second buffer
+  }
   float* gu_buf = dmsg != nullptr ? dmsg : dmsg_update;
   const int pair_share = (dmsg != nullptr && rho == 1.f) ? 1 : 0;
   hipStream_t st = (hipStream_t)stream;
