@@ -48,6 +48,9 @@ def parse():
   ap.add_argument("--copy-probe", action="store_true",
                   help="also run one plain device copy of one fp32 plane (reference point for "
                        "hardware byte counters)")
+  ap.add_argument("--peak-probe", action="store_true",
+                  help="also time plain device copy / add / fill kernels on one fp32 plane of the "
+                       "workload (reported under \"measured_stream_rates\")")
   ap.add_argument("--module-probe", action="store_true",
                   help="also time forward+backward through the nn.Module surface, which allocates "
                        "its buffers on every call as the reference's does (reported under "
@@ -97,6 +100,27 @@ def cpu_baseline(cfg, budget_s=15.0):
           "sample": "%s forward only (the reference has no CPU backward), first %d rows x %d "
                     "columns of %s, %d labels, %d directions, 1 iteration, unit edge weights, "
                     "%.1f s" % (mode, rows, W, cfg["name"], L, n_dir, dt)}
+
+
+def peak_probe(dst, src, reps=10):
+  """What this GPU sustains for plain streaming kernels on tensors of the workload's plane size:
+  copy (1 read + 1 write), add (2 reads + 1 write), fill (1 write); GB/s of bytes moved."""
+  import torch
+  nbytes = dst.numel() * 4
+  other = torch.empty_like(dst)
+  res = {}
+  for name, fn, moved in (("copy", lambda: other.copy_(src), 2 * nbytes),
+                          ("add", lambda: torch.add(src, dst, out=other), 3 * nbytes),
+                          ("fill", lambda: other.zero_(), nbytes)):
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      fn()
+    torch.cuda.synchronize()
+    res[name + "_GBs"] = moved * reps / (time.perf_counter() - t0) / 1e9
+  res["plane_bytes"] = nbytes
+  return res
 
 
 def module_probe(cfg, algs, unary, edge, dcost, reps=3):
@@ -295,6 +319,8 @@ def main():
       "other_kernels_ms": {k: round(stats[k][1], 3) for k in stats if k not in kernels},
 
   }
+  if a.peak_probe:
+    out["measured_stream_rates"] = peak_probe(cost, unary)
   if a.module_probe and training:
     out["module_surface"] = module_probe(cfg, algs, unary, edge, dcost)
   if a.edge_probe:
