@@ -171,6 +171,14 @@ int mpl_edge_shift(int mode, const float* image, int batch, int channels, int he
 /* Message of the last failed call on this thread ("" if none). */
 const char* mpl_last_error(void);
 
+/* Process-wide switches (no counterpart in the reference).
+ * MPL_OPT_PACKED_SCANS (default 1): launches of at least 2048 chains with at most 32 labels, whose
+ * planes stay below 2 GiB, are scanned with several chains per wavefront; 0 forces the
+ * one-chain-per-wavefront kernels, 2 packs whenever the label count allows it (the results agree
+ * to the parity tolerance; 0 and 2 are meant for tests and comparisons). */
+#define MPL_OPT_PACKED_SCANS 0
+int mpl_set_option(int option, int value);
+
 /* Library version: major * 100 + minor. */
 int mpl_version(void);
 

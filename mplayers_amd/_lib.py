@@ -8,7 +8,7 @@ LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hi
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
            "mpl_selftest_wave_ops", "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
            "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_trwp_soft_forward",
-           "mpl_trwp_soft_backward", "mpl_soft_weighted_message", "mpl_soft_weighted_message_back")
+           "mpl_trwp_soft_backward", "mpl_soft_weighted_message", "mpl_soft_weighted_message_back", "mpl_set_option")
 
 KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combine", "other",
                 "fwd_sweep_all", "bwd_sweep_all", "unary_all")
@@ -48,6 +48,7 @@ def load():
   lib.mpl_trwp_soft_backward.argtypes = [sp, cf, ci] + [vp] * 11
   lib.mpl_soft_weighted_message.argtypes = [ci, ci, vp, vp, vp, vp]
   lib.mpl_soft_weighted_message_back.argtypes = [ci, ci, vp, vp, vp, vp, vp]
+  lib.mpl_set_option.argtypes = [ci, ci]
   lib.mpl_edge_shift.argtypes = [ci, vp, ci, ci, ci, ci, ci, cf, cf, cf, vp, vp, vp]
   lib.mpl_selftest_wave_ops.argtypes = [ctypes.POINTER(ci)]
   lib.mpl_n_chains.argtypes = [ci, ci, ci]
@@ -58,6 +59,13 @@ def load():
   lib.mpl_last_error.restype = ctypes.c_char_p
   _lib = lib
   return lib
+
+
+OPT_PACKED_SCANS = 0
+
+
+def set_option(option, value):
+  check(load().mpl_set_option(int(option), int(value)), "set_option")
 
 
 def profile_begin():

@@ -459,8 +459,11 @@ void fill_dirs(const mpl_shape* s, int first, int count, int* dirs, int* prefix,
 
 int labels_per_lane(int L) { return (L + kWave - 1) / kWave; }
 
+bool g_packed_scans = true;  // mpl_set_option(MPL_OPT_PACKED_SCANS, ...)
+
 void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st);
+  if (g_packed_scans && launch_packed_fwd(p, train, jacobi, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_fwd<1>(p, train, jacobi, st); break;
     case 2: launch_sweep_fwd<2>(p, train, jacobi, st); break;
@@ -471,6 +474,7 @@ void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
 
 void launch_bwd(const BackParams& p, bool jacobi, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st);
+  if (g_packed_scans && launch_packed_bwd(p, jacobi, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_bwd<1>(p, jacobi, st); break;
     case 2: launch_sweep_bwd<2>(p, jacobi, st); break;
@@ -526,6 +530,16 @@ extern "C" {
 const char* mpl_last_error(void) { return g_err; }
 
 int mpl_version(void) { return 100; }
+
+int mpl_set_option(int option, int value) {
+  if (option == MPL_OPT_PACKED_SCANS) {
+    if (value < 0 || value > 2) return fail(MPL_EINVAL, "set_option: packed scans take 0, 1 or 2");
+    g_packed_scans = value != 0;
+    set_packed_policy(value == 2);
+    return MPL_OK;
+  }
+  return fail(MPL_EINVAL, "set_option: unknown option %d", option);
+}
 
 int mpl_profile_begin(void) {
   std::lock_guard<std::mutex> lk(g_prof_mu);

@@ -353,6 +353,7 @@ struct SweepParams {
   const CtxDesc* desc;             // may be null: dense path
   uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
+  int pack;                        // packed scans (mp_pack.hip): chains per wavefront
   int first_iter;                  // Gauss-Seidel: first iteration (planes not yet swept hold the
                                    // caller's initial messages, which need not be read when zero)
   int u_pair_share;                // Jacobi: directions d and d^1 read the U plane of the even one
@@ -386,6 +387,7 @@ struct BackParams {
   float* dedge;             // (n_dir_total, P) accumulates
   float* dctx;              // accumulates
   const float* edge_label;  // soft TRWP: (n_dir_total, P, L, L) duals of this iteration
+  int pack;                 // packed scans (mp_pack.hip): chains per wavefront
 };
 
 // records the message mpl_last_error() returns on this thread and returns `code`
@@ -398,6 +400,14 @@ template <int R>
 void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 
 // a_s (kMaxL floats) + the context: (L,L) for 2-D tables and for the one-label-per-lane dense path
+// packed scans for small label counts (mp_pack.hip): several chains per wavefront.
+// The launchers return false, without launching, when the problem does not qualify.
+constexpr int kPackedMaxL = 32;
+constexpr int kPackedMinChains = 2048;  // two wavefronts per SIMD of the 256 CUs when unpacked
+void set_packed_policy(bool always);  // tests: pack whatever the number of chains
+bool launch_packed_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st);
+bool launch_packed_bwd(const BackParams& p, bool jacobi, hipStream_t st);
+
 // soft-weighted TRWP (mp_soft.hip): one direction per launch, L <= 64
 void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st);
 void launch_soft_bwd(const BackParams& p, hipStream_t st);

@@ -1,0 +1,492 @@
+// Scans for small label counts (L <= 32) on gfx950: several chains share one wavefront.
+//
+// With one chain per wavefront a 21-label problem (the segmentation case) uses a third of the
+// lanes.  Here a wavefront walks G = floor(64 / L) chains of one direction at once: lane = g * L + l
+// carries label l of the wave's g-th chain, every address is per lane, and the two cross-lane
+// patterns of the recurrence work on L-lane segments:
+//   * "value of front label fd of my chain" is a ds_bpermute from lane g * L + fd,
+//   * min / sum / max over the labels of a chain is a shift-down tree of ds_bpermute steps that
+//     ends in the first lane of the segment, followed by one broadcast.
+// The step itself is the dense O(L^2) scan of the reference for any context (1-D or 2-D, any sign of
+// the edge weights): HorizontalKernel & co., TRWP_forward.cu:82-376, and the reverse scans of
+// TRWP_backward.cu:49-275, with the same belief-plane / shared-gradient-plane bookkeeping as the
+// one-chain-per-wave kernels (mp_fwd.hip, mp_bwd.hip).
+//
+// Planes are addressed from their start with 32-bit byte offsets, so a plane (B*H*W*L floats) must
+// stay below 2 GiB; larger problems take the one-chain-per-wave kernels.
+
+#include "mp_common.h"
+
+namespace mpl {
+namespace {
+
+__device__ __forceinline__ float bperm_f(int addr, float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(int, x)));
+}
+__device__ __forceinline__ int bperm_i(int addr, int x) { return __builtin_amdgcn_ds_bpermute(addr, x); }
+
+// A lane's place in its segment and the bpermute addresses of the shift-down tree.
+struct Seg {
+  int l;         // label
+  int first;     // byte address (lane * 4) of the segment's first lane
+  int down[5];   // byte address of lane + 16, 8, 4, 2, 1 when that lane belongs to the segment, else own
+  bool has[5];
+};
+
+__device__ __forceinline__ Seg make_seg(int lane, int L, int G) {
+  Seg s;
+  const int g = lane / L;
+  s.l = lane - g * L;
+  const bool in = g < G;
+  s.first = (in ? g * L : lane) * 4;
+#pragma unroll
+  for (int k = 0; k < 5; ++k) {
+    const int off = 16 >> k;
+    s.has[k] = in && (s.l + off < L);
+    s.down[k] = (s.has[k] ? lane + off : lane) * 4;
+  }
+  return s;
+}
+
+__device__ __forceinline__ float seg_min(const Seg& s, float x) {
+#pragma unroll
+  for (int k = 0; k < 5; ++k) x = fminf(x, bperm_f(s.down[k], x));
+  return bperm_f(s.first, x);
+}
+__device__ __forceinline__ int seg_max(const Seg& s, int x) {
+#pragma unroll
+  for (int k = 0; k < 5; ++k) {
+    const int y = bperm_i(s.down[k], x);
+    x = y > x ? y : x;
+  }
+  return bperm_i(s.first, x);
+}
+__device__ __forceinline__ float seg_sum(const Seg& s, float x) {
+#pragma unroll
+  for (int k = 0; k < 5; ++k) {
+    const float y = bperm_f(s.down[k], x);
+    x += s.has[k] ? y : 0.f;
+  }
+  return bperm_f(s.first, x);
+}
+
+// full symmetric context table tab[fd * L + cd] = ctx(cd, fd), TRWP_forward.cu:101-113
+__device__ __forceinline__ void fill_table(const float* ctx, int L, int ctx2d, int lane, float* tab) {
+  for (int i = lane; i < L * L; i += kWave) {
+    const int fd = i / L, cd = i - fd * L;
+    const int lo = cd < fd ? cd : fd, hi = cd < fd ? fd : cd;
+    tab[i] = ctx[ctx2d ? lo * L + hi : hi - lo];
+  }
+}
+
+// The chains of this wavefront: direction, and per lane the first pixel (index over the whole
+// batch), the number of pixels (0 for idle lanes) and the pixel stride.
+struct PackedChains {
+  int dir, pstep, n, pix0, n_max;
+  bool on;
+};
+
+template <typename Params>
+__device__ __forceinline__ PackedChains locate_packed(const Params& p, int lane, int L, int G) {
+  int di = 0;
+  while (di + 1 < p.n_dirs && (int)blockIdx.x >= p.block_prefix[di + 1]) ++di;
+  PackedChains c;
+  c.dir = p.dirs[di];
+  const int wave = (int)blockIdx.x - p.block_prefix[di];
+  const DirGeom geo = make_dir(c.dir, p.H, p.W);
+  const int g = lane / L;
+  const int64_t total = (int64_t)p.B * geo.n_chains;
+  const int64_t idx = (int64_t)wave * G + g;
+  c.on = (g < G) && (idx < total);
+  c.n = 0;
+  c.pix0 = 0;
+  if (c.on) {
+    const int bv = (int)(idx / geo.n_chains);
+    const int ch = (int)(idx - (int64_t)bv * geo.n_chains);
+    int h0, w0;
+    chain_start(geo, p.H, p.W, ch, &h0, &w0, &c.n);
+    c.pix0 = bv * p.H * p.W + h0 * p.W + w0;
+  }
+  c.pstep = geo.hs * p.W + geo.ws;
+  c.n_max = (int)(-wave_min(-(float)c.n));
+  return c;
+}
+
+__device__ __forceinline__ float ldf(rsrc_t r, unsigned off) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, MPL_LD_AUX));
+}
+__device__ __forceinline__ void stf(rsrc_t r, unsigned off, float v) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, (int)off, 0, MPL_ST_AUX);
+}
+
+struct PixPF {
+  float s, md, mi, w;
+};
+
+// LT > 0: label count known at compile time (21): front-label loop unrolled, context column in
+// registers.
+template <bool TRAIN, bool JACOBI, int LT>
+__global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) {
+  extern __shared__ float smem[];
+  float* tab = smem;  // L * L
+  const int L = LT > 0 ? LT : p.L;
+  const int G = p.pack;
+  const int lane = threadIdx.x;
+  const PackedChains ch = locate_packed(p, lane, L, G);
+  const Seg sg = make_seg(lane, L, G);
+  fill_table(p.ctx, L, p.ctx2d, lane, tab);
+  __syncthreads();
+  if (!JACOBI && ch.n_max < 2) return;
+
+  const int64_t P = (int64_t)p.B * p.H * p.W;
+  const int64_t N = P * L;
+  const int dir = ch.dir;
+  const int plane_bytes = (int)(N * 4);
+  const bool md_zero = !JACOBI && p.first_iter && p.desc != nullptr && p.desc->msg_nonzero == 0;
+  const bool mi_zero = md_zero && (dir & 1) == 0;
+  const int udir = p.u_pair_share ? (dir & ~1) : dir;
+  const rsrc_t dS = make_rsrc(JACOBI ? p.msg_in + (int64_t)udir * N : p.belief, plane_bytes);
+  const rsrc_t dMd = make_rsrc(p.msg_in + (int64_t)dir * N, (JACOBI || md_zero) ? 0 : plane_bytes);
+  const rsrc_t dMi = make_rsrc(p.msg_in + (int64_t)(dir ^ 1) * N, (JACOBI || mi_zero) ? 0 : plane_bytes);
+  const rsrc_t dMo = make_rsrc(p.msg_out + (int64_t)dir * N, plane_bytes);
+  const rsrc_t dSo = make_rsrc(JACOBI ? nullptr : p.belief_out, JACOBI ? 0 : plane_bytes);
+  const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P, (int)(P * 4));
+  const rsrc_t dImin = make_rsrc(TRAIN ? p.idx_min + (int64_t)dir * N : nullptr, TRAIN ? (int)N : 0);
+  const rsrc_t dInorm = make_rsrc(TRAIN ? p.idx_norm + (int64_t)dir * P : nullptr, TRAIN ? (int)P : 0);
+  const float rho = p.rho;
+  const float inf = INFINITY;
+  const int l = sg.l;
+  const bool on = ch.on;
+  const int n = ch.n;
+
+  float tcol[LT > 0 ? LT : 1];
+  if (LT > 0) {
+#pragma unroll
+    for (int fd = 0; fd < LT; ++fd) tcol[fd] = tab[fd * LT + l];
+  }
+
+  int ld_pix = ch.pix0, ld_t = 0;
+  auto load_next = [&]() {
+    PixPF r;
+    const bool act = on && ld_t < n;
+    const unsigned eo = act ? (unsigned)(ld_pix * L + l) * 4u : (unsigned)kDeadOffset;
+    r.s = ldf(dS, eo);
+    if (!JACOBI) {
+      r.md = ldf(dMd, eo);
+      r.mi = ldf(dMi, eo);
+    } else {
+      r.md = r.mi = 0.f;
+    }
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                        dW, act ? ld_pix * 4 : kDeadOffset, 0, 0));
+    ld_pix += ch.pstep;
+    ld_t += 1;
+    return r;
+  };
+
+  float prev = 0.f, uf;
+  {
+    const PixPF p0 = load_next();
+    const float un = JACOBI ? p0.s : fmaf(p0.s - p0.md, rho, -p0.mi);
+    uf = on ? un : inf;
+    if (JACOBI)  // the buffers alternate: the chain start is written with the zeros it keeps
+      stf(dMo, (on && n >= 1) ? (unsigned)(ch.pix0 * L + l) * 4u : (unsigned)kDeadOffset, 0.f);
+  }
+
+  constexpr int kOps = (JACOBI ? 1 : 3) + 1 + (JACOBI ? 1 : 2) + (TRAIN ? 2 : 0);
+  constexpr int D = ring_depth(kOps);
+  PixPF ring[D];
+#pragma unroll
+  for (int u = 0; u < D; ++u) ring[u] = load_next();
+
+  int st_pix = ch.pix0 + ch.pstep;
+  for (int t0 = 1; t0 < ch.n_max; t0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int t = t0 + u;
+      const bool live = on && t < n;
+      wait_vmem<(D - 1) * kOps>();
+      const PixPF px = ring[u];
+      ring[u] = load_next();
+      const float tt = px.s - px.md;
+      const float x = JACOBI ? px.s : fmaf(tt, rho, -px.mi);  // UpdateUnaryKernel, :70-78
+      const float un = on ? x : inf;
+      const float w = px.w;
+      const float a = fmaf(rho, prev, uf);
+      // v[cd] = min_fd a[fd] + w * ctx(cd, fd), largest fd on ties (TRWP_forward.cu:127-153)
+      float best = inf;
+      int arg = L - 1;
+      if constexpr (LT > 0) {
+#pragma unroll
+        for (int fd = LT - 1; fd >= 0; --fd) {
+          const float val = fmaf(w, tcol[fd], bperm_f(sg.first + fd * 4, a));
+          const bool take = (fd == LT - 1) || (val < best);
+          best = take ? val : best;
+          if (TRAIN) arg = take ? fd : arg;
+        }
+      } else {
+#pragma unroll 4
+        for (int fd = L - 1; fd >= 0; --fd) {
+          const float val = fmaf(w, tab[fd * L + l], bperm_f(sg.first + fd * 4, a));
+          const bool take = (fd == L - 1) || (val < best);
+          best = take ? val : best;
+          if (TRAIN) arg = take ? fd : arg;
+        }
+      }
+      const float nmin = seg_min(sg, on ? best : inf);  // MsgNormNaive, commonCUDA.cuh:92-129
+      const float m = best - nmin;
+      prev = on ? m : 0.f;
+      uf = un;
+      const unsigned eo = live ? (unsigned)(st_pix * L + l) * 4u : (unsigned)kDeadOffset;
+      stf(dMo, eo, m);
+      if (!JACOBI) stf(dSo, eo, tt + m);
+      if (TRAIN) {
+        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)arg, dImin,
+                                             live ? st_pix * L + l : kDeadOffset, 0, MPL_ST_AUX);
+        const int nidx = seg_max(sg, (on && best == nmin) ? l : -1);  // largest label on ties
+        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm,
+                                             (live && l == 0) ? st_pix : kDeadOffset, 0, 0);
+      }
+      st_pix += ch.pstep;
+    }
+  }
+}
+
+struct PixPB {
+  float a, hd, hi;
+  int fd, nidx;
+  float w, de;
+};
+
+template <bool JACOBI, int LT>
+__global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
+  extern __shared__ float smem[];
+  const int L = LT > 0 ? LT : p.L;
+  const int G = p.pack;
+  float* tab = smem;           // L * L
+  float* pairs = smem + L * L; // G tables of L * L: dcontext per (cd, fd) pair and chain slot
+  const int lane = threadIdx.x;
+  const PackedChains ch = locate_packed(p, lane, L, G);
+  const Seg sg = make_seg(lane, L, G);
+  fill_table(p.ctx, L, p.ctx2d, lane, tab);
+  for (int i = lane; i < G * L * L; i += kWave) pairs[i] = 0.f;
+  __syncthreads();
+
+  const int64_t P = (int64_t)p.B * p.H * p.W;
+  const int64_t N = P * L;
+  const int dir = ch.dir;
+  const int plane_bytes = (int)(N * 4);
+  const bool read_h = !JACOBI && !p.first_touch;
+  const bool inv_from_a = !JACOBI && p.inv_from_a;
+  const int gdir = p.gu_pair_share ? (dir & ~1) : dir;
+  const rsrc_t dA = make_rsrc(JACOBI ? p.gu_in + (int64_t)gdir * p.gu_stride : p.a_in, plane_bytes);
+  const rsrc_t dAo = make_rsrc(JACOBI ? p.du_out + (int64_t)dir * N : p.a_out, plane_bytes);
+  float* hbase = JACOBI ? p.du_out : p.h;
+  const rsrc_t dHdIn = make_rsrc(hbase + (int64_t)dir * N, read_h ? plane_bytes : 0);
+  const rsrc_t dHiIn = make_rsrc(hbase + (int64_t)(dir ^ 1) * N, (read_h && !inv_from_a) ? plane_bytes : 0);
+  const rsrc_t dHdOut = make_rsrc(hbase + (int64_t)dir * N, (JACOBI || p.skip_hd_store) ? 0 : plane_bytes);
+  const rsrc_t dHiOut = make_rsrc(hbase + (int64_t)(dir ^ 1) * N, JACOBI ? 0 : plane_bytes);
+  const rsrc_t dImin = make_rsrc(p.idx_min + (int64_t)dir * N, (int)N);
+  const rsrc_t dInorm = make_rsrc(p.idx_norm + (int64_t)dir * P, (int)P);
+  const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P, (int)(P * 4));
+  const rsrc_t dDe = make_rsrc(p.dedge + (int64_t)dir * P, (int)(P * 4));
+  const float rho = p.rho;
+  const int l = sg.l;
+  const bool on = ch.on;
+  const int n = ch.n;
+  float* my_pairs = pairs + (lane / L < G ? lane / L : 0) * L * L + l * L;  // row of this label
+
+  // every chain is walked from its own last pixel: step s visits t = n - 1 - s
+  int ld_pix = ch.pix0 + (n - 1) * ch.pstep, ld_t = n - 1;
+  auto load_next = [&]() {
+    PixPB r;
+    const bool act = on && ld_t >= 0;
+    const unsigned eo = act ? (unsigned)(ld_pix * L + l) * 4u : (unsigned)kDeadOffset;
+    r.a = ldf(dA, eo);
+    if (!JACOBI) {
+      r.hd = ldf(dHdIn, eo);
+      r.hi = ldf(dHiIn, eo);
+      if (inv_from_a) r.hi = -r.a;
+    } else {
+      r.hd = r.hi = 0.f;
+    }
+    r.fd = __builtin_amdgcn_raw_buffer_load_b8(dImin, act ? ld_pix * L + l : kDeadOffset, 0, MPL_LD_AUX);
+    r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, act ? ld_pix : kDeadOffset, 0, 0);
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                        dW, act ? ld_pix * 4 : kDeadOffset, 0, 0));
+    r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                         dDe, (act && l == 0) ? ld_pix * 4 : kDeadOffset, 0, 0));
+    ld_pix -= ch.pstep;
+    ld_t -= 1;
+    return r;
+  };
+
+  constexpr int kOps = (JACOBI ? 1 : 3) + 4 + (JACOBI ? 1 : 3) + 1;
+  constexpr int D = ring_depth(kOps);
+  PixPB ring[D];
+#pragma unroll
+  for (int u = 0; u < D; ++u) ring[u] = load_next();
+
+  float sc = 0.f;  // dU of the current pixel: what the previous step scattered into it
+  int st_pix = ch.pix0 + (n - 1) * ch.pstep;
+  for (int s0 = 0; s0 < ch.n_max; s0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int t = n - 1 - (s0 + u);  // per lane
+      const bool here = on && t >= 0;  // this lane's chain has a pixel at this step
+      wait_vmem<(D - 1) * kOps>();
+      const PixPB px = ring[u];
+      ring[u] = load_next();
+      // gradient w.r.t. the normalised message of this pixel (none at the chain start, t == 0)
+      const bool edge = on && t >= 1;
+      float g = edge ? fmaf(rho, sc, JACOBI ? px.a : px.a + px.hd) : 0.f;
+      const float tot = seg_sum(sg, g);  // MsgNormNaiveBack, commonCUDA.cuh:131-145
+      if (edge && l == px.nidx) g -= tot;
+      const int fd = px.fd;
+      // dU[q, f] = sum of g[c] over the labels c of this chain whose argmin is f
+      float scn = 0.f;
+      if constexpr (LT > 0) {
+#pragma unroll
+        for (int c = 0; c < LT; ++c) {
+          const float gc = bperm_f(sg.first + c * 4, g);
+          const int fc = bperm_i(sg.first + c * 4, fd);
+          scn += (fc == l) ? gc : 0.f;
+        }
+      } else {
+#pragma unroll 4
+        for (int c = 0; c < L; ++c) {
+          const float gc = bperm_f(sg.first + c * 4, g);
+          const int fc = bperm_i(sg.first + c * 4, fd);
+          scn += (fc == l) ? gc : 0.f;
+        }
+      }
+      // dedge_weights[p] += ctx(cd, fd) * g;  dcontext[(cd, fd)] += w * g for cd != fd
+      // (TRWP_backward.cu:109-112)
+      const int fdc = edge ? fd : 0;
+      const float det = seg_sum(sg, tab[fdc * L + l] * g);
+      if (edge && fdc != l) my_pairs[fdc] = fmaf(px.w, g, my_pairs[fdc]);
+      const unsigned eo = here ? (unsigned)(st_pix * L + l) * 4u : (unsigned)kDeadOffset;
+      if (JACOBI) {
+        stf(dAo, eo, sc);
+      } else {
+        const float an = fmaf(rho, sc, px.a);  // g_k += rho * dU for every k, dunary too
+        stf(dAo, eo, an);
+        stf(dHdOut, eo, -an);          // g_dir = 0 after its sweep
+        stf(dHiOut, eo, px.hi - sc);   // g_inv -= dU
+      }
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
+                                            (edge && l == 0) ? st_pix * 4 : kDeadOffset, 0, 0);
+      sc = here ? scn : 0.f;
+      st_pix -= ch.pstep;
+    }
+  }
+  __syncthreads();
+  // fold the pair tables of all chain slots into dcontext's bins
+  if (!p.ctx2d) {
+    if (lane >= 1 && lane < L) {
+      float acc = 0.f;
+      for (int g2 = 0; g2 < G; ++g2)
+        for (int c = 0; c < L; ++c) {
+          if (c + lane < L) acc += pairs[g2 * L * L + c * L + c + lane];
+          if (c - lane >= 0) acc += pairs[g2 * L * L + c * L + c - lane];
+        }
+      if (acc != 0.f) atomicAdd(&p.dctx[lane], acc);
+    }
+  } else {
+    for (int i = lane; i < L * L; i += kWave) {
+      const int c = i / L, f = i - c * L;
+      if (c >= f) continue;
+      float v = 0.f;
+      for (int g2 = 0; g2 < G; ++g2) v += pairs[g2 * L * L + i] + pairs[g2 * L * L + f * L + c];
+      if (v != 0.f) atomicAdd(&p.dctx[i], v);
+    }
+  }
+}
+
+// prefix sums of wavefronts per direction for G chains per wavefront
+template <typename Params>
+int64_t chains_in_launch(const Params& p) {
+  int64_t c = 0;
+  for (int i = 0; i < p.n_dirs; ++i) c += (int64_t)p.B * make_dir(p.dirs[i], p.H, p.W).n_chains;
+  return c;
+}
+
+template <typename Params>
+Params with_wave_prefix(const Params& p, int G) {
+  Params q = p;
+  q.pack = G;
+  q.block_prefix[0] = 0;
+  for (int i = 0; i < p.n_dirs; ++i) {
+    const int64_t chains = (int64_t)p.B * make_dir(p.dirs[i], p.H, p.W).n_chains;
+    q.block_prefix[i + 1] = q.block_prefix[i] + (int)((chains + G - 1) / G);
+  }
+  return q;
+}
+
+}  // namespace
+
+bool g_pack_always = false;  // set_packed_policy
+
+int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains) {
+  if (L > kPackedMaxL) return 0;
+  if ((int64_t)B * H * W * L * 4 >= (int64_t)kDeadOffset) return 0;  // 32-bit plane offsets
+  // A packed step issues fewer instructions per chain but has the longer dependent chain (its
+  // reductions go through ds_bpermute): it pays once every SIMD of the 256 CUs would otherwise
+  // hold two or more wavefronts (measured: 516 chains of 129 pixels and 21 labels per launch are
+  // 25 % faster unpacked, 2064 chains 15-40 % faster packed).
+  if (chains < (g_pack_always ? 1 : kPackedMinChains)) return 0;
+  int G = kWave / L;
+  return G > 16 ? 16 : G;
+}
+
+void set_packed_policy(bool always) { g_pack_always = always; }
+
+bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, hipStream_t st) {
+  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0));
+  if (G < 2) return false;
+  const SweepParams p = with_wave_prefix(p0, G);
+  const int blocks = p.block_prefix[p.n_dirs];
+  const size_t lds = sizeof(float) * p.L * p.L;
+#define MPL_PACKED_FWD(LT)                                                                 \
+  do {                                                                                     \
+    if (train) {                                                                           \
+      if (jacobi)                                                                          \
+        packed_fwd_kernel<true, true, LT><<<blocks, kWave, lds, st>>>(p);                  \
+      else                                                                                 \
+        packed_fwd_kernel<true, false, LT><<<blocks, kWave, lds, st>>>(p);                 \
+    } else {                                                                               \
+      if (jacobi)                                                                          \
+        packed_fwd_kernel<false, true, LT><<<blocks, kWave, lds, st>>>(p);                 \
+      else                                                                                 \
+        packed_fwd_kernel<false, false, LT><<<blocks, kWave, lds, st>>>(p);                \
+    }                                                                                      \
+  } while (0)
+  if (p.L == 21)
+    MPL_PACKED_FWD(21);
+  else
+    MPL_PACKED_FWD(0);
+#undef MPL_PACKED_FWD
+  return true;
+}
+
+bool launch_packed_bwd(const BackParams& p0, bool jacobi, hipStream_t st) {
+  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0));
+  if (G < 2) return false;
+  const BackParams p = with_wave_prefix(p0, G);
+  const int blocks = p.block_prefix[p.n_dirs];
+  const size_t lds = sizeof(float) * p.L * p.L * (1 + G);
+  if (p.L == 21) {
+    if (jacobi)
+      packed_bwd_kernel<true, 21><<<blocks, kWave, lds, st>>>(p);
+    else
+      packed_bwd_kernel<false, 21><<<blocks, kWave, lds, st>>>(p);
+  } else {
+    if (jacobi)
+      packed_bwd_kernel<true, 0><<<blocks, kWave, lds, st>>>(p);
+    else
+      packed_bwd_kernel<false, 0><<<blocks, kWave, lds, st>>>(p);
+  }
+  return true;
+}
+
+}  // namespace mpl
