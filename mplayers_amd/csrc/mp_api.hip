@@ -422,10 +422,15 @@ int launch_ok(const char* what) {
   return MPL_OK;
 }
 
+// One pass over the data with as many workgroups as it takes measured 3-8 % faster than a
+// grid-stride loop of 32 workgroups per CU on the 2.3 GB planes; the cap only bounds the grid.
+#ifndef MPL_EW_BLOCKS_PER_CU
+#define MPL_EW_BLOCKS_PER_CU 4096
+#endif
 int elementwise_blocks(int64_t n) {
   int64_t b = (n + 256 * 4 - 1) / (256 * 4);
   if (b < 1) b = 1;
-  if (b > 256 * 32) b = 256 * 32;
+  if (b > 256 * MPL_EW_BLOCKS_PER_CU) b = 256 * MPL_EW_BLOCKS_PER_CU;
   return (int)b;
 }
 
