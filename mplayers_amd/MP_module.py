@@ -173,13 +173,17 @@ class MPModule(torch.nn.Module):
         create_label_context(self.args, enable_seg=self.args.enable_seg,
                              enable_symmetric=self.args.enable_symmetric)
 
-  def _effective_label_context(self):
-    """Re-parameterisation of the learned context (MP_module.py:207-220)."""
-    label_context = self.label_context * 1
+  def _effective_label_context(self, weight_first=False):
+    """Re-parameterisation of the learned context (MP_module.py:207-220).  weight_first: the term
+    weight scales the stored parameter before the re-parameterisation instead of the sigmoid's
+    output (the hard/soft module, MP_module_hard_soft.py:148-163)."""
+    term_weight = self.args.mpnet_term_weight
+    label_context = self.label_context * (term_weight if weight_first else 1)
     mode = self.args.mpnet_smoothness_train
     if mode == 'sigmoid':
       valid = label_context[self.label_context_loc].flatten()
-      label_context[self.label_context_loc] = 2 * self.args.mpnet_term_weight * torch.sigmoid(valid)
+      scale = 2 if weight_first else 2 * term_weight
+      label_context[self.label_context_loc] = scale * torch.sigmoid(valid)
     elif mode == 'softmax':
       valid = label_context[self.label_context_loc].flatten()
       norm = nn.Softmax(dim=0)(valid)

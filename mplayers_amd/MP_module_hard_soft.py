@@ -1,7 +1,8 @@
-"""Python surface of the hard/soft TRWP layer: TRWPFunction and MPModule with the names, arguments
-and return tuples of the reference's pytorch/MP_module_hard_soft.py:13-182 (the module mpnet.py:35
-builds its CRF layer from).  `args.mpnet_enable_soft` switches between the min-sum operator and the
-soft-weighted one; everything runs in the HIP library of this package.
+"""Hard / soft-weighted TRWP layer behind the surface of the reference's
+pytorch/MP_module_hard_soft.py:13-182 (the module mpnet.py:35 builds its CRF layer from): a
+`TRWPFunction` with four outputs and an `MPModule` with five.  `args.mpnet_enable_soft` selects the
+soft-weighted operator (softmin expectation over the front labels) or the min-sum one; both run in
+the HIP library of this package.
 
   TRWPFunction.apply(unary (B, cv, H, W, L), label_context, edge_weights (n_dir, B, cv, H, W) | None,
                      args) -> (cost_final, label_all, message_edge_label, cost_index)
@@ -11,150 +12,117 @@ soft-weighted one; everything runs in the HIP library of this package.
                        message_edge_label, cost_index)
 """
 import torch
-import torch.nn as nn
 
 from . import lib_seg, lib_stereo
-from .label_context import create_label_context
+from .MP_module import MPModule as _HardModule
+
+_U8 = dict(dtype=torch.uint8)
 
 
-def _ops_for(n_disp):
+def _operators(n_disp):
   # MP_module_hard_soft.py:20: the segmentation build for 21 labels, the stereo build otherwise
   return (lib_seg if n_disp == 21 else lib_stereo).TRWP_hard_soft
 
 
+def _none_u8():
+  return torch.empty(0, **_U8)
+
+
 class TRWPFunction(torch.autograd.Function):
-  """MP_module_hard_soft.py:13-108."""
+  """MP_module_hard_soft.py:13-108.  Outputs beyond the cost: per-iteration labels (empty unless
+  args.enable_saving_label), the stored duals of the soft operator (empty in hard mode or outside
+  training) and the normalisation indices."""
 
   @staticmethod
   def forward(ctx, unary, label_context, edge_weights, args):
-    batch, cv, h, w, n_disp = unary.size()
-    rho, n_iter, n_dir = args.rho, int(args.mpnet_max_iter), int(args.mpnet_n_dirs)
-    training = args.training
-    ops = _ops_for(n_disp)
-    u8 = dict(dtype=torch.uint8)
-    # only the initial messages have to be zero; the library writes every element of the other
-    # tensors that is read later, except the stored duals of chain-start pixels, which callers
-    # can see in the returned tensor and which therefore start at zero as in the reference
-    message = unary.new_zeros(n_dir, batch, cv, h, w, n_disp)
-    cost_final = unary.new_empty(batch, cv, h, w, n_disp)
-    unary_update = unary.new_empty(batch, cv, h, w, n_disp)
-    enable_edge_weights = edge_weights is not None
-    if not enable_edge_weights:
-      edge_weights = unary.new_ones(n_dir, batch, cv, h, w)
-    label_all = (unary.new_empty(n_iter, batch, cv, h, w, **u8) if args.enable_saving_label
-                 else torch.empty(0, **u8))
-    if args.mpnet_enable_soft:
+    shape = tuple(unary.shape)                      # (batch, cv, h, w, n_disp)
+    n_disp = shape[-1]
+    n_iter, n_dir = int(args.mpnet_max_iter), int(args.mpnet_n_dirs)
+    soft, training = bool(args.mpnet_enable_soft), bool(args.training)
+    per_dir = (n_dir,) + shape
+    per_iter = (n_iter, n_dir) + shape[:-1]
+    had_weights = edge_weights is not None
+    if not had_weights:
+      edge_weights = unary.new_ones((n_dir,) + shape[:-1])
+    # The initial messages must be zero.  Of the rest, only what a caller can look at is cleared
+    # (the operators leave the entries of chain-start pixels untouched); scratch is not.
+    message = unary.new_zeros(per_dir)
+    cost_final = unary.new_empty(shape)
+    scratch = unary.new_empty(shape)
+    label_all = (unary.new_empty((n_iter,) + shape[:-1], **_U8) if args.enable_saving_label
+                 else _none_u8())
+    cost_index = unary.new_zeros(per_iter, **_U8) if training else _none_u8()
+    message_edge_label = torch.empty(0, dtype=torch.float32)
+    message_index = _none_u8()
+    op = _operators(n_disp)
+    if soft:
       if training:
-        message_edge_label = unary.new_zeros(n_iter, n_dir, batch, cv, h, w, n_disp, n_disp)
-        cost_index = unary.new_zeros(n_iter, n_dir, batch, cv, h, w, **u8)
-      else:
-        message_edge_label = torch.empty(0, dtype=torch.float32)
-        cost_index = torch.empty(0, **u8)
-      ops.forward_soft(rho, n_iter, unary, label_context, edge_weights, message,
-                       message_edge_label, cost_index, cost_final, unary_update, label_all)
-      message_index = torch.empty(0, dtype=torch.float32)
+        message_edge_label = unary.new_zeros(per_iter + (n_disp, n_disp))
+      op.forward_soft(args.rho, n_iter, unary, label_context, edge_weights, message,
+                      message_edge_label, cost_index, cost_final, scratch, label_all)
     else:
       if training:
-        message_index = unary.new_empty(n_iter, n_dir, batch, cv, h, w, n_disp, **u8)
-        cost_index = unary.new_zeros(n_iter, n_dir, batch, cv, h, w, **u8)
-      else:
-        message_index = torch.empty(0, **u8)
-        cost_index = torch.empty(0, **u8)
-      ops.forward(rho, n_iter, 0, unary, label_context, edge_weights, message, cost_final,
-                  message_index, cost_index, unary_update, label_all)
-      message_edge_label = torch.empty(0, dtype=torch.float32)
-    ctx.intermediate_results = (rho, args, message_edge_label, message_index, cost_index,
-                                label_context, edge_weights, enable_edge_weights)
+        message_index = unary.new_empty(per_iter + (n_disp,), **_U8)
+      op.forward(args.rho, n_iter, 0, unary, label_context, edge_weights, message, cost_final,
+                 message_index, cost_index, scratch, label_all)
+    ctx.saved = dict(args=args, soft=soft, blocks=message_edge_label, index=message_index,
+                     cost_index=cost_index, context=label_context, weights=edge_weights,
+                     had_weights=had_weights)
     return cost_final, label_all, message_edge_label, cost_index
 
   @staticmethod
   def backward(ctx, dcost_final, dlabel_all, dmessage_edge_label, dcost_index):
+    saved = ctx.saved
+    del ctx.saved
+    args = saved["args"]
     dcost_final = dcost_final.contiguous()
-    rho, args, message_edge_label, message_index, cost_index, label_context, edge_weights, \
-        enable_edge_weights = ctx.intermediate_results
-    del ctx.intermediate_results
     # a caller may impose the normalisation indices (MP_module_hard_soft.py:77)
-    cost_index = args.msg_norm_index if (args.msg_norm_index is not None) else cost_index
-    n_iter, n_dir, batch, cv, h, w = cost_index.size()
-    n_disp = args.n_classes
-    ops = _ops_for(n_disp)
-    dunary = dcost_final.new_empty(batch, cv, h, w, n_disp)
-    dmessage = dcost_final.new_empty(n_dir, batch, cv, h, w, n_disp)
-    dunary_update = dcost_final.new_empty(0)
-    dedge_weights = dcost_final.new_zeros(n_dir, batch, cv, h, w)
-    if args.enable_seg:
-      dlabel_context = dcost_final.new_zeros(n_disp, n_disp)
+    cost_index = saved["cost_index"] if args.msg_norm_index is None else args.msg_norm_index
+    n_iter, n_dir = cost_index.shape[:2]
+    shape = tuple(cost_index.shape[2:]) + (args.n_classes,)
+    n_disp = shape[-1]
+    dunary = dcost_final.new_empty(shape)
+    scratch = dcost_final.new_empty((n_dir,) + shape)
+    unused = dcost_final.new_empty(0)
+    dedge_weights = dcost_final.new_zeros((n_dir,) + shape[:-1])
+    dlabel_context = dcost_final.new_zeros((n_disp, n_disp) if args.enable_seg else (n_disp,))
+    op = _operators(n_disp)
+    if saved["soft"]:
+      op.backward_soft(args.rho, dcost_final, saved["context"], saved["weights"], saved["blocks"],
+                       cost_index, dunary, dlabel_context, dedge_weights, scratch, unused)
     else:
-      dlabel_context = dcost_final.new_zeros(n_disp)
-    if args.mpnet_enable_soft:
-      ops.backward_soft(rho, dcost_final, label_context, edge_weights, message_edge_label,
-                        cost_index, dunary, dlabel_context, dedge_weights, dmessage, dunary_update)
-    else:
-      ops.backward(rho, label_context, edge_weights, dcost_final, message_index, cost_index,
-                   dunary, dlabel_context, dedge_weights, dmessage, dunary_update)
-    dedge_weights = dedge_weights if enable_edge_weights else None
-    return dunary, dlabel_context, dedge_weights, None, None, None
+      op.backward(args.rho, saved["context"], saved["weights"], dcost_final, saved["index"],
+                  cost_index, dunary, dlabel_context, dedge_weights, scratch, unused)
+    return (dunary, dlabel_context, dedge_weights if saved["had_weights"] else None, None, None,
+            None)
 
 
-class MPModule(torch.nn.Module):
-  """MP_module_hard_soft.py:111-182.  Reads from `args`: mpnet_mrf_mode ('TRWP'), mpnet_enable_soft,
-  mpnet_max_iter, mpnet_n_dirs, n_classes, mpnet_term_weight, mpnet_smoothness_train / _mode /
-  _trunct_value / _trunct_loc, mpnet_diag_value, enable_symmetric; writes rho, enable_saving_label,
-  enable_seg and, per call, training and msg_norm_index."""
+class MPModule(_HardModule):
+  """MP_module_hard_soft.py:111-182.  Shares the label-context handling with the hard module; the
+  differences are the constructor (no min-over-directions switch; only TRWP), the place of the term
+  weight (it scales the stored parameter before the re-parameterisation, :148-163) and the two
+  extra inputs / outputs of forward."""
 
   def __init__(self, args, enable_create_label_context=False, enable_saving_label=False):
-    super(MPModule, self).__init__()
-    self.args = args
-    self.args.enable_saving_label = enable_saving_label
-    self.args.rho = 0.5 if (args.mpnet_mrf_mode == 'TRWP') else 1
-    self.args.enable_seg = True if (args.n_classes == 21) else False
-    self.smoothness_train = args.mpnet_smoothness_train if args.mpnet_smoothness_train else None
-    self.smoothness_mode = args.mpnet_smoothness_mode if args.mpnet_smoothness_mode else None
+    super(MPModule, self).__init__(args, enable_create_label_context=enable_create_label_context,
+                                   enable_saving_label=enable_saving_label)
+    self.smoothness_train = args.mpnet_smoothness_train or None
+    self.smoothness_mode = args.mpnet_smoothness_mode or None
     self.smoothness_trunct_value = args.mpnet_smoothness_trunct_value
     self.smoothness_trunct_loc = args.mpnet_smoothness_trunct_loc
-    if enable_create_label_context:
-      self.create_label_context()
-
-  def get_label_context(self):
-    return self.label_context, self.label_context_loc, self.label_context_diag_loc
-
-  def set_label_context(self, label_context, label_context_loc, label_context_diag_loc):
-    self.label_context = label_context
-    self.label_context_loc = label_context_loc
-    self.label_context_diag_loc = label_context_diag_loc
-
-  def create_label_context(self):
-    self.label_context, self.label_context_loc, self.label_context_diag_loc = \
-        create_label_context(self.args, enable_seg=self.args.enable_seg,
-                             enable_symmetric=self.args.enable_symmetric)
 
   def forward(self, unary, edge_weights=None, msg_norm_index=None, pairwise_terms=None):
+    assert self.args.mpnet_mrf_mode == 'TRWP'
     unary = unary.permute(0, 1, 3, 4, 2).contiguous()
     if edge_weights is not None:
       edge_weights = edge_weights.unsqueeze(1).permute(2, 0, 1, 3, 4).contiguous()
-    # the term weight scales the stored parameter before the re-parameterisation (:148-163)
-    label_context = self.label_context * self.args.mpnet_term_weight
-    mode = self.args.mpnet_smoothness_train
-    if mode == 'sigmoid':
-      valid = label_context[self.label_context_loc].flatten()
-      label_context[self.label_context_loc] = 2 * torch.sigmoid(valid)
-    elif mode == 'softmax':
-      valid = label_context[self.label_context_loc].flatten()
-      norm = nn.Softmax(dim=0)(valid)
-      label_context[self.label_context_loc] = norm * valid.max() / norm.max()
-    if mode in {'sigmoid', 'softmax'}:
-      diag = self.label_context_diag_loc
-      label_context[tuple(diag) if isinstance(diag, list) else diag] = self.args.mpnet_diag_value
-    if edge_weights is not None:
       assert unary.size()[-3:-1] == edge_weights.size()[-2:]
-    if unary.is_cuda and (msg_norm_index is not None):
+    label_context = self._effective_label_context(weight_first=True)
+    if msg_norm_index is not None and unary.is_cuda:
       msg_norm_index = msg_norm_index.cuda()
     self.args.msg_norm_index = msg_norm_index
     self.args.training = self.training
-    if self.args.mpnet_mrf_mode == 'TRWP':
-      cost_final, cost_all, message_vector, message_index = \
-          TRWPFunction.apply(unary, label_context, edge_weights, self.args)
-    else:
-      assert False
-    cost_final = cost_final.permute(0, 1, 4, 2, 3).contiguous()
-    return cost_final, label_context.unsqueeze(0), cost_all, message_vector, message_index
+    cost_final, label_all, blocks, cost_index = TRWPFunction.apply(unary, label_context,
+                                                                   edge_weights, self.args)
+    return (cost_final.permute(0, 1, 4, 2, 3).contiguous(), label_context.unsqueeze(0), label_all,
+            blocks, cost_index)
