@@ -58,6 +58,9 @@ def load():
     getattr(lib, name).restype = ci
   lib.mpl_last_error.restype = ctypes.c_char_p
   _lib = lib
+  policy = os.environ.get("MPLAYERS_PACKED_SCANS")  # 0 | 1 | 2, see mpl_set_option
+  if policy is not None:
+    check(lib.mpl_set_option(OPT_PACKED_SCANS, int(policy)), "set_option")
   return lib
 
 
