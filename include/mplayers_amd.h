@@ -47,7 +47,7 @@ typedef struct mpl_shape {
 /* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.
  * msg: initial messages in, final normalised messages out.  msg_min_index/msg_norm_index NULL =>
  * inference (no index stores).  label_all NULL => no per-iteration labels.  unary_update: scratch
- * plane (holds the running belief).  cost_final doubles as scratch until the final aggregation. */
+ * plane (carries the running belief during the call).  cost_final doubles as scratch until the final aggregation. */
 int mpl_trwp_forward(const mpl_shape* shape, float rho, int n_iter, int enable_min_a_dir,
                      const float* unary, const float* context, const float* edge_weights,
                      float* msg, float* cost_final, uint8_t* msg_min_index,

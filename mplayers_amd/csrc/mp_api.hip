@@ -633,6 +633,7 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
     for (int d = 0; d < s->n_dir; ++d) {  // Gauss-Seidel over directions: TRWP_forward.cu:440-518
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
       p.first_iter = (it == 0);
+      p.skip_s_store = (it == n_iter - 1) && (d == s->n_dir - 1);  // cost_final is re-summed
       if (train) {
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
         p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
@@ -756,7 +757,9 @@ int mpl_trwp_backward(const mpl_shape* s, float rho, int n_iter, const float* co
       p.a_in = first ? dcost_final : dunary;  // CostAggregateKernelBack: every g_k starts as dcost
       p.first_touch = (it == n_iter - 1) && (d & 1);
       p.inv_from_a = (d & 1) ? 0 : 1;  // the launch before an even direction swept d + 1 = d ^ 1
-      p.skip_hd_store = (d & 1) ? 1 : 0;
+      // in the last iteration walked (it == 0) the even sweeps leave h planes nobody reads again
+      p.skip_hd_store = ((d & 1) || it == 0) ? 1 : 0;
+      p.skip_hi_store = (!(d & 1) && it == 0) ? 1 : 0;
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       launch_bwd(p, false, st);

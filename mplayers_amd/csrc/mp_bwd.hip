@@ -340,9 +340,10 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
         }
         buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, an);
         // h_dir = -A is only read by the next launch when that one sweeps the opposite
-        // direction, which derives it from A instead: nothing is stored then
+        // direction, which derives it from A instead: nothing is stored then (nor after the last
+        // sweeps of the pass, whose h planes nobody reads)
         buf_store<R, VEC>(make_rsrc(bHd, p.skip_hd_store ? 0 : nrec), foff, so, hdn);
-        buf_store<R, VEC>(make_rsrc(bHi, nrec), foff, so, hin);
+        buf_store<R, VEC>(make_rsrc(bHi, p.skip_hi_store ? 0 : nrec), foff, so, hin);
       }
       // each pixel receives over exactly one edge per direction: plain read-modify-write
       __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,

@@ -354,6 +354,7 @@ struct SweepParams {
   uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
   int pack;                        // packed scans (mp_pack.hip): chains per wavefront
+  int skip_s_store;                // Gauss-Seidel: last sweep of the call, nobody reads S after it
   int first_iter;                  // Gauss-Seidel: first iteration (planes not yet swept hold the
                                    // caller's initial messages, which need not be read when zero)
   int u_pair_share;                // Jacobi: directions d and d^1 read the U plane of the even one
@@ -373,7 +374,8 @@ struct BackParams {
   float* h;                 // (n_dir_total, N) planes h_k
   int first_touch;          // h_dir and h_inv have not been written yet: read as zero
   int inv_from_a;           // h_inv == -A (the previous launch swept the opposite direction)
-  int skip_hd_store;        // the next launch sweeps the opposite direction and overwrites h_dir
+  int skip_hd_store;        // h_dir is not read again before it is overwritten (or ever)
+  int skip_hi_store;        // h_inv is never read again (last sweeps of the backward pass)
   // ISGMR: gu_in planes (plane stride gu_stride; 0 on the first iteration where gu_k = dcost_final),
   // du_out (n_dir_total, N) receives dU_d in place of gu_d
   const float* gu_in;

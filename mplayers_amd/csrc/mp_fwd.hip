@@ -361,7 +361,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       const unsigned so = sp * (unsigned)vbytes;
       const int nrec = live ? (int)(so + (unsigned)vbytes) : 0;  // nothing is stored past the end
       buf_store<R, VEC>(make_rsrc(bMo, nrec), foff, so, m);
-      if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, nrec), foff, so, sn);
+      if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, p.skip_s_store ? 0 : nrec), foff, so, sn);
       if (TRAIN) {
         const unsigned sob = sp * (unsigned)L;
         buf_store_u8<R, VEC>(make_rsrc(bImin, live ? (int)(sob + (unsigned)L) : 0), lab0, sob, fd_idx);

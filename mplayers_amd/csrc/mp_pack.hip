@@ -149,7 +149,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
   const rsrc_t dMd = make_rsrc(p.msg_in + (int64_t)dir * N, (JACOBI || md_zero) ? 0 : plane_bytes);
   const rsrc_t dMi = make_rsrc(p.msg_in + (int64_t)(dir ^ 1) * N, (JACOBI || mi_zero) ? 0 : plane_bytes);
   const rsrc_t dMo = make_rsrc(p.msg_out + (int64_t)dir * N, plane_bytes);
-  const rsrc_t dSo = make_rsrc(JACOBI ? nullptr : p.belief_out, JACOBI ? 0 : plane_bytes);
+  const rsrc_t dSo = make_rsrc(JACOBI ? nullptr : p.belief_out, (JACOBI || p.skip_s_store) ? 0 : plane_bytes);
   const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P, (int)(P * 4));
   const rsrc_t dImin = make_rsrc(TRAIN ? p.idx_min + (int64_t)dir * N : nullptr, TRAIN ? (int)N : 0);
   const rsrc_t dInorm = make_rsrc(TRAIN ? p.idx_norm + (int64_t)dir * P : nullptr, TRAIN ? (int)P : 0);
@@ -285,7 +285,7 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
   const rsrc_t dHdIn = make_rsrc(hbase + (int64_t)dir * N, read_h ? plane_bytes : 0);
   const rsrc_t dHiIn = make_rsrc(hbase + (int64_t)(dir ^ 1) * N, (read_h && !inv_from_a) ? plane_bytes : 0);
   const rsrc_t dHdOut = make_rsrc(hbase + (int64_t)dir * N, (JACOBI || p.skip_hd_store) ? 0 : plane_bytes);
-  const rsrc_t dHiOut = make_rsrc(hbase + (int64_t)(dir ^ 1) * N, JACOBI ? 0 : plane_bytes);
+  const rsrc_t dHiOut = make_rsrc(hbase + (int64_t)(dir ^ 1) * N, (JACOBI || p.skip_hi_store) ? 0 : plane_bytes);
   const rsrc_t dImin = make_rsrc(p.idx_min + (int64_t)dir * N, (int)N);
   const rsrc_t dInorm = make_rsrc(p.idx_norm + (int64_t)dir * P, (int)P);
   const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P, (int)(P * 4));
