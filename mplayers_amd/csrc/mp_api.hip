@@ -633,6 +633,7 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
     for (int d = 0; d < s->n_dir; ++d) {  // Gauss-Seidel over directions: TRWP_forward.cu:440-518
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
       p.first_iter = (it == 0);
+      p.pair_q = 1;
       p.skip_s_store = (it == n_iter - 1) && (d == s->n_dir - 1);  // cost_final is re-summed
       if (train) {
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;

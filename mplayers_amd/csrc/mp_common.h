@@ -354,6 +354,7 @@ struct SweepParams {
   uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
   int pack;                        // packed scans (mp_pack.hip): chains per wavefront
+  int pair_q;                      // Gauss-Seidel: belief plane holds Q between the sweeps of a pair
   int skip_s_store;                // Gauss-Seidel: last sweep of the call, nobody reads S after it
   int first_iter;                  // Gauss-Seidel: first iteration (planes not yet swept hold the
                                    // caller's initial messages, which need not be read when zero)

@@ -218,6 +218,14 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // not been swept yet, and neither has the opposite one when this direction is the even one
   const bool md_zero = !JACOBI && p.first_iter && desc.msg_nonzero == 0;
   const bool mi_zero = md_zero && (dir & 1) == 0;
+  // Gauss-Seidel pairs (p.pair_q): between the sweep of an even direction and the sweep of its
+  // opposite the belief plane holds Q = S - m_dir - m_inv, which neither sweep changes:
+  //   first sweep  (even):  reads S, m_dir, m_inv; stores m_dir' and Q
+  //   second sweep (odd):   reads Q and m_inv (= m_even'), not its own old messages:
+  //                         S - m_dir = Q + m_inv;  stores m_dir' and S = Q + m_inv + m_dir'
+  // (at a chain start, where no message is written, the plane is converted with the old values)
+  const bool pair_first = !JACOBI && p.pair_q && (dir & 1) == 0;
+  const bool pair_second = !JACOBI && p.pair_q && (dir & 1) == 1;
   // loads of the next pixel; past the end of the chain the last pixel is fetched again
   const int last_p = ch.pix0 + (n - 1) * ch.pstep;
   int ld_p = ch.pix0;
@@ -230,7 +238,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
     if (!JACOBI) {
       // planes that still hold all-zero initial messages are read through an empty descriptor
-      buf_load<R, VEC>(make_rsrc(bMd, md_zero ? 0 : nrec), foff, so, r.md);
+      buf_load<R, VEC>(make_rsrc(bMd, (md_zero || (pair_second && ld_t > 0)) ? 0 : nrec), foff, so,
+                       r.md);
       buf_load<R, VEC>(make_rsrc(bMi, mi_zero ? 0 : nrec), foff, so, r.mi);
     }
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
@@ -244,12 +253,23 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   float prev[R], uf[R];
   {
     const PixF<R> p0 = load_next();
+    float conv[R];  // the start pixel's belief-plane value in the other representation
+#pragma unroll
+    for (int j = 0; j < R; ++j) conv[j] = 0.f;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
       prev[j] = 0.f;
       float un = p0.s[j];
-      if (!JACOBI) un = fmaf(p0.s[j] - p0.md[j], rho, -p0.mi[j]);
+      if (!JACOBI) {
+        const float t0 = pair_second ? p0.s[j] + p0.mi[j] : p0.s[j] - p0.md[j];
+        un = fmaf(t0, rho, -p0.mi[j]);
+        conv[j] = pair_second ? t0 + p0.md[j] : t0 - p0.mi[j];
+      }
       uf[j] = valid[j] ? un : inf;
+    }
+    if (!JACOBI && p.pair_q && !p.skip_s_store) {
+      const unsigned so = (unsigned)ch.pix0 * (unsigned)vbytes;
+      buf_store<R, VEC>(make_rsrc(bSo, (int)(so + (unsigned)vbytes)), foff, so, conv);
     }
     if (JACOBI) {
       float z[R];
@@ -284,7 +304,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       for (int j = 0; j < R; ++j) {
         float x = px.s[j];
         if (!JACOBI) {
-          tt[j] = px.s[j] - px.md[j];       // unary + the other directions' messages
+          // unary + the other directions' messages
+          tt[j] = pair_second ? px.s[j] + px.mi[j] : px.s[j] - px.md[j];
           x = fmaf(tt[j], rho, -px.mi[j]);  // UpdateUnaryKernel, TRWP_forward.cu:70-78
         } else {
           tt[j] = 0.f;
@@ -353,7 +374,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
 #pragma unroll
       for (int j = 0; j < R; ++j) {
         m[j] = v[j] - nmin;  // MsgNormNaive, commonCUDA.cuh:126-128
-        sn[j] = tt[j] + m[j];
+        sn[j] = pair_first ? tt[j] - px.mi[j] : tt[j] + m[j];
         prev[j] = valid[j] ? m[j] : 0.f;
         uf[j] = un[j];
       }
@@ -385,7 +406,7 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
   const int lane = threadIdx.x;
   const int L = p.L;
   const ChainCtx ch = locate_chain(p);
-  if (!JACOBI && ch.n < 2) return;  // nothing to write
+  if (!JACOBI && !p.pair_q && ch.n < 2) return;  // nothing to write
 
   CtxDesc desc;
   if (p.desc != nullptr) {

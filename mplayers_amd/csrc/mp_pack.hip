@@ -136,7 +136,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
   const Seg sg = make_seg(lane, L, G);
   fill_table(p.ctx, L, p.ctx2d, lane, tab);
   __syncthreads();
-  if (!JACOBI && ch.n_max < 2) return;
+  if (!JACOBI && !p.pair_q && ch.n_max < 2) return;
 
   const int64_t P = (int64_t)p.B * p.H * p.W;
   const int64_t N = P * L;
@@ -144,9 +144,13 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
   const int plane_bytes = (int)(N * 4);
   const bool md_zero = !JACOBI && p.first_iter && p.desc != nullptr && p.desc->msg_nonzero == 0;
   const bool mi_zero = md_zero && (dir & 1) == 0;
+  const bool pair_first = !JACOBI && p.pair_q && (dir & 1) == 0;   // see mp_fwd.hip
+  const bool pair_second = !JACOBI && p.pair_q && (dir & 1) == 1;
   const int udir = p.u_pair_share ? (dir & ~1) : dir;
   const rsrc_t dS = make_rsrc(JACOBI ? p.msg_in + (int64_t)udir * N : p.belief, plane_bytes);
   const rsrc_t dMd = make_rsrc(p.msg_in + (int64_t)dir * N, (JACOBI || md_zero) ? 0 : plane_bytes);
+  const rsrc_t dMdRing = make_rsrc(p.msg_in + (int64_t)dir * N,
+                                   (JACOBI || md_zero || pair_second) ? 0 : plane_bytes);
   const rsrc_t dMi = make_rsrc(p.msg_in + (int64_t)(dir ^ 1) * N, (JACOBI || mi_zero) ? 0 : plane_bytes);
   const rsrc_t dMo = make_rsrc(p.msg_out + (int64_t)dir * N, plane_bytes);
   const rsrc_t dSo = make_rsrc(JACOBI ? nullptr : p.belief_out, (JACOBI || p.skip_s_store) ? 0 : plane_bytes);
@@ -172,7 +176,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
     const unsigned eo = act ? (unsigned)(ld_pix * L + l) * 4u : (unsigned)kDeadOffset;
     r.s = ldf(dS, eo);
     if (!JACOBI) {
-      r.md = ldf(dMd, eo);
+      r.md = ldf(ld_t == 0 ? dMd : dMdRing, eo);
       r.mi = ldf(dMi, eo);
     } else {
       r.md = r.mi = 0.f;
@@ -187,8 +191,12 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
   float prev = 0.f, uf;
   {
     const PixPF p0 = load_next();
-    const float un = JACOBI ? p0.s : fmaf(p0.s - p0.md, rho, -p0.mi);
+    const float t0 = pair_second ? p0.s + p0.mi : p0.s - p0.md;
+    const float un = JACOBI ? p0.s : fmaf(t0, rho, -p0.mi);
     uf = on ? un : inf;
+    if (!JACOBI && p.pair_q)  // convert the belief plane at the chain start as well
+      stf(dSo, (on && n >= 1) ? (unsigned)(ch.pix0 * L + l) * 4u : (unsigned)kDeadOffset,
+          pair_second ? t0 + p0.md : t0 - p0.mi);
     if (JACOBI)  // the buffers alternate: the chain start is written with the zeros it keeps
       stf(dMo, (on && n >= 1) ? (unsigned)(ch.pix0 * L + l) * 4u : (unsigned)kDeadOffset, 0.f);
   }
@@ -208,7 +216,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
       wait_vmem<(D - 1) * kOps>();
       const PixPF px = ring[u];
       ring[u] = load_next();
-      const float tt = px.s - px.md;
+      const float tt = pair_second ? px.s + px.mi : px.s - px.md;
       const float x = JACOBI ? px.s : fmaf(tt, rho, -px.mi);  // UpdateUnaryKernel, :70-78
       const float un = on ? x : inf;
       const float w = px.w;
@@ -239,7 +247,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
       uf = un;
       const unsigned eo = live ? (unsigned)(st_pix * L + l) * 4u : (unsigned)kDeadOffset;
       stf(dMo, eo, m);
-      if (!JACOBI) stf(dSo, eo, tt + m);
+      if (!JACOBI) stf(dSo, eo, pair_first ? tt - px.mi : tt + m);
       if (TRAIN) {
         __builtin_amdgcn_raw_buffer_store_b8((unsigned char)arg, dImin,
                                              live ? st_pix * L + l : kDeadOffset, 0, MPL_ST_AUX);
