@@ -63,3 +63,34 @@ def test_random_case(gpu, oracle, seed):
   for name, g, r in (("dunary", gu, du), ("dcontext", gc, dc), ("dedge", ge, de)):
     err = np.abs(g.astype(np.float64) - r).max()
     assert err <= 1e-4 * max(1.0, np.abs(r).max()), (name, err)
+
+
+@pytest.mark.parametrize("mode,rho", [("ISGMR", 0.7), ("ISGMR", 0.5), ("TRWP", 1.0), ("TRWP", 0.3)])
+@pytest.mark.parametrize("L,n_dir", [(21, 8), (96, 4), (7, 16)])
+def test_other_rho_values(gpu, oracle, mode, rho, L, n_dir):
+  """The nn.Module fixes rho (0.5 for TRWP, 1 for ISGMR) but the operators take any value; ISGMR
+  shares planes between opposite directions only at rho == 1, so other values take other paths."""
+  rng = np.random.default_rng(int(rho * 100) + L)
+  B, H, W, n_iter = 2, 6, 7, 3
+  k = np.arange(L, dtype=np.float32)
+  ctx = np.triu(rng.random((L, L)), 1).astype(np.float32) if L == 21 else \
+      (0.3 * np.minimum(k, 3)).astype(np.float32)
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ew = (0.1 + rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  dcost = rng.standard_normal((B, 1, H, W, L)).astype(np.float32)
+  ref = oracle.forward(mode, unary, ctx, ew, n_dir, n_iter, rho, want_gaps=True)
+  got = gpu.gpu_forward(mode, unary, ctx, ew, n_dir, n_iter, rho)
+  belief = ref["cost_final"]
+  tol = 1e-5 * max(1.0, float(np.abs(belief).max()))
+  gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=belief)
+  gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost")
+  gpu.assert_indices_match_off_ties(got["msg_min_index"], ref["msg_min_index"], ref["gap_min"],
+                                    4 * tol, "min index")
+  du, dc, de = oracle.backward(mode, ctx.astype(np.float64), ew.astype(np.float64),
+                               dcost.astype(np.float64), ref["msg_min_index"],
+                               ref["msg_norm_index"], rho)
+  gu, gc, ge = gpu.gpu_backward(mode, ctx, ew, dcost, ref["msg_min_index"], ref["msg_norm_index"],
+                                rho, garbage_scratch=True)
+  for name, g, r in (("dunary", gu, du), ("dcontext", gc, dc), ("dedge", ge, de)):
+    err = np.abs(g.astype(np.float64) - r).max()
+    assert err <= 1e-4 * max(1.0, np.abs(r).max()), (name, err)
