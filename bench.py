@@ -58,6 +58,9 @@ def parse():
   ap.add_argument("--edge-probe", action="store_true",
                   help="also time the edge-weight producer on an image of the workload's size "
                        "(reported under \"edge_weights\")")
+  ap.add_argument("--terms-probe", action="store_true",
+                  help="also time the stereo data cost of an image pair of the workload's size and "
+                       "the energies of n_iter labellings (reported under \"mrf_terms\")")
   return ap.parse_args()
 
 
@@ -171,6 +174,35 @@ def edge_probe(B, H, W, n_dir, dev, channels=3, reps=20):
   nbytes = B * channels * H * W * 4 * (1 + n_dir)
   return {"mode": "edge_net", "image": [B, channels, H, W], "n_dirs": n_dir, "ms": ms,
           "algorithmic_GBs": nbytes / (ms * 1e-3) / 1e9,
+          "note": "wall time per call including the allocation of the result"}
+
+
+def terms_probe(H, W, L, n_dir, n_iter, dev, reps=10):
+  """Stereo data cost of a 3-band H x W pair for L disparities (writes the (H, W, L) fp32 volume
+  the layers take as unary) and the energies of n_iter labellings of it."""
+  import torch
+  from mplayers_amd import compute_terms
+  left = torch.randint(0, 256, (H, W, 3), dtype=torch.uint8, device=dev)
+  right = torch.roll(left, -5, dims=1)
+  labels = torch.randint(0, L, (n_iter, 1, H, W), dtype=torch.uint8, device=dev)
+  context = torch.arange(L, dtype=torch.float32, device=dev).clamp(max=3)
+
+  def timed(fn):
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+      fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps * 1e3
+
+  cost = compute_terms.stereo_data_cost(left, right, L)
+  ms_cost = timed(lambda: compute_terms.stereo_data_cost(left, right, L))
+  unary = cost.view(1, H, W, L)
+  ms_energy = timed(lambda: compute_terms.mrf_energy(unary, context, labels, None, n_dir))
+  return {"image": [H, W, 3], "n_disp": L,
+          "data_cost_ms": ms_cost, "data_cost_written_GBs": H * W * L * 4 / (ms_cost * 1e-3) / 1e9,
+          "energy_labellings": n_iter, "energy_ms": ms_energy,
           "note": "wall time per call including the allocation of the result"}
 
 
@@ -325,6 +357,8 @@ def main():
     out["module_surface"] = module_probe(cfg, algs, unary, edge, dcost)
   if a.edge_probe:
     out["edge_weights"] = edge_probe(B, H, W, n_dir, dev)
+  if a.terms_probe:
+    out["mrf_terms"] = terms_probe(H, W, L, n_dir, n_iter, dev)
   if not a.no_cpu_baseline:
     out["cpu_baseline"] = cpu_baseline(cfg)
   print(json.dumps(out))

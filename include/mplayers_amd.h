@@ -168,6 +168,38 @@ int mpl_edge_shift(int mode, const float* image, int batch, int channels, int he
                    int n_dirs, float sigma, float threshold, float penalty, float* out,
                    double* dir_sums, void* stream);
 
+/* Stereo data term, the layers' upstream in the reference's energy-minimisation driver: replaces
+ * computeDSI (MPLayers/aux/aux.cpp:5-98) as called by compute_all_terms
+ * (MPLayers/aux/auxPy.cpp:22,62-66: birchfield = 1, squared_diffs = 0, trunc_diffs = 255).
+ * left/right: device images, (H, W, bands) uint8, interleaved; the first min(3, bands) bands are
+ * compared.  data_cost (H, W, n_labels) fp32, fully written: the matching cost of pixel (y, x)
+ * with (y, x - d) of the right image, summed over the colour bands and truncated at
+ * colours * |trunc_diffs| (trunc_diffs^2 for squared differences); matches outside the image cost
+ * min(colours * 255 [* 255], truncation).  Integer arithmetic, exact. */
+int mpl_stereo_data_cost(const uint8_t* left, const uint8_t* right, int height, int width,
+                         int bands, int n_labels, int birchfield, int squared_diffs,
+                         int trunc_diffs, float* data_cost, void* stream);
+
+/* Gradient cues of the same driver: replaces computeCues (MPLayers/aux/aux.cpp:100-170) and the
+ * re-packing of MPLayers/aux/auxPy.cpp:83-99.  h_cue (H, W-1) and v_cue (W, H-1) fp32 hold
+ * grad_penalty where the summed squared colour difference to the right / lower neighbour is below
+ * colours * grad_thresh^2, else 1. */
+int mpl_gradient_cues(const uint8_t* image, int height, int width, int bands, int grad_thresh,
+                      float grad_penalty, float* h_cue, float* v_cue, void* stream);
+
+/* Energy of labellings, the layers' downstream in the same driver: replaces calEnergy
+ * (tools/matlab/MRF/calEnergy.m:2-48), generalised from the 4-connected grid to the layers'
+ * direction table and to their edge weights.  labels (n_labelings, batch, H, W) uint8 (for
+ * instance the label_all output of a forward call); unary, context, edge_weights (may be NULL:
+ * all ones) as in mpl_trwp_forward.  energy (n_labelings, 2) fp64, overwritten:
+ *   energy[i][0] = sum_p unary[p, x_p]
+ *   energy[i][1] = sum over even directions d and pixels p with q = p - r_d inside the image of
+ *                  edge_weights[d, p] * ctx(x_p, x_q)          (every undirected edge once)
+ * accumulated in fp64 with atomics (the order of the partial sums is not fixed). */
+int mpl_mrf_energy(const mpl_shape* shape, int n_labelings, const float* unary,
+                   const float* context, const float* edge_weights, const uint8_t* labels,
+                   double* energy, void* stream);
+
 /* Message of the last failed call on this thread ("" if none). */
 const char* mpl_last_error(void);
 
