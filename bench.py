@@ -49,8 +49,9 @@ def parse():
                   help="also run one plain device copy of one fp32 plane (reference point for "
                        "hardware byte counters)")
   ap.add_argument("--peak-probe", action="store_true",
-                  help="also time plain device copy / add / fill kernels on one fp32 plane of the "
-                       "workload (reported under \"measured_stream_rates\")")
+                  help="also time the library's copy probes on planes of the workload's size: one-pass "
+                       "streaming kernels and scan-shaped kernels (one long-lived wavefront per row "
+                       "or column) for several read:write mixes (\"measured_stream_rates\")")
   ap.add_argument("--module-probe", action="store_true",
                   help="also time forward+backward through the nn.Module surface, which allocates "
                        "its buffers on every call as the reference's does (reported under "
@@ -105,24 +106,38 @@ def cpu_baseline(cfg, budget_s=15.0):
                     "%.1f s" % (mode, rows, W, cfg["name"], L, n_dir, dt)}
 
 
-def peak_probe(dst, src, reps=10):
-  """What this GPU sustains for plain streaming kernels on tensors of the workload's plane size:
-  copy (1 read + 1 write), add (2 reads + 1 write), fill (1 write); GB/s of bytes moved."""
+def peak_probe(H, W, L, dev, reps=5):
+  """What this GPU sustains on planes of the workload's size, in GB/s of bytes moved: one-pass
+  streaming kernels (the shape of the element-wise passes) and long-lived one-wavefront-per-chain
+  kernels that move n_in planes in and n_out planes out pixel by pixel (the shape of the scans,
+  without their arithmetic): mpl_probe_copy."""
+  import ctypes
   import torch
-  nbytes = dst.numel() * 4
-  other = torch.empty_like(dst)
-  res = {}
-  for name, fn, moved in (("copy", lambda: other.copy_(src), 2 * nbytes),
-                          ("add", lambda: torch.add(src, dst, out=other), 3 * nbytes),
-                          ("fill", lambda: other.zero_(), nbytes)):
-    fn()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(reps):
-      fn()
-    torch.cuda.synchronize()
-    res[name + "_GBs"] = moved * reps / (time.perf_counter() - t0) / 1e9
-  res["plane_bytes"] = nbytes
+  from mplayers_amd import _lib
+  if L % 4:
+    return {"note": "the probe needs a label count that is a multiple of 4"}
+  lib = _lib.load()
+  n = H * W * L
+  src = torch.zeros(4 * n, dtype=torch.float32, device=dev)
+  dst = torch.empty(3 * n, dtype=torch.float32, device=dev)
+  stream = torch.cuda.current_stream().cuda_stream
+  res = {"plane_bytes": 4 * n}
+  start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  for shape, sname in ((2, "stream"), (0, "rows"), (1, "columns")):
+    for n_in, n_out in ((1, 1), (3, 0), (1, 3), (3, 2), (4, 3)):
+      def run():
+        _lib.check(lib.mpl_probe_copy(shape, n_in, n_out, ctypes.c_void_p(src.data_ptr()),
+                                      ctypes.c_void_p(dst.data_ptr()), H, W, L,
+                                      ctypes.c_void_p(stream)), "probe_copy")
+      run()
+      torch.cuda.synchronize()
+      start.record()
+      for _ in range(reps):
+        run()
+      stop.record()
+      torch.cuda.synchronize()
+      ms = start.elapsed_time(stop) / reps
+      res["%s_%din_%dout_GBs" % (sname, n_in, n_out)] = round((n_in + n_out) * 4 * n / ms / 1e6, 1)
   return res
 
 
@@ -352,7 +367,7 @@ def main():
 
   }
   if a.peak_probe:
-    out["measured_stream_rates"] = peak_probe(cost, unary)
+    out["measured_stream_rates"] = peak_probe(H, W, L, dev)
   if a.module_probe and training:
     out["module_surface"] = module_probe(cfg, algs, unary, edge, dcost)
   if a.edge_probe:

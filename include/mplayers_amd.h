@@ -200,6 +200,18 @@ int mpl_mrf_energy(const mpl_shape* shape, int n_labelings, const float* unary,
                    const float* context, const float* edge_weights, const uint8_t* labels,
                    double* energy, void* stream);
 
+/* Bandwidth probe (diagnostic, no counterpart in the reference): moves n_in planes of
+ * (height, width, n_labels) fp32 from `in` to n_out planes at `out` (sum of the inputs, + k for
+ * plane k) in the scans' access shape -- one long-lived wavefront per row (MPL_PROBE_ROWS) or per
+ * column (MPL_PROBE_COLUMNS), one pixel vector per step, eight pixels in flight -- or as a one-pass
+ * streaming kernel (MPL_PROBE_STREAM).  `in` holds n_in planes, `out` max(n_out, 1); (n_in, n_out)
+ * is one of (1,1) (1,3) (3,0) (3,2) (4,3); n_labels a multiple of 4. */
+#define MPL_PROBE_ROWS 0
+#define MPL_PROBE_COLUMNS 1
+#define MPL_PROBE_STREAM 2
+int mpl_probe_copy(int shape, int n_in, int n_out, const float* in, float* out, int height,
+                   int width, int n_labels, void* stream);
+
 /* Message of the last failed call on this thread ("" if none). */
 const char* mpl_last_error(void);
 

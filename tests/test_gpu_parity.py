@@ -201,3 +201,37 @@ def test_min_a_dir_and_initial_messages(gpu, oracle):
   ref = oracle.forward("TRWP", unary, ctx, None, n_dir, 2, 0.5)
   got = gpu.gpu_forward("TRWP", unary, ctx, None, n_dir, 1, 0.5, msg_init=first["msg"])
   gpu.assert_values_close(got["msg"], ref["msg"], what="continued msg", belief=ref["cost_final"])
+
+
+@pytest.mark.gpu
+def test_copy_probe_moves_what_it_claims(gpu):
+  """The bandwidth probe's kernels write the sum of their input planes (+ k for output plane k) to
+  every element, whatever the access shape, and reject shapes they do not implement."""
+  import ctypes
+  import torch
+  from mplayers_amd import _lib
+  lib = _lib.load()
+  H, W, L = 13, 21, 44
+  n = H * W * L
+  src = torch.randn(4 * n, device="cuda")
+  stream = torch.cuda.current_stream().cuda_stream
+  for shape in (0, 1, 2):
+    for n_in, n_out in ((1, 1), (1, 3), (3, 2), (4, 3), (3, 0)):
+      dst = torch.full((3 * n,), -7.0, device="cuda")
+      rc = lib.mpl_probe_copy(shape, n_in, n_out, ctypes.c_void_p(src.data_ptr()),
+                              ctypes.c_void_p(dst.data_ptr()), H, W, L, ctypes.c_void_p(stream))
+      assert rc == 0, lib.mpl_last_error()
+      want = src.view(4, n)[0].clone()
+      for k in range(1, n_in):
+        want = want + src.view(4, n)[k]
+      for k in range(3):
+        got = dst.view(3, n)[k]
+        if k < n_out:
+          assert torch.equal(got, want + k), (shape, n_in, n_out, k)
+        else:
+          assert bool((got == -7.0).all()), (shape, n_in, n_out, k)
+  dst = torch.empty(3 * n, device="cuda")
+  args = (ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()))
+  assert lib.mpl_probe_copy(0, 2, 2, *args, H, W, L, ctypes.c_void_p(stream)) != 0
+  assert lib.mpl_probe_copy(3, 1, 1, *args, H, W, L, ctypes.c_void_p(stream)) != 0
+  assert lib.mpl_probe_copy(0, 1, 1, *args, H, W, 42, ctypes.c_void_p(stream)) != 0
