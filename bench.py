@@ -59,6 +59,9 @@ def parse():
   ap.add_argument("--edge-probe", action="store_true",
                   help="also time the edge-weight producer on an image of the workload's size "
                        "(reported under \"edge_weights\")")
+  ap.add_argument("--graph-probe", action="store_true",
+                  help="also capture one step in a HIP graph and time its replays (the library only "
+                       "launches kernels, so a step is capturable; reported under \"graph_replay\")")
   ap.add_argument("--terms-probe", action="store_true",
                   help="also time the stereo data cost of an image pair of the workload's size and "
                        "the energies of n_iter labellings (reported under \"mrf_terms\")")
@@ -374,6 +377,19 @@ def main():
     out["edge_weights"] = edge_probe(B, H, W, n_dir, dev)
   if a.terms_probe:
     out["mrf_terms"] = terms_probe(H, W, L, n_dir, n_iter, dev)
+  if a.graph_probe:
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      step()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+      graph.replay()
+    torch.cuda.synchronize()
+    g_ms = (time.perf_counter() - t0) / a.steps * 1e3
+    out["graph_replay"] = {"ms_per_step": g_ms, "eager_ms_per_step": out["ms_per_step"],
+                           "speedup": out["ms_per_step"] / g_ms}
   if not a.no_cpu_baseline:
     out["cpu_baseline"] = cpu_baseline(cfg)
   print(json.dumps(out))
