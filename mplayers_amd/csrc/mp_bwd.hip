@@ -55,11 +55,15 @@ template <int R, bool VEC, bool MASK, bool JACOBI, bool SMALL>
 __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   extern __shared__ float smem[];
   const int L = p.L;
-  const int n_ctx = p.ctx2d ? L * L : L;
+  // 2-D context tables exist for at most 64 labels, i.e. only with one label per lane
+  const bool ctx2d = (R == 1) && p.ctx2d;
+  const int n_ctx = ctx2d ? L * L : L;
   float* sc_s = smem;              // kMaxL floats: scatter target of the slow path
-  float* g0_s = sc_s + kMaxL;      // kMaxL floats: weighted gradients of popular class 0, by label
-  float* g1_s = g0_s + kMaxL;      // same for class 1
-  float* ctx_s = g1_s + kMaxL;     // context table
+  // weighted gradients of popular class 0 by label, with L zeros on either side so that the
+  // gather at label f +- k needs no range checks: 3 * L floats, data at [L, 2L)
+  float* g0_s = sc_s + kMaxL;
+  float* g1_s = g0_s + 3 * L;      // same for class 1
+  float* ctx_s = g1_s + 3 * L;     // context table
   float* hist_s = ctx_s + n_ctx;   // dcontext accumulator of the slow path (and of 2-D contexts)
   // one label per lane and at most kSmallL labels: the scatter is a loop over source labels and
   // dcontext is accumulated per (cd, fd) pair, each lane owning the row of its label
@@ -76,7 +80,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     ctx_s[i] = p.ctx[i];
     hist_s[i] = 0.f;
   }
-  for (int i = lane; i < 3 * kMaxL; i += kWave) sc_s[i] = 0.f;  // sc_s, g0_s, g1_s
+  for (int i = lane; i < kMaxL + 6 * L; i += kWave) sc_s[i] = 0.f;  // sc_s, g0_s, g1_s
   if (small_l)
     for (int i = lane; i < L * L; i += kWave) pair_s[i] = 0.f;
   __syncthreads();
@@ -193,7 +197,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           if (!valid[0]) g = 0.f;
           // this lane's own pair: dedge and dcontext (TRWP_backward.cu:109-112)
           const int ao = fd > cd ? fd - cd : cd - fd;
-          const int ci = !valid[0] ? 0 : (p.ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
+          const int ci = !valid[0] ? 0 : (ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
           const float de = ctx_s[ci] * g;
           if (valid[0] && cd != fd) pair_s[cd * L + fd] = fmaf(w, g, pair_s[cd * L + fd]);
           // dU[q, f] = sum of g[c] over the labels c that point at f: one source label per trip
@@ -225,13 +229,13 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           const int d = fd - cd;
           const int ao = d < 0 ? -d : d;
           const bool c0 = fd == f0;
-          const bool c1 = (fd == f1) && !c0;
+          const bool c1 = (fd == f1) & !c0;
           p0 += c0 ? gv[j] : 0.f;
           p1 += c1 ? gv[j] : 0.f;
-          off[j] = (c0 || c1) ? kPopular : d;
-          any_left = any_left || (!(c0 || c1) && ao > kNear && valid[j]);
+          off[j] = (c0 | c1) ? kPopular : d;
+          any_left |= !(c0 | c1) & (ao > kNear) & valid[j];
           // dedge_weights[cur] += ctx(cd, fd) * value
-          const int ci = !valid[j] ? 0 : (p.ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
+          const int ci = !valid[j] ? 0 : (ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
           de = fmaf(ctx_s[ci], gv[j], de);
         }
         const float s0sum = wave_sum(p0);
@@ -268,34 +272,29 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           scn[j] = own + tp[j] + tn[j] + (cd == f0 ? s0sum : 0.f) + (cd == f1 ? s1sum : 0.f);
         }
         // dcontext += edge_weight * value where cd != fd (TRWP_backward.cu:111-112)
-        if (!p.ctx2d) {
+        if (!ctx2d) {
 #pragma unroll
           for (int o = 1; o <= kNear; ++o) near_acc[o] = fmaf(w, near_t[o], near_acc[o]);
           // popular classes: bin |cd - f| is reached from labels f + k and f - k; gather through LDS
+          // (bin 0 collects the popular label's own value twice; it is never flushed)
 #pragma unroll
           for (int j = 0; j < R; ++j)
-            if (valid[j]) g0_s[lab0 + j] = (px.fd[j] == f0) ? w * gv[j] : 0.f;
+            if (valid[j]) g0_s[L + lab0 + j] = (px.fd[j] == f0) ? w * gv[j] : 0.f;
           __syncthreads();
 #pragma unroll
           for (int j = 0; j < R; ++j) {
-            const int k = lab0 + j;
-            const int hi_l = f0 + k, lo_l = f0 - k;
-            const float a = (k >= 1 && hi_l < L) ? g0_s[hi_l < L ? hi_l : 0] : 0.f;
-            const float b = (k >= 1 && lo_l >= 0) ? g0_s[lo_l >= 0 ? lo_l : 0] : 0.f;
-            hist_reg[j] += a + b;
+            const int k = valid[j] ? lab0 + j : 0;
+            hist_reg[j] += g0_s[L + f0 + k] + g0_s[L + f0 - k];
           }
           if (f1 != f0) {
 #pragma unroll
             for (int j = 0; j < R; ++j)
-              if (valid[j]) g1_s[lab0 + j] = (px.fd[j] == f1) ? w * gv[j] : 0.f;
+              if (valid[j]) g1_s[L + lab0 + j] = (px.fd[j] == f1) ? w * gv[j] : 0.f;
             __syncthreads();
 #pragma unroll
             for (int j = 0; j < R; ++j) {
-              const int k = lab0 + j;
-              const int hi_l = f1 + k, lo_l = f1 - k;
-              const float a = (k >= 1 && hi_l < L) ? g1_s[hi_l < L ? hi_l : 0] : 0.f;
-              const float b = (k >= 1 && lo_l >= 0) ? g1_s[lo_l >= 0 ? lo_l : 0] : 0.f;
-              hist_reg[j] += a + b;
+              const int k = valid[j] ? lab0 + j : 0;
+              hist_reg[j] += g1_s[L + f1 + k] + g1_s[L + f1 - k];
             }
           }
         } else {
@@ -313,7 +312,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
             const int ao = off[j] < 0 ? -off[j] : off[j];
             if (valid[j] && off[j] != kPopular && ao > kNear) {
               atomicAdd(&sc_s[px.fd[j]], gv[j]);
-              if (!p.ctx2d) atomicAdd(&hist_s[ao], w * gv[j]);
+              if (!ctx2d) atomicAdd(&hist_s[ao], w * gv[j]);
             }
           }
           __syncthreads();
@@ -356,7 +355,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   __syncthreads();
   if (small_l) {
     // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D)
-    if (!p.ctx2d) {
+    if (!ctx2d) {
       if (lane >= 1 && lane < L) {
         float acc = 0.f;
         for (int c = 0; c < L; ++c) {
@@ -378,10 +377,10 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     float v = hist_s[i];
     if (v != 0.f) atomicAdd(&p.dctx[i], v);
   }
-  if (!p.ctx2d) {
+  if (!ctx2d) {
 #pragma unroll
     for (int j = 0; j < R; ++j)
-      if (valid[j] && hist_reg[j] != 0.f) atomicAdd(&p.dctx[lab0 + j], hist_reg[j]);
+      if (valid[j] && lab0 + j >= 1 && hist_reg[j] != 0.f) atomicAdd(&p.dctx[lab0 + j], hist_reg[j]);
 #pragma unroll
     for (int k = 1; k <= kNear; ++k) {
       const float v = wave_sum(near_acc[k]);
@@ -393,7 +392,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 template <int R, bool VEC, bool MASK>
 void launch_vm(const BackParams& p, bool jacobi, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
-  const size_t lds = sizeof(float) * (3 * kMaxL + 2 * (p.ctx2d ? p.L * p.L : p.L) +
+  const size_t lds = sizeof(float) * (kMaxL + 6 * p.L + 2 * (p.ctx2d ? p.L * p.L : p.L) +
                                       ((R == 1 && p.L <= kSmallL) ? p.L * p.L : 0));
   if constexpr (R == 1) {
     if (p.L <= kSmallL) {
