@@ -85,6 +85,18 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     for (int i = lane; i < L * L; i += kWave) pair_s[i] = 0.f;
   __syncthreads();
 
+  // Offsets |fd - cd| come from the band of the context (entries below its constant tail) or from
+  // the far candidate, which is nearly always one of the popular targets.  A 1-D context with a
+  // band of K entries therefore needs label shifts up to K - 1 only; rarer offsets within kNear
+  // fall through to the slow path, so any choice here is exact.
+  int near_max = kNear;
+  if (!ctx2d && !small_l) {
+    int kb = 0;
+    for (int i = lane; i < L; i += kWave) kb = (ctx_s[i] != ctx_s[L - 1]) ? i + 1 : kb;
+    kb = (int)-wave_min(-(float)kb);  // wave maximum: entries at and beyond kb equal the last one
+    near_max = kb - 1 < 1 ? 1 : (kb - 1 > kNear ? kNear : kb - 1);
+  }
+
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t img_p = (int64_t)ch.bv * HW;  // first pixel of this batch item
   const int64_t img_e = img_p * L;
@@ -233,7 +245,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           p0 += c0 ? gv[j] : 0.f;
           p1 += c1 ? gv[j] : 0.f;
           off[j] = (c0 | c1) ? kPopular : d;
-          any_left |= !(c0 | c1) & (ao > kNear) & valid[j];
+          any_left |= !(c0 | c1) & (ao > near_max) & valid[j];
           // dedge_weights[cur] += ctx(cd, fd) * value
           const int ci = !valid[j] ? 0 : (ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
           de = fmaf(ctx_s[ci], gv[j], de);
@@ -247,6 +259,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
         for (int o = kNear; o >= 1; --o) {
           near_t[o] = 0.f;
+          if (o > near_max) continue;  // wave-uniform
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             const float cp = (off[j] == o) ? gv[j] : 0.f;
@@ -310,7 +323,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             const int ao = off[j] < 0 ? -off[j] : off[j];
-            if (valid[j] && off[j] != kPopular && ao > kNear) {
+            if (valid[j] && off[j] != kPopular && ao > near_max) {
               atomicAdd(&sc_s[px.fd[j]], gv[j]);
               if (!ctx2d) atomicAdd(&hist_s[ao], w * gv[j]);
             }
