@@ -251,7 +251,9 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           de = fmaf(ctx_s[ci], gv[j], de);
         }
         const float s0sum = wave_sum(p0);
-        const float s1sum = wave_sum(p1);
+        // nothing belongs to the second class when both popular targets coincide (the usual case)
+        float s1sum = 0.f;
+        if (f1 != f0) s1sum = wave_sum(p1);
         // near targets: sc_next[l] += g[l - o] where index(l - o) == l, |o| <= kNear
         float tp[R], tn[R], near_t[kNear + 1];
 #pragma unroll
