@@ -59,6 +59,10 @@ def parse():
   ap.add_argument("--edge-probe", action="store_true",
                   help="also time the edge-weight producer on an image of the workload's size "
                        "(reported under \"edge_weights\")")
+  ap.add_argument("--caller-clears-messages", action="store_true",
+                  help="the reference's contract: the step zero-fills `msg` and the operators read "
+                       "it as initial messages (default: msg_uninit=1, the library starts the "
+                       "messages at zero itself and the step does not touch `msg` beforehand)")
   ap.add_argument("--graph-probe", action="store_true",
                   help="also capture one step in a HIP graph and time its replays (the library only "
                        "launches kernels, so a step is capturable; reported under \"graph_replay\")")
@@ -268,10 +272,13 @@ def main():
   else:
     imin = inorm = empty
 
+  uninit = not a.caller_clears_messages
+
   def step():
     for alg in algs:
       rho = 1.0 if alg == "ISGMR" else 0.5
-      msg.zero_()
+      if alg == "SOFT" or not uninit:
+        msg.zero_()
       if alg == "SOFT":
         lib_stereo.TRWP_hard_soft.forward_soft(rho, n_iter, unary, context, edge, msg, soft_blocks,
                                                inorm, cost, belief, empty)
@@ -280,13 +287,13 @@ def main():
                                                   dunary, dctx, dedge, dmsg, dscratch)
       elif alg == "TRWP":
         lib_stereo.TRWP.forward(rho, n_iter, 0, unary, context, edge, msg, cost, imin, inorm,
-                                belief, empty)
+                                belief, empty, msg_uninit=uninit)
         if training:
           lib_stereo.TRWP.backward(rho, context, edge, dcost, imin, inorm, dunary, dctx, dedge,
                                    dmsg, dscratch)
       else:
         lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, context, edge, msg, cost, imin, inorm,
-                                 belief, msg_tmp, empty)
+                                 belief, msg_tmp, empty, msg_uninit=uninit)
         if training:
           lib_stereo.ISGMR.backward(0, rho, context, edge, dcost, imin, inorm, dunary, dctx,
                                     dedge, dmsg, dscratch, dmsg_tmp)
@@ -360,7 +367,10 @@ def main():
                              "iterations" % (cfg["name"], "+".join(algs),
                                              "fwd+bwd" if training else "fwd", B, H, W, L, n_dir,
                                              n_iter),
-                 "scale": a.scale},
+                 "scale": a.scale,
+                 "initial_messages": ("zero by declaration (msg_uninit): the library writes every "
+                                      "element itself" if uninit else
+                                      "tensor cleared by the caller inside the timed step")},
       "roofline": roofline,
       "whole_step_frac_of_hbm_roofline": whole,
       "contract_bytes_per_unit": contract,

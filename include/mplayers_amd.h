@@ -42,6 +42,10 @@ typedef struct mpl_shape {
   int width;
   int n_disp; /* labels, <= MPL_MAX_LABELS */
   int ctx2d;  /* 1: (L,L) context table (the reference selects it by n_disp == 21); needs L <= 64 */
+  int msg_uninit; /* forward calls only.  0: `msg` holds the initial messages (the reference's
+               * contract: the caller zero-fills it).  1: the contents of `msg` on entry are
+               * ignored; the messages start at zero and the library writes every element itself,
+               * which saves the caller's memset and the passes that would read the zeros back */
 } mpl_shape;
 
 /* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.

@@ -18,7 +18,8 @@ KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combi
 class Shape(ctypes.Structure):
   """struct mpl_shape"""
   _fields_ = [("n_dir", ctypes.c_int), ("batch", ctypes.c_int), ("height", ctypes.c_int),
-              ("width", ctypes.c_int), ("n_disp", ctypes.c_int), ("ctx2d", ctypes.c_int)]
+              ("width", ctypes.c_int), ("n_disp", ctypes.c_int), ("ctx2d", ctypes.c_int),
+              ("msg_uninit", ctypes.c_int)]
 
 
 class KernelStat(ctypes.Structure):

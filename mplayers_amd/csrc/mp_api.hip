@@ -501,7 +501,21 @@ SweepParams base_fwd_params(const mpl_shape* s, float rho, const float* edge, co
   p.edge = edge;
   p.ctx = ctx;
   p.desc = desc;
+  p.u_stride = (int64_t)s->batch * s->height * s->width * s->n_disp;
   return p;
+}
+
+// plain zero fill (a kernel, so that a caller may capture the call in a graph)
+__global__ void __launch_bounds__(256) zero_fill_kernel(float* __restrict__ dst, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = 0.f;
+}
+
+void zero_fill(float* dst, int64_t n, hipStream_t st) {
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  zero_fill_kernel<<<(int)blocks, 256, 0, st>>>(dst, n);
 }
 
 // cost_final is not written before the final aggregation, so its first bytes carry the context
@@ -617,7 +631,13 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   const bool train = msg_min_index != nullptr;
 
   const CtxDesc* desc = make_desc(s, context, cost_final, st);
-  {
+  // Messages that start at zero by declaration: S = unary, so the belief plane need not be built
+  // (the first pair of sweeps reads `unary` in its place: Q = S - m_0 - m_1 = unary, too, and the
+  // even sweep has nothing to store), no plane of initial messages is read (the descriptor's
+  // flag stays 0), and the first sweep of every direction writes the zero of its chain starts.
+  const bool uninit = s->msg_uninit != 0 && desc != nullptr;
+  if (s->msg_uninit != 0 && !uninit) zero_fill(msg, (int64_t)s->n_dir * N, st);
+  if (!uninit) {
     Timed timed(MPL_KERNEL_BELIEF, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
     int* flag = desc != nullptr ? &const_cast<CtxDesc*>(desc)->msg_nonzero : nullptr;
@@ -625,7 +645,6 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   }
 
   SweepParams p = base_fwd_params(s, rho, edge_weights, context, desc);
-  p.belief = unary_update;
   p.belief_out = unary_update;
   p.msg_in = msg;
   p.msg_out = msg;
@@ -634,7 +653,10 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
       p.first_iter = (it == 0);
       p.pair_q = 1;
-      p.skip_s_store = (it == n_iter - 1) && (d == s->n_dir - 1);  // cost_final is re-summed
+      p.belief = (uninit && it == 0 && d <= 1) ? unary : unary_update;
+      p.zero_start = (uninit && it == 0) ? 1 : 0;
+      p.skip_s_store = ((it == n_iter - 1) && (d == s->n_dir - 1)) ||  // cost_final is re-summed
+                       (uninit && it == 0 && d == 0);
       if (train) {
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
         p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
@@ -680,6 +702,11 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   p.belief_out = nullptr;
   fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
   p.u_pair_share = (rho == 1.f) ? 1 : 0;
+  // Messages that start at zero by declaration: U_d = rho * unary in the first iteration, so at
+  // rho = 1 its sweeps read `unary` itself and the pass that would store U is skipped (the
+  // sweeps write every element of their output buffer, chain starts included).
+  const bool unary_as_u = s->msg_uninit != 0 && rho == 1.f;
+  if (s->msg_uninit != 0 && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {
     // Jacobi over directions (ISGMR_forward.cu:506-622): every direction reads the old messages,
@@ -691,13 +718,17 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
     const bool out_of_place = (it == 0) && (n_iter & 1);
     float* ubuf = out_of_place ? other : have;
     float* nxt = out_of_place ? have : other;
-    {
+    if (it == 0 && unary_as_u) {
+      p.msg_in = unary;
+      p.u_stride = 0;
+    } else {
       Timed timed(MPL_KERNEL_UNARY_ALL, st);
       const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update);
       MPL_EW_LAUNCH(isgmr_unary_kernel, v4, s->n_dir, N, st, unary, have, ubuf, s->n_dir, N, rho,
                     p.u_pair_share);
+      p.msg_in = ubuf;
+      p.u_stride = N;
     }
-    p.msg_in = ubuf;
     p.msg_out = nxt;
     if (train) {
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
@@ -846,6 +877,7 @@ int mpl_trwp_soft_forward(const mpl_shape* s, float rho, int n_iter, const float
   const int64_t P = (int64_t)s->batch * s->height * s->width;
   const int64_t N = P * s->n_disp;
   const bool train = msg_edge_label != nullptr;
+  if (s->msg_uninit != 0) zero_fill(msg, (int64_t)s->n_dir * N, st);
   {
     Timed timed(MPL_KERNEL_BELIEF, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);

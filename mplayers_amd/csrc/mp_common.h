@@ -359,6 +359,10 @@ struct SweepParams {
   int first_iter;                  // Gauss-Seidel: first iteration (planes not yet swept hold the
                                    // caller's initial messages, which need not be read when zero)
   int u_pair_share;                // Jacobi: directions d and d^1 read the U plane of the even one
+  int64_t u_stride;                // Jacobi: elements between the U planes of msg_in (0: all directions
+                                   // read the one plane at msg_in)
+  int zero_start;                  // Gauss-Seidel: store zeros at the chain start of msg_out (the
+                                   // caller's buffer is undefined and this is its first sweep)
   float* edge_label;               // soft TRWP: (n_dir_total, P, L, L) duals of this iteration, or null
 };
 

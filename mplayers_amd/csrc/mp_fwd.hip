@@ -177,7 +177,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // Jacobi: the plane of this direction in msg_in holds U itself (written by the host's
   // element-wise pass before the sweeps), so one plane is read per pixel instead of three
   const float* __restrict__ bS =
-      (JACOBI ? p.msg_in + (int64_t)(p.u_pair_share ? (dir & ~1) : dir) * N : p.belief) + img_e;
+      (JACOBI ? p.msg_in + (int64_t)(p.u_pair_share ? (dir & ~1) : dir) * p.u_stride : p.belief) + img_e;
   const float* __restrict__ bMd = p.msg_in + (int64_t)dir * N + img_e;
   const float* __restrict__ bMi = p.msg_in + (int64_t)(dir ^ 1) * N + img_e;
   float* __restrict__ bMo = p.msg_out + (int64_t)dir * N + img_e;
@@ -271,7 +271,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       const unsigned so = (unsigned)ch.pix0 * (unsigned)vbytes;
       buf_store<R, VEC>(make_rsrc(bSo, (int)(so + (unsigned)vbytes)), foff, so, conv);
     }
-    if (JACOBI) {
+    if (JACOBI || p.zero_start) {
       float z[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) z[j] = 0.f;

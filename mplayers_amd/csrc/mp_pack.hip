@@ -147,7 +147,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
   const bool pair_first = !JACOBI && p.pair_q && (dir & 1) == 0;   // see mp_fwd.hip
   const bool pair_second = !JACOBI && p.pair_q && (dir & 1) == 1;
   const int udir = p.u_pair_share ? (dir & ~1) : dir;
-  const rsrc_t dS = make_rsrc(JACOBI ? p.msg_in + (int64_t)udir * N : p.belief, plane_bytes);
+  const rsrc_t dS = make_rsrc(JACOBI ? p.msg_in + (int64_t)udir * p.u_stride : p.belief, plane_bytes);
   const rsrc_t dMd = make_rsrc(p.msg_in + (int64_t)dir * N, (JACOBI || md_zero) ? 0 : plane_bytes);
   const rsrc_t dMdRing = make_rsrc(p.msg_in + (int64_t)dir * N,
                                    (JACOBI || md_zero || pair_second) ? 0 : plane_bytes);
@@ -197,7 +197,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
     if (!JACOBI && p.pair_q)  // convert the belief plane at the chain start as well
       stf(dSo, (on && n >= 1) ? (unsigned)(ch.pix0 * L + l) * 4u : (unsigned)kDeadOffset,
           pair_second ? t0 + p0.md : t0 - p0.mi);
-    if (JACOBI)  // the buffers alternate: the chain start is written with the zeros it keeps
+    if (JACOBI || p.zero_start)  // the chain start is written with the zeros it keeps
       stf(dMo, (on && n >= 1) ? (unsigned)(ch.pix0 * L + l) * 4u : (unsigned)kDeadOffset, 0.f);
   }
 

@@ -86,10 +86,13 @@ class TRWP(object):
 
   @staticmethod
   def forward(rho, n_iter, enable_min_a_dir, unary, context, edge_weights, msg, cost_final,
-              msg_min_index, msg_norm_index, unary_update, label_all):
+              msg_min_index, msg_norm_index, unary_update, label_all, msg_uninit=False):
+    """msg_uninit (not in the reference): True declares that `msg` holds no initial messages --
+    they start at zero and the library writes every element, so the caller need not clear it."""
     lib = _lib.load()
     shape, _, _ = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
                                      msg_norm_index, unary_update, label_all, n_iter)
+    shape.msg_uninit = int(bool(msg_uninit))
     with torch.cuda.device(unary.device):
       rc = lib.mpl_trwp_forward(shape, float(rho), int(n_iter), int(enable_min_a_dir),
                                 _ptr(unary), _ptr(context), _ptr(edge_weights), _ptr(msg),
@@ -127,10 +130,13 @@ class ISGMR(object):
 
   @staticmethod
   def forward(enable_sgm, rho, n_iter, enable_min_a_dir, unary, context, edge_weights, msg,
-              cost_final, msg_min_index, msg_norm_index, unary_update, msg_update, label_all):
+              cost_final, msg_min_index, msg_norm_index, unary_update, msg_update, label_all,
+              msg_uninit=False):
+    """msg_uninit (not in the reference): see TRWP.forward."""
     lib = _lib.load()
     shape, _, N = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
                                      msg_norm_index, unary_update, label_all, n_iter)
+    shape.msg_uninit = int(bool(msg_uninit))
     _check("msg_update", msg_update, torch.float32, shape.n_dir * N)
     with torch.cuda.device(unary.device):
       rc = lib.mpl_isgmr_forward(shape, int(enable_sgm), float(rho), int(n_iter),
