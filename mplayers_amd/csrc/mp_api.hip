@@ -29,6 +29,8 @@ __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __r
   r.c0_is_min = 0;
   r.cmax = 0.f;
   r.msg_nonzero = 0;
+  r.linear = 0;
+  r.slope = 0.f;
   if (!ctx2d) {
     float tail = ctx[L - 1];
     int k = L - 1;
@@ -45,6 +47,17 @@ __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __r
       r.band_k = k;
       r.cmax = tail;
       r.c0_is_min = c0min ? 1 : 0;
+    }
+    // truncated linear, bit for bit: c[k] == min(c[1] * k, c[L-1])
+    if (ok && L >= 2 && ctx[0] == 0.f && ctx[1] >= 0.f) {
+      const float slope = ctx[1];
+      bool lin = true;
+      for (int i = 0; i < L; ++i) lin = lin && (ctx[i] == fminf(slope * (float)i, tail));
+      if (lin) {
+        r.linear = 1;
+        r.slope = slope;
+        r.cmax = tail;
+      }
     }
   }
   *d = r;

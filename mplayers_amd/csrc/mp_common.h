@@ -111,6 +111,61 @@ __device__ __forceinline__ float wave_sum(float x) {
 
 __device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
 
+template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf>
+__device__ __forceinline__ int dpp_i(int old, int src) {
+  return __builtin_amdgcn_update_dpp(old, src, CTRL, ROW_MASK, BANK_MASK, false);
+}
+
+// Inclusive scans over the 64 lanes.  Prefix: lane i gets the result over lanes 0..i (shifts within
+// the rows of 16 lanes, then the row totals travel through the row broadcasts).  Suffix: lane i
+// gets the result over lanes i..63 (there is no broadcast in that direction: the three later row
+// totals are read back as scalars).
+__device__ __forceinline__ float lane_prefix_min(float x) {
+  const float inf = INFINITY;
+  x = fminf(x, dpp_f<0x111>(inf, x));
+  x = fminf(x, dpp_f<0x112>(inf, x));
+  x = fminf(x, dpp_f<0x114>(inf, x));
+  x = fminf(x, dpp_f<0x118>(inf, x));
+  x = fminf(x, dpp_f<0x142, 0xa>(inf, x));
+  x = fminf(x, dpp_f<0x143, 0xc>(inf, x));
+  return x;
+}
+__device__ __forceinline__ int lane_prefix_max(int x) {
+  constexpr int lo = -0x7fffffff - 1;
+  x = max(x, dpp_i<0x111>(lo, x));
+  x = max(x, dpp_i<0x112>(lo, x));
+  x = max(x, dpp_i<0x114>(lo, x));
+  x = max(x, dpp_i<0x118>(lo, x));
+  x = max(x, dpp_i<0x142, 0xa>(lo, x));
+  x = max(x, dpp_i<0x143, 0xc>(lo, x));
+  return x;
+}
+__device__ __forceinline__ float lane_suffix_min(float x, int lane) {
+  const float inf = INFINITY;
+  x = fminf(x, dpp_f<0x101>(inf, x));  // row_shl:1 ... 8: lane i of a row gets the row's lanes i..15
+  x = fminf(x, dpp_f<0x102>(inf, x));
+  x = fminf(x, dpp_f<0x104>(inf, x));
+  x = fminf(x, dpp_f<0x108>(inf, x));
+  const float r1 = readlane_f(x, 16), r2 = readlane_f(x, 32), r3 = readlane_f(x, 48);
+  const float m2 = fminf(r2, r3), m1 = fminf(r1, m2);
+  const int row = lane >> 4;
+  const float later = row == 0 ? m1 : (row == 1 ? m2 : (row == 2 ? r3 : inf));
+  return fminf(x, later);
+}
+__device__ __forceinline__ int lane_suffix_min(int x, int lane) {
+  constexpr int hi = 0x7fffffff;
+  x = min(x, dpp_i<0x101>(hi, x));
+  x = min(x, dpp_i<0x102>(hi, x));
+  x = min(x, dpp_i<0x104>(hi, x));
+  x = min(x, dpp_i<0x108>(hi, x));
+  const int r1 = __builtin_amdgcn_readlane(x, 16), r2 = __builtin_amdgcn_readlane(x, 32),
+            r3 = __builtin_amdgcn_readlane(x, 48);
+  const int m2 = min(r2, r3), m1 = min(r1, m2);
+  const int row = lane >> 4;
+  const int later = row == 0 ? m1 : (row == 1 ? m2 : (row == 2 ? r3 : hi));
+  return min(x, later);
+}
+
 // largest label (R*lane + j) whose predicate is set; `dflt` when none is
 template <int R>
 __device__ __forceinline__ int last_label(const bool (&pred)[R], int dflt) {
@@ -332,6 +387,8 @@ struct CtxDesc {
   int c0_is_min;  // c[0] <= c[k] for all k
   float cmax;
   int msg_nonzero;  // set by the belief pass when some initial message is not zero
+  int linear;       // c[k] == min(slope * k, c[L-1]) exactly for every k, slope >= 0 (truncated linear)
+  float slope;
 };
 
 // ------------------------------------------------------------------------------------------------

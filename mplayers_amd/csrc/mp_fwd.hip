@@ -159,8 +159,90 @@ __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, c
   }
 }
 
+// O(L log L / 64) step for truncated linear contexts c[k] = min(s*k, cmax) of any width, w >= 0.
+// With t = w*s,
+//   min_{fd <= cd} a[fd] + t*(cd - fd) =  t*cd + prefixmin_{fd <= cd} (a[fd] - t*fd)
+//   min_{fd >= cd} a[fd] + t*(fd - cd) = -t*cd + suffixmin_{fd >= cd} (a[fd] + t*fd)
+// so two scans over the labels find, for every cd, the best front label on either side; a label
+// beyond the truncation can only win where the far candidate min(a) + w*cmax is at least as good.
+// The scans run on rounded differences, so they only *select* the candidates (the largest label
+// among equals on each side, as the reference's scan order does); the values are then evaluated
+// from the table exactly as the dense scan does, a[fd] + w*c[|cd - fd|], and compared with the far
+// candidate.  A selection off by the rounding of t*L picks a value within a few ulp of the largest
+// belief of the true minimum.
+template <int R, bool TRAIN>
+__device__ __forceinline__ void linear_step(const float (&a)[R], float w, float slope, float cmax,
+                                            float amin, int fstar, int lab0, int lane, int L,
+                                            float* a_s, const float* ctx_s, float (&v)[R],
+                                            int (&fd_idx)[R]) {
+  const float inf = INFINITY;
+  constexpr int big = 0x7fffffff;
+  const float t = w * slope;
+  float gm[R], gp[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const float l = (float)(lab0 + j);
+    gm[j] = fmaf(-t, l, a[j]);
+    gp[j] = fmaf(t, l, a[j]);
+    a_s[lab0 + j] = a[j];  // staged for the gathers below
+  }
+  // left side: prefix minimum and its largest achiever (the largest label up to cd whose own
+  // prefix minimum it is)
+  float q[R], pl[R];
+  q[0] = gm[0];
+#pragma unroll
+  for (int j = 1; j < R; ++j) q[j] = fminf(q[j - 1], gm[j]);
+  const float before = wave_shr1(lane_prefix_min(q[R - 1]), inf);
+  int qi[R], il[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    pl[j] = fminf(before, q[j]);
+    const int f = (gm[j] == pl[j]) ? lab0 + j : -1;
+    qi[j] = j == 0 ? f : max(qi[j > 0 ? j - 1 : 0], f);
+  }
+  const int before_i = dpp_i<0x138>(-1, lane_prefix_max(qi[R - 1]));  // lane i <- lane i-1
+#pragma unroll
+  for (int j = 0; j < R; ++j) il[j] = max(max(before_i, qi[j]), 0);
+  // right side: suffix minimum; its largest achiever is where the plateau of that minimum ends
+  float sfx[R], pr[R], nx[R];
+  sfx[R - 1] = gp[R - 1];
+#pragma unroll
+  for (int j = R - 2; j >= 0; --j) sfx[j] = fminf(sfx[j + 1], gp[j]);
+  const float after = wave_shl1(lane_suffix_min(sfx[0], lane), inf);
+#pragma unroll
+  for (int j = 0; j < R; ++j) pr[j] = fminf(after, sfx[j]);
+#pragma unroll
+  for (int j = 0; j < R - 1; ++j) nx[j] = pr[j + 1];
+  nx[R - 1] = wave_shl1(pr[0], inf);
+  int si[R], ir[R];
+#pragma unroll
+  for (int j = R - 1; j >= 0; --j) {
+    const int b = (pr[j] < nx[j]) ? lab0 + j : big;
+    si[j] = j == R - 1 ? b : min(si[j < R - 1 ? j + 1 : j], b);
+  }
+  const int after_i = dpp_i<0x130>(big, lane_suffix_min(si[0], lane));  // lane i <- lane i+1
+#pragma unroll
+  for (int j = 0; j < R; ++j) ir[j] = min(min(after_i, si[j]), L - 1);
+  __syncthreads();  // a_s
+  const float far = fmaf(w, cmax, amin);
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int cd = lab0 + j;
+    const int kl = cd - il[j], kr = ir[j] - cd;
+    const float vl = fmaf(w, ctx_s[kl < 0 ? 0 : (kl < L ? kl : L - 1)], a_s[il[j]]);
+    const float vr = fmaf(w, ctx_s[kr < 0 ? 0 : kr], a_s[ir[j]]);
+    const bool tr = vr <= vl;  // the larger front label wins ties
+    float best = tr ? vr : vl;
+    int arg = tr ? ir[j] : il[j];
+    const bool lt = far < best, eq = far == best;
+    if (TRAIN) fd_idx[j] = lt ? fstar : (eq ? (arg > fstar ? arg : fstar) : arg);
+    v[j] = lt ? far : best;
+  }
+  __syncthreads();  // the next step overwrites a_s
+}
+
 // One chain.  KT: > 0 band with compile-time K, 0 band with run-time K, -1 dense, -21 dense with
-// exactly 21 labels.
+// exactly 21 labels, -2 truncated linear context of any width (linear_step).
 // VEC: L % R == 0 (vector accesses).  MASK: some lanes own labels >= L.
 template <int R, bool VEC, bool MASK, bool TRAIN, bool JACOBI, int KT>
 __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
@@ -319,7 +401,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       for (int j = 0; j < R; ++j) a[j] = fmaf(rho, prev[j], uf[j]);
       float nmin;
       bool need_nmin = true;
-      if (KT >= 0 && w >= 0.f) {
+      if ((KT >= 0 || KT == -2) && w >= 0.f) {
         float am = a[0];
 #pragma unroll
         for (int j = 1; j < R; ++j) am = fminf(am, a[j]);
@@ -331,14 +413,19 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
           for (int j = 0; j < R; ++j) pr[j] = (a[j] == amin);
           fstar = last_label<R>(pr, L - 1);
         }
-        band_step<R, TRAIN, (KT > 0 ? KT : 0)>(a, w, K, c_reg, ctx_s, cmax, amin, fstar, lab0, v,
-                                               fd_idx);
-        if (c0min) {
+        if constexpr (KT == -2) {
+          linear_step<R, TRAIN>(a, w, desc.slope, cmax, amin, fstar, lab0, lane, L, a_s, ctx_s, v,
+                                fd_idx);
+        } else {
+          band_step<R, TRAIN, (KT > 0 ? KT : 0)>(a, w, K, c_reg, ctx_s, cmax, amin, fstar, lab0, v,
+                                                 fd_idx);
+        }
+        if (KT != -2 && c0min) {
           // every candidate is >= amin + w*c[0], which the centre tap of label argmin(a) attains
           nmin = fmaf(w, KT > 0 ? c_reg[0] : ctx_s[0], amin);
           need_nmin = false;
         }
-      } else if (R == 1 && KT < 0) {
+      } else if (R == 1 && KT < 0 && desc.band_k == 0) {  // (the full table is in LDS then)
         if constexpr (LT > 0) {
           // 21 labels: the scan over front labels fully unrolled, context column in registers
           float best = inf;
@@ -416,6 +503,8 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
     desc.c0_is_min = 0;
     desc.cmax = 0.f;
     desc.msg_nonzero = 1;
+    desc.linear = 0;
+    desc.slope = 0.f;
   }
   // context table into LDS (dense path, run-time band taps, negative-weight fallback)
   if (R == 1 && desc.band_k == 0) {
@@ -431,6 +520,11 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
   }
   __syncthreads();
 
+  // wide truncated-linear contexts: two label scans instead of 2K-1 taps or the dense scan
+  if (desc.linear && !p.ctx2d && (desc.band_k == 0 || desc.band_k > 4)) {
+    run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -2>(p, desc, ch, a_s, ctx_s);
+    return;
+  }
   switch (desc.band_k) {
     case 0:
       if (R == 1 && L == 21)
