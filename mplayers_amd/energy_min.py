@@ -22,6 +22,7 @@ import numpy as np
 import torch
 
 from . import compute_terms
+from .label_context import create_label_context
 from .MP_module import MPModule
 
 
@@ -97,9 +98,15 @@ def build_terms(args):
   if args.synthetic is None and args.img_name in ('house', 'penguin'):
     path = '%s/Denoise/%s_unary.csv' % (args.data_dir, args.img_name)
     _, _, n_disp, cost = parse_unary_cost(path)
-    # the denoising problems take their pairwise table unscaled (main.py:112-127)
-    table = compute_terms.smoothness_context(n_disp, args.context, args.truncated)
-    return cost.to(device), table.to(device), n_disp
+    # the denoising problems build their pairwise table with the label-context builder
+    # (main.py:112-127): the term weight is applied there and the truncation acts on the
+    # (squared) cost itself, a negative value meaning none
+    ctx_args = argparse.Namespace(
+        n_classes=n_disp, mpnet_smoothness_mode=args.context, mpnet_smoothness_train=None,
+        mpnet_smoothness_trunct_loc=-1, mpnet_smoothness_trunct_value=args.truncated,
+        mpnet_term_weight=args.p_weight, enable_cuda=False)
+    table, _, _ = create_label_context(ctx_args, enable_seg=True, enable_symmetric=True)
+    return cost.to(device), table.detach().to(device), n_disp
   if args.synthetic is not None:
     left, right, _ = synthetic_stereo_pair(args.synthetic[0], args.synthetic[1], args.n_disp)
   else:

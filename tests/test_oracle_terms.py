@@ -252,3 +252,21 @@ def test_unary_csv_and_synthetic_pair(tmp_path):
   # the true disparity has zero plain matching cost wherever the match is inside the image
   dsi = terms_oracle.compute_dsi(left, right, 8, birchfield=0)
   assert (dsi[ys, xs, disp[ys, xs]] == 0).all()
+
+
+def test_denoising_terms_follow_the_label_context_builder(tmp_path):
+  """house / penguin: unary from the CSV file, pairwise table from create_label_context with the
+  truncation acting on the squared cost and the term weight applied (MPLayers/main.py:112-127)."""
+  import argparse
+  from mplayers_amd import energy_min
+  from mplayers_amd.label_context import create_label_context
+  n = 9
+  ns = argparse.Namespace(n_classes=n, mpnet_smoothness_mode="TQ", mpnet_smoothness_train=None,
+                          mpnet_smoothness_trunct_loc=-1, mpnet_smoothness_trunct_value=20,
+                          mpnet_term_weight=5, enable_cuda=False)
+  table, _, _ = create_label_context(ns, enable_seg=True, enable_symmetric=True)
+  k = np.abs(np.arange(n)[:, None] - np.arange(n)[None, :])
+  assert (table.detach().numpy() == 5 * np.minimum(k * k, 20)).all()
+  ns.mpnet_smoothness_trunct_value = -1
+  table, _, _ = create_label_context(ns, enable_seg=True, enable_symmetric=True)
+  assert (table.detach().numpy() == 5 * k * k).all()
