@@ -57,6 +57,50 @@ __device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&val
   __syncthreads();
 }
 
+// Dense O(L^2) step for 1-D contexts and several labels per lane, without LDS in its loop.  The
+// front labels are visited in ascending order; a[fd] is broadcast with v_readlane, and the context
+// values c[|cd - fd|] of the lane's labels are kept in registers and moved one label up per front
+// label (c[|cd - (fd+1)|] of label cd is c[|(cd-1) - fd|] of label cd - 1; c[fd+1] enters at
+// label 0).  `<=` on the ascending scan keeps the largest front label among equals, as the
+// reference's descending scan with `<` does.
+template <int R, bool TRAIN>
+__device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L, int lab0,
+                                             const float* ctx_s, float (&v)[R], int (&fd_idx)[R]) {
+  float c_own[R], cv[R];  // c[label] of the lane's labels; the sliding c[|label - fd|]
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int l = lab0 + j;
+    c_own[j] = ctx_s[l < L ? l : L - 1];
+    cv[j] = c_own[j];
+    v[j] = INFINITY;
+    fd_idx[j] = L - 1;
+  }
+  for (int fd0 = 0; fd0 < L; fd0 += R) {
+    const int src = fd0 / R;  // the lane that owns front labels fd0 .. fd0 + R - 1
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+      const int fd = fd0 + u;
+      if (fd < L) {  // wave-uniform; always true when L is a multiple of R
+        const float af = readlane_f(a[u], src);
+        // c[fd + 1]: the next label's own entry (past the last label the value is never used)
+        const float cn = u + 1 < R ? readlane_f(c_own[u + 1 < R ? u + 1 : 0], src)
+                                   : readlane_f(c_own[0], (src + 1) & 63);
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const float val = fmaf(w, cv[j], af);
+          const bool take = val <= v[j];
+          v[j] = take ? val : v[j];
+          if (TRAIN) fd_idx[j] = take ? fd : fd_idx[j];
+        }
+        const float in0 = wave_shr1(cv[R - 1], cn);
+#pragma unroll
+        for (int j = R - 1; j > 0; --j) cv[j] = cv[j - 1];
+        cv[0] = in0;
+      }
+    }
+  }
+}
+
 // Dense step for L <= 64 (one label per lane): a[fd] is broadcast with v_readlane and the context
 // comes from a full table tab[fd * L + cd] in LDS, which consecutive lanes read without bank
 // conflicts.  Same scan order as dense_step.
@@ -443,7 +487,10 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
           dense_step_r1<TRAIN>(a[0], L, w, lane, ctx_s, v[0], fd_idx[0]);
         }
       } else if (live) {
-        dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
+        if constexpr (R > 1)  // (2-D tables exist for one label per lane only)
+          dense1d_step<R, TRAIN>(a, w, L, lab0, ctx_s, v, fd_idx);
+        else
+          dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
       } else {
 #pragma unroll
         for (int j = 0; j < R; ++j) {
