@@ -89,8 +89,10 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   // the far candidate, which is nearly always one of the popular targets.  A 1-D context with a
   // band of K entries therefore needs label shifts up to K - 1 only; rarer offsets within kNear
   // fall through to the slow path, so any choice here is exact.
+  // (With one label per lane the step is short and the scans are bound by its latency, which
+  // the wave-uniform branches would lengthen: the narrowing is for several labels per lane.)
   int near_max = kNear;
-  if (!ctx2d && !small_l) {
+  if (R > 1 && !ctx2d && !small_l) {
     int kb = 0;
     for (int i = lane; i < L; i += kWave) kb = (ctx_s[i] != ctx_s[L - 1]) ? i + 1 : kb;
     kb = (int)-wave_min(-(float)kb);  // wave maximum: entries at and beyond kb equal the last one
@@ -253,7 +255,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
         const float s0sum = wave_sum(p0);
         // nothing belongs to the second class when both popular targets coincide (the usual case)
         float s1sum = 0.f;
-        if (f1 != f0) s1sum = wave_sum(p1);
+        if (R == 1 || f1 != f0) s1sum = wave_sum(p1);
         // near targets: sc_next[l] += g[l - o] where index(l - o) == l, |o| <= kNear
         float tp[R], tn[R], near_t[kNear + 1];
 #pragma unroll
@@ -261,7 +263,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
         for (int o = kNear; o >= 1; --o) {
           near_t[o] = 0.f;
-          if (o > near_max) continue;  // wave-uniform
+          if (R > 1 && o > near_max) continue;  // wave-uniform
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             const float cp = (off[j] == o) ? gv[j] : 0.f;
