@@ -164,6 +164,11 @@ def main(argv=None):
     raise RuntimeError('energy_min needs a GPU (there is no CPU path in this build)')
   if args.synthetic is not None and args.img_name == 'tsukuba':
     args.img_name = 'synthetic'
+  if args.mode == 'SGM' and args.n_iter != 1:
+    # SGM is one Jacobi iteration by definition; the reference moves this mode to its CPU path
+    # because its GPU module insists on a single iteration (MP_module.py:205-206, main.py:239-241)
+    print('SGM: running 1 iteration instead of %d' % args.n_iter)
+    args.n_iter = 1
   # MPModule fixes rho per mode as the reference's does; the option only names the result file
   rho = args.rho if args.rho is not None else (0.5 if args.mode == 'TRWP' else 1)
   file_path = result_path(args, rho) if args.enable_saving_label else None

@@ -174,6 +174,13 @@ def test_compute_all_terms_from_image_files(gpu, tmp_path):
   assert (table1.cpu().numpy() == np.minimum(k * k, 4)).all()
 
 
+def test_driver_runs_sgm_as_one_iteration(gpu, tmp_path):
+  from mplayers_amd import energy_min
+  res = energy_min.main(["--synthetic", "24", "32", "--mode", "SGM", "--n_dir", "8", "--n_iter", "5",
+                         "--n_disp", "8", "--context", "TL", "--truncated", "2"])
+  assert res["labels"].shape[0] == 1 and res["energy"].shape == (1, 2)
+
+
 @pytest.mark.parametrize("mode,n_dir", [("TRWP", 4), ("ISGMR", 8), ("TRWP", 16)])
 def test_energy_minimisation_driver(gpu, tmp_path, mode, n_dir):
   """End to end on a random-dot stereo pair: the layer's labelling has a far lower energy than the
