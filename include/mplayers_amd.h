@@ -216,6 +216,13 @@ int mpl_mrf_energy(const mpl_shape* shape, int n_labelings, const float* unary,
 int mpl_probe_copy(int shape, int n_in, int n_out, const float* in, float* out, int height,
                    int width, int n_labels, void* stream);
 
+/* Batched 2-D transpose src (batch, rows, cols) -> dst (batch, cols, rows), fp32: the layout change
+ * between the network's (batch, labels, H, W) tensors and the kernels' (batch, H, W, labels), which
+ * the reference's module does with permute().contiguous() (pytorch/MP_module.py:199,203,233).
+ * rows = labels, cols = H*W on the way in; rows = H*W, cols = labels on the way out. */
+int mpl_transpose(const float* src, float* dst, int batch, int64_t rows, int64_t cols,
+                  void* stream);
+
 /* Message of the last failed call on this thread ("" if none). */
 const char* mpl_last_error(void);
 

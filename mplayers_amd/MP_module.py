@@ -15,6 +15,7 @@ import torch.nn as nn
 
 from . import lib_seg, lib_stereo
 from .label_context import create_label_context
+from .layout import labels_first, labels_last
 
 
 def _ops_for(n_disp):
@@ -197,7 +198,7 @@ class MPModule(torch.nn.Module):
 
   def forward(self, unary, edge_weights=None):
     # label axis innermost for the kernels; direction axis outermost for the edge weights
-    unary = unary.permute(0, 1, 3, 4, 2).contiguous()
+    unary = labels_last(unary)
     if edge_weights is not None:
       edge_weights = edge_weights.unsqueeze(1).permute(2, 0, 1, 3, 4).contiguous()
       assert unary.size()[-3:-1] == edge_weights.size()[-2:]
@@ -211,5 +212,5 @@ class MPModule(torch.nn.Module):
       cost_final, cost_all = TRWPFunction.apply(unary, label_context, edge_weights, self.args)
     else:
       assert False
-    cost_final = cost_final.permute(0, 1, 4, 2, 3).contiguous()
+    cost_final = labels_first(cost_final)
     return cost_final, label_context.unsqueeze(0), cost_all, None, None

@@ -14,6 +14,7 @@ the HIP library of this package.
 import torch
 
 from . import lib_seg, lib_stereo
+from .layout import labels_first, labels_last
 from .MP_module import MPModule as _HardModule
 
 _U8 = dict(dtype=torch.uint8)
@@ -113,7 +114,7 @@ class MPModule(_HardModule):
 
   def forward(self, unary, edge_weights=None, msg_norm_index=None, pairwise_terms=None):
     assert self.args.mpnet_mrf_mode == 'TRWP'
-    unary = unary.permute(0, 1, 3, 4, 2).contiguous()
+    unary = labels_last(unary)
     if edge_weights is not None:
       edge_weights = edge_weights.unsqueeze(1).permute(2, 0, 1, 3, 4).contiguous()
       assert unary.size()[-3:-1] == edge_weights.size()[-2:]
@@ -124,5 +125,5 @@ class MPModule(_HardModule):
     self.args.training = self.training
     cost_final, label_all, blocks, cost_index = TRWPFunction.apply(unary, label_context,
                                                                    edge_weights, self.args)
-    return (cost_final.permute(0, 1, 4, 2, 3).contiguous(), label_context.unsqueeze(0), label_all,
+    return (labels_first(cost_final), label_context.unsqueeze(0), label_all,
             blocks, cost_index)

@@ -24,7 +24,8 @@ HIPCC_FLAGS = [
 def _units():
   units = [("mp_api", "mp_api.hip", []), ("mp_edge", "mp_edge.hip", []),
            ("mp_soft", "mp_soft.hip", []), ("mp_pack", "mp_pack.hip", []),
-           ("mp_terms", "mp_terms.hip", []), ("mp_probe", "mp_probe.hip", [])]
+           ("mp_terms", "mp_terms.hip", []), ("mp_probe", "mp_probe.hip", []),
+           ("mp_layout", "mp_layout.hip", [])]
   for r in (1, 2, 3, 4):
     units.append(("mp_fwd_r%d" % r, "mp_fwd.hip", ["-DMPL_INST_R=%d" % r]))
     units.append(("mp_bwd_r%d" % r, "mp_bwd.hip", ["-DMPL_INST_R=%d" % r]))

@@ -9,7 +9,7 @@ SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_is
            "mpl_selftest_wave_ops", "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
            "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_trwp_soft_forward",
            "mpl_trwp_soft_backward", "mpl_soft_weighted_message", "mpl_soft_weighted_message_back", "mpl_set_option",
-           "mpl_stereo_data_cost", "mpl_gradient_cues", "mpl_mrf_energy", "mpl_probe_copy")
+           "mpl_stereo_data_cost", "mpl_gradient_cues", "mpl_mrf_energy", "mpl_probe_copy", "mpl_transpose")
 
 KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combine", "other",
                 "fwd_sweep_all", "bwd_sweep_all", "unary_all")
@@ -56,6 +56,7 @@ def load():
   lib.mpl_gradient_cues.argtypes = [vp, ci, ci, ci, ci, cf, vp, vp, vp]
   lib.mpl_mrf_energy.argtypes = [sp, ci, vp, vp, vp, vp, vp, vp]
   lib.mpl_probe_copy.argtypes = [ci, ci, ci, vp, vp, ci, ci, ci, vp]
+  lib.mpl_transpose.argtypes = [vp, vp, ci, ctypes.c_int64, ctypes.c_int64, vp]
   lib.mpl_selftest_wave_ops.argtypes = [ctypes.POINTER(ci)]
   lib.mpl_n_chains.argtypes = [ci, ci, ci]
   lib.mpl_profile_begin.argtypes = []
