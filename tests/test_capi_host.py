@@ -169,3 +169,52 @@ def test_synthetic_configs_are_seeded_and_shaped():
   c4 = synthetic.make_config("C4", scale=0.1, mode="ISGMR")
   assert c4["rho"] == 1.0 and c4["context"].shape == (21, 21)
   assert torch.equal(torch.tril(c4["context"]), torch.zeros(21, 21))
+
+
+def test_product_never_touches_the_oracle_or_scratch_files():
+  """The package, the bench and the entry points may not import anything from oracle/ (test
+  infrastructure; bench.py's cpu_baseline leg and smoke() are the two allowed users) nor read the
+  builder's scratch folder."""
+  import os
+  import re
+  root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+  pkg = os.path.join(root, "mplayers_amd")
+  offenders = []
+  for dirpath, _, files in os.walk(pkg):
+    for name in files:
+      if not name.endswith((".py", ".hip", ".h")):
+        continue
+      text = open(os.path.join(dirpath, name)).read()
+      if re.search(r"^\s*(from|import)\s+oracle\b", text, re.M) or re.search(r"(^|[\"'/\s])_work/", text):
+        offenders.append(os.path.relpath(os.path.join(dirpath, name), root))
+  assert offenders == []
+  bench = open(os.path.join(root, "bench.py")).read()
+  uses = [m.start() for m in re.finditer(r"from oracle|import oracle", bench)]
+  body = bench[bench.index("def cpu_baseline"):]
+  end = body.index("\ndef ", 1)
+  assert all(bench.index("def cpu_baseline") <= u < bench.index("def cpu_baseline") + end for u in uses)
+  assert not re.search(r"(^|[\"'/\s])_work/", bench)
+
+
+def test_new_entry_points_validate_before_launching():
+  """Terms, probe and transpose entry points answer bad arguments with MPL_EINVAL on the host."""
+  import ctypes
+  from mplayers_amd import _lib
+  lib = _lib.load()
+  null = ctypes.c_void_p(None)
+  one = ctypes.c_void_p(16)   # never dereferenced: every call below fails validation first
+  assert lib.mpl_stereo_data_cost(null, one, 4, 4, 3, 8, 1, 0, 255, one, null) != 0
+  assert lib.mpl_stereo_data_cost(one, one, 0, 4, 3, 8, 1, 0, 255, one, null) != 0
+  assert lib.mpl_gradient_cues(null, 4, 4, 3, 8, ctypes.c_float(2), one, one, null) != 0
+  assert lib.mpl_gradient_cues(one, 4, 4, 3, 8, ctypes.c_float(2), null, one, null) != 0
+  shape = _lib.Shape(3, 1, 4, 4, 8, 0)      # odd direction count
+  assert lib.mpl_mrf_energy(ctypes.byref(shape), 1, one, one, null, one, one, null) != 0
+  shape = _lib.Shape(4, 1, 4, 4, 8, 0)
+  assert lib.mpl_mrf_energy(ctypes.byref(shape), 1, one, one, null, null, one, null) != 0
+  assert lib.mpl_mrf_energy(ctypes.byref(shape), 0, one, one, null, one, one, null) == 0  # nothing to do
+  assert lib.mpl_probe_copy(0, 2, 2, one, one, 4, 4, 8, null) != 0
+  assert lib.mpl_probe_copy(0, 1, 1, one, one, 4, 4, 6, null) != 0
+  assert lib.mpl_transpose(null, one, 1, 4, 4, null) != 0
+  assert lib.mpl_transpose(one, one, 1, -1, 4, null) != 0
+  assert lib.mpl_transpose(one, one, 0, 4, 4, null) == 0                                  # empty
+  assert b"" != lib.mpl_last_error()
