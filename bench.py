@@ -274,7 +274,7 @@ def main():
 
   uninit = not a.caller_clears_messages
 
-  def step():
+  def step(uninit=uninit):
     for alg in algs:
       rho = 1.0 if alg == "ISGMR" else 0.5
       if alg == "SOFT" or not uninit:
@@ -379,6 +379,19 @@ def main():
       "other_kernels_ms": {k: round(stats[k][1], 3) for k in stats if k not in kernels},
 
   }
+  if uninit and "SOFT" not in algs:
+    # the same step under the reference's contract, for comparison: `msg` zero-filled by the
+    # caller inside the step and read back by the operators as initial messages
+    n_ref = min(3, a.steps)
+    step(uninit=False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n_ref):
+      step(uninit=False)
+    torch.cuda.synchronize()
+    ref_ms = (time.perf_counter() - t0) / n_ref * 1e3
+    out["caller_cleared_messages"] = {"ms_per_step": ref_ms, "steps": n_ref,
+                                      "value": units_per_step / (ref_ms * 1e-3)}
   if a.peak_probe:
     out["measured_stream_rates"] = peak_probe(H, W, L, dev)
   if a.module_probe and training:
