@@ -138,7 +138,10 @@ __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
         for (int fd = 0; fd < LT; ++fd) {
           dual[fd] = fmaf(w, tcol[fd], readlane_f(a, fd));
           mn = fminf(mn, dual[fd]);
-          if (TRAIN && valid) tile[wbase + fd * wstep] = dual[fd];
+        }
+        if (TRAIN && valid) {  // one predicated region for the whole column, not one per store
+#pragma unroll
+          for (int fd = 0; fd < LT; ++fd) tile[wbase + fd * wstep] = dual[fd];
         }
         // pass 2: softmin weights and the expected dual
 #pragma unroll
@@ -327,7 +330,11 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
             const float dd = gs * ex[fd] * (soft1 - dual[fd]);  // :110-113
             de = fmaf(tcol[fd], dd, de);
             hreg[fd] = fmaf(w, dd, hreg[fd]);
-            if (valid) grad[fd * Lp + lane] = dd;
+            ex[fd] = dd;
+          }
+          if (valid) {  // one predicated region for the whole column, not one per store
+#pragma unroll
+            for (int fd = 0; fd < LT; ++fd) grad[fd * Lp + lane] = ex[fd];
           }
         } else {
 #pragma unroll 4
