@@ -349,12 +349,12 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
           const float inv = 1.f / se;
           const float soft1 = fmaf(sd, inv, 1.f);
           const float gs = gv * inv;
+          if (valid) {  // (lanes without a label carry gv = 0 and would add nothing)
 #pragma unroll 4
-          for (int fd = 0; fd < L; ++fd) {
-            const float dual = tile[dbase + fd * dstep];
-            const float dd = gs * fast_exp(mn - dual) * (soft1 - dual);  // :110-113
-            de = fmaf(tab[fd * L + col], dd, de);
-            if (valid) {
+            for (int fd = 0; fd < L; ++fd) {
+              const float dual = tile[dbase + fd * dstep];
+              const float dd = gs * fast_exp(mn - dual) * (soft1 - dual);  // :110-113
+              de = fmaf(tab[fd * L + col], dd, de);
               hist[fd * L + lane] = fmaf(w, dd, hist[fd * L + lane]);  // this lane's own entries
               grad[fd * Lp + lane] = dd;
             }
