@@ -272,6 +272,74 @@ __global__ void __launch_bounds__(256) label_kernel(const float* __restrict__ un
   }
 }
 
+// The same for label counts that are a multiple of 4: a group of `group` lanes (a power of two
+// >= L/4) per pixel, 16 bytes per lane and plane, 64/group pixels per wavefront; the argmin is a
+// butterfly over the group on (value, label) pairs.
+__global__ void __launch_bounds__(256) label_quad_kernel(const float* __restrict__ unary,
+                                                         const float* __restrict__ msg, int n_dir,
+                                                         int64_t P, int L, int group, float factor,
+                                                         int min_a_dir, uint8_t* __restrict__ label) {
+  const int64_t N = P * L;
+  const int sub = threadIdx.x & (group - 1);
+  const int64_t pix = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / group;
+  float best = INFINITY;
+  int arg = 0x7fffffff;
+  if (pix < P && sub * 4 < L) {
+    const int64_t i = pix * L + sub * 4;
+    Pack<4> v = ld_pack<4>(unary + i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v.v[j] *= factor;
+    if (min_a_dir) {
+      Pack<4> mn = ld_pack<4>(msg + i);
+      for (int k = 1; k < n_dir; ++k) {
+        Pack<4> m = ld_pack<4>(msg + (int64_t)k * N + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (m.v[j] < mn.v[j]) mn.v[j] = m.v[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v.v[j] += mn.v[j];
+    } else {
+      for (int k = 0; k < n_dir; ++k) {
+        Pack<4> m = ld_pack<4>(msg + (int64_t)k * N + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v.v[j] += m.v[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (v.v[j] < best) {
+        best = v.v[j];
+        arg = sub * 4 + j;
+      }
+  }
+  for (int o = 1; o < group; o <<= 1) {
+    float ob = __shfl_xor(best, o);
+    int oa = __shfl_xor(arg, o);
+    if (ob < best || (ob == best && oa < arg)) {
+      best = ob;
+      arg = oa;
+    }
+  }
+  if (pix < P && sub == 0) label[pix] = (uint8_t)((arg < L) ? arg : 0);
+}
+
+static void launch_labels(const float* unary, const float* msg, int n_dir, int64_t P, int L,
+                          float factor, int min_a_dir, uint8_t* label, hipStream_t st) {
+  const bool aligned = (((uintptr_t)unary | (uintptr_t)msg) & 15) == 0;
+  if ((L & 3) == 0 && aligned) {
+    int group = 1;
+    while (group * 4 < L) group <<= 1;
+    const int64_t blocks = (P * group + 255) / 256;
+    label_quad_kernel<<<(unsigned)blocks, 256, 0, st>>>(unary, msg, n_dir, P, L, group, factor,
+                                                        min_a_dir, label);
+  } else {
+    const int64_t waves = (P < 256 * 64) ? P : 256 * 64;
+    label_kernel<<<(int)((waves + 3) / 4), 256, 0, st>>>(unary, msg, n_dir, P, L, factor, min_a_dir,
+                                                         label);
+  }
+}
+
 // ISGMR: after all directions of an iteration have been scanned back (X_k = dU_k):
 //   dunary += rho * sum_k X_k ;  gu_k = rho * (sum - X_k) - X_{k^1}   (written to G)
 // (UpdateUnaryKernelBack summed over directions + SumMsgKernel, ISGMR_backward.cu:39-60, 482-483)
@@ -677,10 +745,8 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
       launch_fwd(p, train, false, st);
     }
     if (label_all) {
-      int64_t waves = (P < 256 * 64) ? P : 256 * 64;
       Timed timed(MPL_KERNEL_LABEL, st);
-      label_kernel<<<(int)((waves + 3) / 4), 256, 0, st>>>(unary, msg, s->n_dir, P, s->n_disp, 1.f,
-                                                           enable_min_a_dir, label_all + it * P);
+      launch_labels(unary, msg, s->n_dir, P, s->n_disp, 1.f, enable_min_a_dir, label_all + it * P, st);
     }
   }
   {
@@ -749,11 +815,8 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
     }
     launch_fwd(p, train, true, st);
     if (label_all) {
-      int64_t waves = (P < 256 * 64) ? P : 256 * 64;
       Timed timed(MPL_KERNEL_LABEL, st);
-      label_kernel<<<(int)((waves + 3) / 4), 256, 0, st>>>(unary, nxt, s->n_dir, P, s->n_disp,
-                                                           factor, enable_min_a_dir,
-                                                           label_all + it * P);
+      launch_labels(unary, nxt, s->n_dir, P, s->n_disp, factor, enable_min_a_dir, label_all + it * P, st);
     }
     have = nxt;
   }
@@ -913,10 +976,8 @@ int mpl_trwp_soft_forward(const mpl_shape* s, float rho, int n_iter, const float
       launch_soft_fwd(p, train, st);
     }
     if (label_all) {
-      int64_t waves = (P < 256 * 64) ? P : 256 * 64;
       Timed timed(MPL_KERNEL_LABEL, st);
-      label_kernel<<<(int)((waves + 3) / 4), 256, 0, st>>>(unary, msg, s->n_dir, P, s->n_disp, 1.f,
-                                                           0, label_all + it * P);
+      launch_labels(unary, msg, s->n_dir, P, s->n_disp, 1.f, 0, label_all + it * P, st);
     }
   }
   {
