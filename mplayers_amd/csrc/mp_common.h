@@ -76,6 +76,11 @@ __device__ __forceinline__ float dpp_f(float old, float src) {
 __device__ __forceinline__ float wave_shl1(float x, float fill) { return dpp_f<0x130>(fill, x); }
 // lane i <- lane i-1 (lane 0 <- fill)
 __device__ __forceinline__ float wave_shr1(float x, float fill) { return dpp_f<0x138>(fill, x); }
+// the same shifts where the lane without a source keeps its own value of x: in place, with no fill
+// register to set up.  For a vector that an earlier filling shift in the same direction produced,
+// that lane already holds the fill, and keeps holding it.
+__device__ __forceinline__ float wave_shl1_keep(float x) { return dpp_f<0x130>(x, x); }
+__device__ __forceinline__ float wave_shr1_keep(float x) { return dpp_f<0x138>(x, x); }
 
 __device__ __forceinline__ float readlane_f(float x, int lane) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), lane));

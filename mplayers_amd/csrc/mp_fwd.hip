@@ -127,7 +127,7 @@ __device__ __forceinline__ void dense_step_r1(float a, int L, float w, int lane,
 //   v[cd] = min( min_{|k|<K} a[cd+k] + w*c[|k|],  min_fd a[fd] + w*cmax )
 // The second term is an upper bound for every label and is attained by all labels farther than the
 // band from argmin(a); fp32 addition is monotone, so the values are bit-identical to the dense scan.
-// KT > 0: K known at compile time, taps c[] in registers.  KT == 0: K at run time, taps in LDS.
+// KT > 0: KT - 1 taps with c[] in registers (KT >= K).  KT == 0: K at run time, taps in LDS.
 template <int R, bool TRAIN, int KT>
 __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, const float* c_reg,
                                           const float* ctx_s, float cmax, float amin, int fstar,
@@ -143,10 +143,12 @@ __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, c
     v[j] = fmaf(w, c0, a[j]);
     off[j] = 0;
   }
-  auto tap = [&](int k, float ck) {
+  // `refill`: up[0] / dn[R-1] still hold unshifted beliefs, so the vacated lane is set to +inf;
+  // from tap R+1 on every vector has been through one such shift and the lane keeps its +inf
+  auto tap = [&](int k, float ck, bool refill) {
     // one-label shifts: up[j] <- a[label + k], dn[j] <- a[label - k]
-    float tu = wave_shl1(up[0], inf);
-    float td = wave_shr1(dn[R - 1], inf);
+    float tu = refill ? wave_shl1(up[0], inf) : wave_shl1_keep(up[0]);
+    float td = refill ? wave_shr1(dn[R - 1], inf) : wave_shr1_keep(dn[R - 1]);
 #pragma unroll
     for (int j = 0; j < R - 1; ++j) up[j] = up[j + 1];
     up[R - 1] = tu;
@@ -155,9 +157,9 @@ __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, c
     dn[0] = td;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      float cu = fmaf(w, ck, up[j]);
-      float cd = fmaf(w, ck, dn[j]);
       if (TRAIN) {
+        float cu = fmaf(w, ck, up[j]);
+        float cd = fmaf(w, ck, dn[j]);
         bool tk = cu <= v[j];  // larger front label wins ties
         v[j] = tk ? cu : v[j];
         off[j] = tk ? k : off[j];
@@ -165,27 +167,40 @@ __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, c
         v[j] = tk2 ? cd : v[j];
         off[j] = tk2 ? -k : off[j];
       } else {
-        v[j] = fminf(v[j], fminf(cu, cd));
+        // x -> fma(w, ck, x) is monotone, so the smaller belief of the two gives the smaller
+        // candidate: one multiply-add per tap and label, the same bits
+        v[j] = fminf(v[j], fmaf(w, ck, fminf(up[j], dn[j])));
       }
     }
   };
   if (KT > 0) {
 #pragma unroll
-    for (int k = 1; k < KT; ++k) tap(k, c_reg[k]);
+    for (int k = 1; k < KT; ++k) tap(k, c_reg[k], k <= R);
   } else {
     // R taps per trip: the R one-label rotations of up[] / dn[] then cancel, so the loop carries
     // no register moves, and the R coefficients are fetched from LDS together
     int k = 1;
-    for (; k + R <= K; k += R) {
+    if (K > R) {
       float cc[R];
 #pragma unroll
-      for (int u = 0; u < R; ++u) cc[u] = ctx_s[k + u];
+      for (int u = 0; u < R; ++u) cc[u] = ctx_s[1 + u];
 #pragma unroll
-      for (int u = 0; u < R; ++u) tap(k + u, cc[u]);
+      for (int u = 0; u < R; ++u) tap(1 + u, cc[u], true);
+      k = 1 + R;
+      for (; k + R <= K; k += R) {
+#pragma unroll
+        for (int u = 0; u < R; ++u) cc[u] = ctx_s[k + u];
+#pragma unroll
+        for (int u = 0; u < R; ++u) tap(k + u, cc[u], false);
+      }
+#pragma unroll
+      for (int u = 0; u < R - 1; ++u)
+        if (k + u < K) tap(k + u, ctx_s[k + u], false);
+    } else {
+#pragma unroll
+      for (int u = 0; u < R - 1; ++u)
+        if (1 + u < K) tap(1 + u, ctx_s[1 + u], true);
     }
-#pragma unroll
-    for (int u = 0; u < R - 1; ++u)
-      if (k + u < K) tap(k + u, ctx_s[k + u]);
   }
   const float far = fmaf(w, cmax, amin);
 #pragma unroll
@@ -582,7 +597,23 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
     case 2: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 2>(p, desc, ch, a_s, ctx_s); break;
     case 3: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 3>(p, desc, ch, a_s, ctx_s); break;
     case 4: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 4>(p, desc, ch, a_s, ctx_s); break;
-    default: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0>(p, desc, ch, a_s, ctx_s); break;
+    default:
+      // wider bands with the taps in registers: the table is constant from band_k on, so the
+      // taps between band_k and the compiled width are the dense scan's own candidates
+      // (only with several labels per lane: the short chains of small label counts gain nothing
+      // and pay for the larger kernel)
+      if constexpr (R >= 2) {
+        if (desc.band_k <= 8) {
+          run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 8>(p, desc, ch, a_s, ctx_s);
+          break;
+        }
+        if (desc.band_k <= 16) {
+          run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 16>(p, desc, ch, a_s, ctx_s);
+          break;
+        }
+      }
+      run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0>(p, desc, ch, a_s, ctx_s);
+      break;
   }
 }
 
