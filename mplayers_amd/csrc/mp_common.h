@@ -91,15 +91,36 @@ __device__ __forceinline__ float uniform_f(float x) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
 }
 
-// min over the 64 lanes, returned wave-uniform
+// Order-preserving map between the bits of a float and a signed integer (its own inverse):
+// x < y  <=>  float_key(x) < float_key(y), with -0 below +0.
+__device__ __forceinline__ int float_key(int bits) { return bits ^ ((bits >> 31) & 0x7fffffff); }
+
+// min over the 64 lanes, returned wave-uniform.  The reduction runs on the integer keys: an integer
+// minimum folds each lane shift into the min instruction itself (the shifted-in lanes read the
+// identity INT_MAX), which the compiler does not do for a float minimum.
 __device__ __forceinline__ float wave_min(float x) {
+  const int top = 0x7fffffff;
+  int k = float_key(__builtin_bit_cast(int, x));
+  auto imin = [](int a, int b) { return a < b ? a : b; };
+  k = imin(k, __builtin_amdgcn_update_dpp(top, k, 0x111, 0xf, 0xf, false));  // row_shr:1
+  k = imin(k, __builtin_amdgcn_update_dpp(top, k, 0x112, 0xf, 0xf, false));  // row_shr:2
+  k = imin(k, __builtin_amdgcn_update_dpp(top, k, 0x114, 0xf, 0xf, false));  // row_shr:4
+  k = imin(k, __builtin_amdgcn_update_dpp(top, k, 0x118, 0xf, 0xf, false));  // row_shr:8: lane 15 of each row holds the row min
+  k = imin(k, __builtin_amdgcn_update_dpp(top, k, 0x142, 0xa, 0xf, false));  // row_bcast:15 into rows 1 and 3
+  k = imin(k, __builtin_amdgcn_update_dpp(top, k, 0x143, 0xc, 0xf, false));  // row_bcast:31 into rows 2 and 3
+  return __builtin_bit_cast(float, float_key(__builtin_amdgcn_readlane(k, 63)));
+}
+
+// the same on the float values themselves (three instructions per step instead of one, but no
+// conversions before and after: the shorter path where little else overlaps the reduction)
+__device__ __forceinline__ float wave_min_f32(float x) {
   const float inf = INFINITY;
-  x = fminf(x, dpp_f<0x111>(inf, x));       // row_shr:1
-  x = fminf(x, dpp_f<0x112>(inf, x));       // row_shr:2
-  x = fminf(x, dpp_f<0x114>(inf, x));       // row_shr:4
-  x = fminf(x, dpp_f<0x118>(inf, x));       // row_shr:8: lane 15 of each row holds the row min
-  x = fminf(x, dpp_f<0x142, 0xa>(inf, x));  // row_bcast:15 into rows 1 and 3
-  x = fminf(x, dpp_f<0x143, 0xc>(inf, x));  // row_bcast:31 into rows 2 and 3
+  x = fminf(x, dpp_f<0x111>(inf, x));
+  x = fminf(x, dpp_f<0x112>(inf, x));
+  x = fminf(x, dpp_f<0x114>(inf, x));
+  x = fminf(x, dpp_f<0x118>(inf, x));
+  x = fminf(x, dpp_f<0x142, 0xa>(inf, x));
+  x = fminf(x, dpp_f<0x143, 0xc>(inf, x));
   return readlane_f(x, 63);
 }
 

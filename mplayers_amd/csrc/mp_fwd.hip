@@ -517,7 +517,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         float vm = inf;
 #pragma unroll
         for (int j = 0; j < R; ++j) vm = fminf(vm, valid[j] ? v[j] : inf);
-        nmin = wave_min(vm);
+        nmin = (KT == -21) ? wave_min_f32(vm) : wave_min(vm);
       }
       float m[R], sn[R];
 #pragma unroll
