@@ -146,15 +146,17 @@ __device__ __forceinline__ int dpp_i(int old, int src) {
 // the rows of 16 lanes, then the row totals travel through the row broadcasts).  Suffix: lane i
 // gets the result over lanes i..63 (there is no broadcast in that direction: the three later row
 // totals are read back as scalars).
+// (the float scans run on the order-preserving integer keys, as wave_min does)
 __device__ __forceinline__ float lane_prefix_min(float x) {
-  const float inf = INFINITY;
-  x = fminf(x, dpp_f<0x111>(inf, x));
-  x = fminf(x, dpp_f<0x112>(inf, x));
-  x = fminf(x, dpp_f<0x114>(inf, x));
-  x = fminf(x, dpp_f<0x118>(inf, x));
-  x = fminf(x, dpp_f<0x142, 0xa>(inf, x));
-  x = fminf(x, dpp_f<0x143, 0xc>(inf, x));
-  return x;
+  constexpr int hi = 0x7fffffff;
+  int k = float_key(__builtin_bit_cast(int, x));
+  k = min(k, dpp_i<0x111>(hi, k));
+  k = min(k, dpp_i<0x112>(hi, k));
+  k = min(k, dpp_i<0x114>(hi, k));
+  k = min(k, dpp_i<0x118>(hi, k));
+  k = min(k, dpp_i<0x142, 0xa>(hi, k));
+  k = min(k, dpp_i<0x143, 0xc>(hi, k));
+  return __builtin_bit_cast(float, float_key(k));
 }
 __device__ __forceinline__ int lane_prefix_max(int x) {
   constexpr int lo = -0x7fffffff - 1;
@@ -165,18 +167,6 @@ __device__ __forceinline__ int lane_prefix_max(int x) {
   x = max(x, dpp_i<0x142, 0xa>(lo, x));
   x = max(x, dpp_i<0x143, 0xc>(lo, x));
   return x;
-}
-__device__ __forceinline__ float lane_suffix_min(float x, int lane) {
-  const float inf = INFINITY;
-  x = fminf(x, dpp_f<0x101>(inf, x));  // row_shl:1 ... 8: lane i of a row gets the row's lanes i..15
-  x = fminf(x, dpp_f<0x102>(inf, x));
-  x = fminf(x, dpp_f<0x104>(inf, x));
-  x = fminf(x, dpp_f<0x108>(inf, x));
-  const float r1 = readlane_f(x, 16), r2 = readlane_f(x, 32), r3 = readlane_f(x, 48);
-  const float m2 = fminf(r2, r3), m1 = fminf(r1, m2);
-  const int row = lane >> 4;
-  const float later = row == 0 ? m1 : (row == 1 ? m2 : (row == 2 ? r3 : inf));
-  return fminf(x, later);
 }
 __device__ __forceinline__ int lane_suffix_min(int x, int lane) {
   constexpr int hi = 0x7fffffff;
@@ -190,6 +180,10 @@ __device__ __forceinline__ int lane_suffix_min(int x, int lane) {
   const int row = lane >> 4;
   const int later = row == 0 ? m1 : (row == 1 ? m2 : (row == 2 ? r3 : hi));
   return min(x, later);
+}
+
+__device__ __forceinline__ float lane_suffix_min(float x, int lane) {
+  return __builtin_bit_cast(float, float_key(lane_suffix_min(float_key(__builtin_bit_cast(int, x)), lane)));
 }
 
 // largest label (R*lane + j) whose predicate is set; `dflt` when none is

@@ -49,9 +49,13 @@ __device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&val
       int cd = labc[j];
       int ci = ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : (cd > fd ? cd - fd : fd - cd);
       float val = fmaf(w, ctx_s[ci], af);
-      bool take = (fd == L - 1) || (val < v[j]);
-      v[j] = take ? val : v[j];
-      if (TRAIN) fd_idx[j] = take ? fd : fd_idx[j];
+      if (TRAIN) {
+        bool take = (fd == L - 1) || (val < v[j]);
+        v[j] = take ? val : v[j];
+        fd_idx[j] = take ? fd : fd_idx[j];
+      } else {
+        v[j] = fminf(v[j], val);
+      }
     }
   }
   __syncthreads();
@@ -63,7 +67,7 @@ __device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&val
 // label (c[|cd - (fd+1)|] of label cd is c[|(cd-1) - fd|] of label cd - 1; c[fd+1] enters at
 // label 0).  `<=` on the ascending scan keeps the largest front label among equals, as the
 // reference's descending scan with `<` does.
-template <int R, bool TRAIN>
+template <int R, bool TRAIN, bool WHOLE>  // WHOLE: L is a multiple of R
 __device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L, int lab0,
                                              const float* ctx_s, float (&v)[R], int (&fd_idx)[R]) {
   float c_own[R], cv[R];  // c[label] of the lane's labels; the sliding c[|label - fd|]
@@ -75,22 +79,29 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L
     v[j] = INFINITY;
     fd_idx[j] = L - 1;
   }
+  // the weight in a vector register: a multiply-add takes one scalar operand, and that is a[fd]
+  float wv = w;
+  asm volatile("" : "+v"(wv));
   for (int fd0 = 0; fd0 < L; fd0 += R) {
     const int src = fd0 / R;  // the lane that owns front labels fd0 .. fd0 + R - 1
 #pragma unroll
     for (int u = 0; u < R; ++u) {
       const int fd = fd0 + u;
-      if (fd < L) {  // wave-uniform; always true when L is a multiple of R
+      if (WHOLE || fd < L) {  // wave-uniform
         const float af = readlane_f(a[u], src);
         // c[fd + 1]: the next label's own entry (past the last label the value is never used)
         const float cn = u + 1 < R ? readlane_f(c_own[u + 1 < R ? u + 1 : 0], src)
                                    : readlane_f(c_own[0], (src + 1) & 63);
 #pragma unroll
         for (int j = 0; j < R; ++j) {
-          const float val = fmaf(w, cv[j], af);
-          const bool take = val <= v[j];
-          v[j] = take ? val : v[j];
-          if (TRAIN) fd_idx[j] = take ? fd : fd_idx[j];
+          const float val = fmaf(wv, cv[j], af);
+          if (TRAIN) {
+            const bool take = val <= v[j];
+            v[j] = take ? val : v[j];
+            fd_idx[j] = take ? fd : fd_idx[j];
+          } else {
+            v[j] = fminf(v[j], val);
+          }
         }
         const float in0 = wave_shr1(cv[R - 1], cn);
 #pragma unroll
@@ -114,9 +125,13 @@ __device__ __forceinline__ void dense_step_r1(float a, int L, float w, int lane,
   for (int fd = L - 1; fd >= 0; --fd) {
     const float af = readlane_f(a, fd);
     const float val = fmaf(w, col[fd * L], af);
-    const bool take = (fd == L - 1) || (val < best);
-    best = take ? val : best;
-    if (TRAIN) arg = take ? fd : arg;
+    if (TRAIN) {
+      const bool take = (fd == L - 1) || (val < best);
+      best = take ? val : best;
+      arg = take ? fd : arg;
+    } else {
+      best = fminf(best, val);
+    }
   }
   v = best;
   fd_idx = arg;
@@ -492,9 +507,13 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
 #pragma unroll
           for (int fd = LT - 1; fd >= 0; --fd) {
             const float val = fmaf(w, tcol[fd], readlane_f(a[0], fd));
-            const bool take = (fd == LT - 1) || (val < best);
-            best = take ? val : best;
-            if (TRAIN) arg = take ? fd : arg;
+            if (TRAIN) {
+              const bool take = (fd == LT - 1) || (val < best);
+              best = take ? val : best;
+              arg = take ? fd : arg;
+            } else {
+              best = fminf(best, val);
+            }
           }
           v[0] = best;
           fd_idx[0] = arg;
@@ -503,7 +522,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         }
       } else if (live) {
         if constexpr (R > 1)  // (2-D tables exist for one label per lane only)
-          dense1d_step<R, TRAIN>(a, w, L, lab0, ctx_s, v, fd_idx);
+          dense1d_step<R, TRAIN, VEC>(a, w, L, lab0, ctx_s, v, fd_idx);
         else
           dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
       } else {
