@@ -785,6 +785,12 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   // rho = 1 its sweeps read `unary` itself and the pass that would store U is skipped (the
   // sweeps write every element of their output buffer, chain starts included).
   const bool unary_as_u = s->msg_uninit != 0 && rho == 1.f;
+  // Four directions at rho = 1: U of a pair of opposite directions is the unary plus the two
+  // messages of the other pair, so the scans can form it on the fly (3 planes read per direction
+  // instead of 1) and the pass that stores U (5 planes in, 2 out per iteration) is dropped; with
+  // more directions the scans would read more than that pass moves.  (Not for the packed scans
+  // of small label counts.)
+  const bool fuse_u = s->n_dir == 4 && rho == 1.f && s->n_disp > 32;
   if (s->msg_uninit != 0 && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {
@@ -797,9 +803,16 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
     const bool out_of_place = (it == 0) && (n_iter & 1);
     float* ubuf = out_of_place ? other : have;
     float* nxt = out_of_place ? have : other;
+    p.u_fused = 0;
     if (it == 0 && unary_as_u) {
       p.msg_in = unary;
       p.u_stride = 0;
+    } else if (fuse_u && !out_of_place) {
+      // the scans read the unary and the old messages of the other pair of directions themselves
+      p.belief = unary;
+      p.msg_in = have;
+      p.u_stride = N;
+      p.u_fused = 1;
     } else {
       Timed timed(MPL_KERNEL_UNARY_ALL, st);
       const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update);

@@ -438,6 +438,8 @@ struct SweepParams {
   int u_pair_share;                // Jacobi: directions d and d^1 read the U plane of the even one
   int64_t u_stride;                // Jacobi: elements between the U planes of msg_in (0: all directions
                                    // read the one plane at msg_in)
+  int u_fused;                     // Jacobi, four directions, rho == 1: `belief` is the unary and msg_in
+                                   // holds the old messages themselves; the scans form U on the fly
   int zero_start;                  // Gauss-Seidel: store zeros at the chain start of msg_out (the
                                    // caller's buffer is undefined and this is its first sweep)
   float* edge_label;               // soft TRWP: (n_dir_total, P, L, L) duals of this iteration, or null

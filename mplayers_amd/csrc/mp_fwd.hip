@@ -318,7 +318,7 @@ __device__ __forceinline__ void linear_step(const float (&a)[R], float w, float 
 // One chain.  KT: > 0 band with compile-time K, 0 band with run-time K, -1 dense, -21 dense with
 // exactly 21 labels, -2 truncated linear context of any width (linear_step).
 // VEC: L % R == 0 (vector accesses).  MASK: some lanes own labels >= L.
-template <int R, bool VEC, bool MASK, bool TRAIN, bool JACOBI, int KT>
+template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI, int KT>
 __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
                                               const ChainCtx& ch, float* a_s, const float* ctx_s) {
   const int L = p.L;
@@ -332,10 +332,14 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // plane bases of this batch item and direction; descriptors are formed per access
   // Jacobi: the plane of this direction in msg_in holds U itself (written by the host's
   // element-wise pass before the sweeps), so one plane is read per pixel instead of three
+  // JACOBI == 2 (four directions, rho == 1): no U plane either; U of the pair {dir, dir^1} is the
+  // unary plus the old messages of the other pair, read here (three planes in, but the pass that
+  // stores U, five planes in and two out per iteration, is not run)
+  const int oth = (dir & ~1) ^ 2;  // the even direction of the other pair
   const float* __restrict__ bS =
-      (JACOBI ? p.msg_in + (int64_t)(p.u_pair_share ? (dir & ~1) : dir) * p.u_stride : p.belief) + img_e;
-  const float* __restrict__ bMd = p.msg_in + (int64_t)dir * N + img_e;
-  const float* __restrict__ bMi = p.msg_in + (int64_t)(dir ^ 1) * N + img_e;
+      (JACOBI == 1 ? p.msg_in + (int64_t)(p.u_pair_share ? (dir & ~1) : dir) * p.u_stride : p.belief) + img_e;
+  const float* __restrict__ bMd = p.msg_in + (int64_t)(JACOBI == 2 ? oth : dir) * N + img_e;
+  const float* __restrict__ bMi = p.msg_in + (int64_t)(JACOBI == 2 ? oth + 1 : (dir ^ 1)) * N + img_e;
   float* __restrict__ bMo = p.msg_out + (int64_t)dir * N + img_e;
   float* __restrict__ bSo = (JACOBI ? nullptr : p.belief_out + img_e);
   uint8_t* __restrict__ bImin = TRAIN ? p.idx_min + (int64_t)dir * N + img_e : nullptr;
@@ -392,11 +396,14 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     const unsigned so = pp * (unsigned)vbytes;
     const int nrec = (int)(so + (unsigned)vbytes);
     buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
-    if (!JACOBI) {
+    if (JACOBI == 0) {
       // planes that still hold all-zero initial messages are read through an empty descriptor
       buf_load<R, VEC>(make_rsrc(bMd, (md_zero || (pair_second && ld_t > 0)) ? 0 : nrec), foff, so,
                        r.md);
       buf_load<R, VEC>(make_rsrc(bMi, mi_zero ? 0 : nrec), foff, so, r.mi);
+    } else if (JACOBI == 2) {
+      buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
+      buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
     }
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
     ld_p += ch.pstep;
@@ -415,7 +422,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
 #pragma unroll
     for (int j = 0; j < R; ++j) {
       prev[j] = 0.f;
-      float un = p0.s[j];
+      float un = JACOBI == 2 ? (p0.s[j] + p0.md[j]) + p0.mi[j] : p0.s[j];
       if (!JACOBI) {
         const float t0 = pair_second ? p0.s[j] + p0.mi[j] : p0.s[j] - p0.md[j];
         un = fmaf(t0, rho, -p0.mi[j]);
@@ -438,7 +445,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
 
   // memory instructions per step: 1 or 3 label vectors + the weight in, 1-2 label vectors
   // (+ indices) out
-  constexpr int kOps = (JACOBI ? 1 : 3) * vec_ops(R, VEC) + 1 + (JACOBI ? 1 : 2) * vec_ops(R, VEC) +
+  constexpr int kOps = (JACOBI == 1 ? 1 : 3) * vec_ops(R, VEC) + 1 + (JACOBI ? 1 : 2) * vec_ops(R, VEC) +
                        (TRAIN ? byte_ops(R, VEC) + 1 : 0);
   constexpr int D = ring_depth(kOps);
   PixF<R> ring[D];
@@ -458,7 +465,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       float tt[R], un[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) {
-        float x = px.s[j];
+        float x = JACOBI == 2 ? (px.s[j] + px.md[j]) + px.mi[j] : px.s[j];
         if (!JACOBI) {
           // unary + the other directions' messages
           tt[j] = pair_second ? px.s[j] + px.mi[j] : px.s[j] - px.md[j];
@@ -566,7 +573,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   }
 }
 
-template <int R, bool VEC, bool MASK, bool TRAIN, bool JACOBI>
+template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI>
 __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
   extern __shared__ float smem[];
   float* a_s = smem;            // kMaxL floats
@@ -640,16 +647,21 @@ template <int R, bool VEC, bool MASK>
 void launch_vm(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = fwd_lds_bytes(p.L, p.ctx2d);
+  const int mode = jacobi ? (p.u_fused ? 2 : 1) : 0;
   if (train) {
-    if (jacobi)
-      sweep_fwd_kernel<R, VEC, MASK, true, true><<<blocks, kWave, lds, st>>>(p);
+    if (mode == 2)
+      sweep_fwd_kernel<R, VEC, MASK, true, 2><<<blocks, kWave, lds, st>>>(p);
+    else if (mode == 1)
+      sweep_fwd_kernel<R, VEC, MASK, true, 1><<<blocks, kWave, lds, st>>>(p);
     else
-      sweep_fwd_kernel<R, VEC, MASK, true, false><<<blocks, kWave, lds, st>>>(p);
+      sweep_fwd_kernel<R, VEC, MASK, true, 0><<<blocks, kWave, lds, st>>>(p);
   } else {
-    if (jacobi)
-      sweep_fwd_kernel<R, VEC, MASK, false, true><<<blocks, kWave, lds, st>>>(p);
+    if (mode == 2)
+      sweep_fwd_kernel<R, VEC, MASK, false, 2><<<blocks, kWave, lds, st>>>(p);
+    else if (mode == 1)
+      sweep_fwd_kernel<R, VEC, MASK, false, 1><<<blocks, kWave, lds, st>>>(p);
     else
-      sweep_fwd_kernel<R, VEC, MASK, false, false><<<blocks, kWave, lds, st>>>(p);
+      sweep_fwd_kernel<R, VEC, MASK, false, 0><<<blocks, kWave, lds, st>>>(p);
   }
 }
 

@@ -450,6 +450,7 @@ int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains) {
 void set_packed_policy(bool always) { g_pack_always = always; }
 
 bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, hipStream_t st) {
+  if (p0.u_fused) return false;  // (set for more than 32 labels only)
   const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0));
   if (G < 2) return false;
   const SweepParams p = with_wave_prefix(p0, G);

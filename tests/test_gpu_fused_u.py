@@ -1,0 +1,90 @@
+"""ISGMR with four directions and more than 32 labels forms U inside the scans (no U pass).  The
+message buffers then alternate differently from the pass-based schedule, so every combination of
+iteration-count parity, cleared / declared-zero / non-zero initial messages and training /
+inference is checked against the oracle, and against the pass-based schedule of the library itself
+(rho slightly off 1 switches the fused mode off; at 8 directions it is never on)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(L, n_iter, seed, H=7, W=9, B=2, n_dir=4):
+  rng = np.random.default_rng(seed)
+  k = np.arange(L, dtype=np.float32)
+  kind = seed % 3
+  if kind == 0:
+    ctx = (0.3 * np.minimum(k, 3)).astype(np.float32)              # band in registers
+  elif kind == 1:
+    ctx = (0.02 * np.minimum(k * k, 150)).astype(np.float32)       # wide band
+  else:
+    ctx = rng.random(L).astype(np.float32)                         # dense
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ew = (0.1 + rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  return unary, ctx, ew
+
+
+@pytest.mark.parametrize("train", [True, False])
+@pytest.mark.parametrize("n_iter", [1, 2, 3, 4])
+@pytest.mark.parametrize("L", [33, 96, 256])
+def test_fused_u_matches_oracle(gpu, oracle, L, n_iter, train):
+  unary, ctx, ew = _case(L, n_iter, seed=L + n_iter)
+  ref = oracle.forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, saving_label=True, want_gaps=True)
+  got = gpu.gpu_forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, training=train, saving_label=True)
+  belief = ref["cost_final"]
+  tol = 1e-5 * max(1.0, float(np.abs(belief).max()))
+  gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=belief)
+  gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost")
+  if train:
+    gpu.assert_indices_match_off_ties(got["msg_min_index"], ref["msg_min_index"], ref["gap_min"],
+                                      4 * tol, "min index")
+    gpu.assert_indices_match_off_ties(got["msg_norm_index"], ref["msg_norm_index"], ref["gap_norm"],
+                                      4 * tol, "norm index")
+
+
+@pytest.mark.parametrize("n_iter", [1, 2, 3])
+def test_fused_u_with_initial_messages(gpu, oracle, n_iter):
+  """Non-zero initial messages (the operator interface allows them) go through the fused scans
+  from the first iteration when the iteration count is even."""
+  L = 64
+  unary, ctx, ew = _case(L, n_iter, seed=77)
+  rng = np.random.default_rng(5)
+  msg0 = rng.random((4,) + unary.shape).astype(np.float32)
+  msg0 -= msg0.min(axis=-1, keepdims=True)
+  ref = oracle.forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, msg_init=msg0)
+  got = gpu.gpu_forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, msg_init=msg0)
+  gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=ref["cost_final"])
+  gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost")
+
+
+@pytest.mark.parametrize("uninit", [False, True])
+@pytest.mark.parametrize("n_iter", [2, 3])
+def test_fused_u_integer_inputs_are_bit_exact(gpu, oracle, n_iter, uninit):
+  """On integer-valued inputs no sum rounds, so the fused schedule, the pass-based one and the
+  oracle agree bit for bit, indices included."""
+  import torch
+  from mplayers_amd import lib_stereo
+  L, B, H, W = 96, 1, 6, 8
+  rng = np.random.default_rng(11 + n_iter)
+  unary = rng.integers(0, 9, size=(B, 1, H, W, L)).astype(np.float32)
+  ctx = np.minimum(np.arange(L), 4).astype(np.float32)
+  ew = rng.integers(1, 3, size=(4, B, 1, H, W)).astype(np.float32)
+  ref = oracle.forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, saving_label=True)
+  dev = "cuda"
+  u8 = dict(dtype=torch.uint8, device=dev)
+  t = lambda a: torch.from_numpy(a).to(dev)
+  msg = torch.full((4, B, 1, H, W, L), float("nan") if uninit else 0.0, device=dev)
+  msg_tmp = torch.full_like(msg, float("nan"))
+  cost = torch.zeros(B, 1, H, W, L, device=dev)
+  scratch = torch.zeros_like(cost)
+  imin = torch.zeros(n_iter, 4, B, 1, H, W, L, **u8)
+  inorm = torch.zeros(n_iter, 4, B, 1, H, W, **u8)
+  label = torch.zeros(n_iter, B, 1, H, W, **u8)
+  lib_stereo.ISGMR.forward(0, 1.0, n_iter, 0, t(unary), t(ctx), t(ew), msg, cost, imin, inorm, scratch,
+                           msg_tmp, label, msg_uninit=uninit)
+  torch.cuda.synchronize()
+  assert np.array_equal(msg.cpu().numpy(), ref["msg"])
+  assert np.array_equal(cost.cpu().numpy(), ref["cost_final"])
+  assert np.array_equal(imin.cpu().numpy(), ref["msg_min_index"])
+  assert np.array_equal(inorm.cpu().numpy(), ref["msg_norm_index"])
+  assert np.array_equal(label.cpu().numpy(), ref["label_all"])
