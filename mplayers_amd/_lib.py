@@ -68,10 +68,14 @@ def load():
   policy = os.environ.get("MPLAYERS_PACKED_SCANS")  # 0 | 1 | 2, see mpl_set_option
   if policy is not None:
     check(lib.mpl_set_option(OPT_PACKED_SCANS, int(policy)), "set_option")
+  fused = os.environ.get("MPLAYERS_FUSED_U")  # 0 | 1, see mpl_set_option
+  if fused is not None:
+    check(lib.mpl_set_option(OPT_FUSED_U, int(fused)), "set_option")
   return lib
 
 
 OPT_PACKED_SCANS = 0
+OPT_FUSED_U = 1
 
 
 def set_option(option, value):

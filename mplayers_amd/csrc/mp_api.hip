@@ -546,6 +546,7 @@ void fill_dirs(const mpl_shape* s, int first, int count, int* dirs, int* prefix,
 int labels_per_lane(int L) { return (L + kWave - 1) / kWave; }
 
 bool g_packed_scans = true;  // mpl_set_option(MPL_OPT_PACKED_SCANS, ...)
+bool g_fused_u = true;       // mpl_set_option(MPL_OPT_FUSED_U, ...)
 
 void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st);
@@ -636,6 +637,11 @@ int mpl_set_option(int option, int value) {
     if (value < 0 || value > 2) return fail(MPL_EINVAL, "set_option: packed scans take 0, 1 or 2");
     g_packed_scans = value != 0;
     set_packed_policy(value == 2);
+    return MPL_OK;
+  }
+  if (option == MPL_OPT_FUSED_U) {
+    if (value < 0 || value > 1) return fail(MPL_EINVAL, "set_option: fused U takes 0 or 1");
+    g_fused_u = value != 0;
     return MPL_OK;
   }
   return fail(MPL_EINVAL, "set_option: unknown option %d", option);
@@ -790,7 +796,7 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   // instead of 1) and the pass that stores U (5 planes in, 2 out per iteration) is dropped; with
   // more directions the scans would read more than that pass moves.  (Not for the packed scans
   // of small label counts.)
-  const bool fuse_u = s->n_dir == 4 && rho == 1.f && s->n_disp > 32;
+  const bool fuse_u = g_fused_u && s->n_dir == 4 && rho == 1.f && s->n_disp > 32;
   if (s->msg_uninit != 0 && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {

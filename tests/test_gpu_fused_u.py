@@ -2,7 +2,7 @@
 message buffers then alternate differently from the pass-based schedule, so every combination of
 iteration-count parity, cleared / declared-zero / non-zero initial messages and training /
 inference is checked against the oracle, and against the pass-based schedule of the library itself
-(rho slightly off 1 switches the fused mode off; at 8 directions it is never on)."""
+(MPL_OPT_FUSED_U = 0)."""
 import numpy as np
 import pytest
 
@@ -88,3 +88,20 @@ def test_fused_u_integer_inputs_are_bit_exact(gpu, oracle, n_iter, uninit):
   assert np.array_equal(imin.cpu().numpy(), ref["msg_min_index"])
   assert np.array_equal(inorm.cpu().numpy(), ref["msg_norm_index"])
   assert np.array_equal(label.cpu().numpy(), ref["label_all"])
+
+
+@pytest.mark.parametrize("n_iter", [2, 5])
+def test_fused_u_agrees_with_the_u_pass(gpu, n_iter):
+  """The same call with the fused mode switched off (the library stores U in a pass of its own):
+  same messages and costs to the parity tolerance, same labels off ties."""
+  from mplayers_amd import _lib
+  unary, ctx, ew = _case(160, n_iter, seed=3, H=9, W=11)
+  try:
+    _lib.set_option(_lib.OPT_FUSED_U, 0)
+    want = gpu.gpu_forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, training=False, saving_label=True)
+  finally:
+    _lib.set_option(_lib.OPT_FUSED_U, 1)
+  got = gpu.gpu_forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, training=False, saving_label=True)
+  gpu.assert_values_close(got["msg"], want["msg"], what="msg", belief=want["cost_final"])
+  gpu.assert_values_close(got["cost_final"], want["cost_final"], what="cost")
+  assert (got["label_all"] != want["label_all"]).mean() < 0.01
