@@ -20,10 +20,11 @@ using namespace mpl;
 
 namespace {
 
-// 1-D context c[0..L-1]: find the constant tail.  One wave.
+// 1-D context c[0..L-1]: find the constant tail and recognise a truncated linear table.  One wave,
+// every lane looks at the entries lane, lane + 64, ...; the findings are combined with ballots.
 __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __restrict__ ctx, int L,
                                                                 int ctx2d, CtxDesc* __restrict__ d) {
-  if (threadIdx.x != 0) return;
+  const int lane = threadIdx.x;
   CtxDesc r;
   r.band_k = 0;
   r.c0_is_min = 0;
@@ -32,35 +33,36 @@ __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __r
   r.linear = 0;
   r.slope = 0.f;
   if (!ctx2d) {
-    float tail = ctx[L - 1];
-    int k = L - 1;
-    while (k > 0 && ctx[k - 1] == tail) --k;  // c[k..L-1] == tail
-    bool ok = (tail == tail);
-    bool c0min = true;
-    for (int i = 0; i < L; ++i) {
-      float v = ctx[i];
-      if (!(v <= tail)) ok = false;
-      if (!(ctx[0] <= v)) c0min = false;
+    const float tail = ctx[L - 1];
+    const float c0 = ctx[0];
+    const float slope = L >= 2 ? ctx[1] : 0.f;
+    int last_ne = -1;  // largest index whose entry differs from the tail
+    bool below = true, c0min = true, lin = true;
+    for (int i = lane; i < L; i += kWave) {
+      const float v = ctx[i];
+      if (!(v == tail)) last_ne = i;
+      below = below && (v <= tail);
+      c0min = c0min && (c0 <= v);
+      lin = lin && (v == fminf(slope * (float)i, tail));
     }
+    int k = (int)-wave_min(-(float)last_ne) + 1;  // c[k..L-1] == tail  (indices < 2^24: exact)
+    const bool ok = (tail == tail) && ballot(!below) == 0;
+    const bool all_c0min = ballot(!c0min) == 0;
+    const bool all_lin = ballot(!lin) == 0;
     if (k < 1) k = 1;  // a constant context: the centre tap alone is the band
     if (ok && k <= kMaxBandK) {
       r.band_k = k;
       r.cmax = tail;
-      r.c0_is_min = c0min ? 1 : 0;
+      r.c0_is_min = all_c0min ? 1 : 0;
     }
     // truncated linear, bit for bit: c[k] == min(c[1] * k, c[L-1])
-    if (ok && L >= 2 && ctx[0] == 0.f && ctx[1] >= 0.f) {
-      const float slope = ctx[1];
-      bool lin = true;
-      for (int i = 0; i < L; ++i) lin = lin && (ctx[i] == fminf(slope * (float)i, tail));
-      if (lin) {
-        r.linear = 1;
-        r.slope = slope;
-        r.cmax = tail;
-      }
+    if (ok && L >= 2 && c0 == 0.f && slope >= 0.f && all_lin) {
+      r.linear = 1;
+      r.slope = slope;
+      r.cmax = tail;
     }
   }
-  *d = r;
+  if (lane == 0) *d = r;
 }
 
 // ------------------------------------------------------------------------------------------------
