@@ -40,6 +40,8 @@ def parse():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--config", default="C5")
   ap.add_argument("--scale", type=float, default=1.0, help="shrink H and W (debugging only)")
+  ap.add_argument("--n-dir", type=int, default=None, choices=[2, 4, 8, 16],
+                  help="run the configuration on another connectivity (not the headline workload)")
   ap.add_argument("--alg", default="both", choices=["both", "TRWP", "ISGMR", "SOFT"],
                   help="SOFT: soft-weighted TRWP (at most 64 labels; stores n_disp^2 floats per "
                        "pixel, direction and iteration)")
@@ -240,7 +242,7 @@ def main():
   dev = torch.device("cuda:0")
   torch.cuda.set_device(dev)
 
-  cfg = synthetic.make_config(a.config, seed=0, scale=a.scale)
+  cfg = synthetic.make_config(a.config, seed=0, scale=a.scale, n_dir=a.n_dir)
   B, H, W, L, n_dir, n_iter = (cfg[k] for k in ("B", "H", "W", "L", "n_dir", "n_iter"))
   algs = ["TRWP", "ISGMR"] if a.alg == "both" else [a.alg]
   training = not a.fwd_only

@@ -90,7 +90,7 @@ CONFIGS = {
 }
 
 
-def make_config(name, seed=0, scale=1.0, mode=None):
+def make_config(name, seed=0, scale=1.0, mode=None, n_dir=None):
   """Builds the inputs of configuration `name` (C1..C5).  scale < 1 shrinks H and W (parity tests
   at sizes a CPU checker finishes in seconds); mode overrides TRWP/ISGMR for the two-algorithm
   configurations.  Returns a dict with the config fields plus unary, context, edge_weights."""
@@ -99,6 +99,8 @@ def make_config(name, seed=0, scale=1.0, mode=None):
     cfg["mode"] = mode
     cfg["rho"] = 0.5 if mode == "TRWP" else 1.0
   cfg["name"] = name
+  if n_dir is not None:
+    cfg["n_dir"] = int(n_dir)  # the same problem on another connectivity (2, 4, 8 or 16 directions)
   H = cfg["H"] = max(2, int(round(cfg["H"] * scale)))
   W = cfg["W"] = max(2, int(round(cfg["W"] * scale)))
   B, L, n_dir = cfg["B"], cfg["L"], cfg["n_dir"]
