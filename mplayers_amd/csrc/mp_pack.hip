@@ -228,17 +228,25 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
 #pragma unroll
         for (int fd = LT - 1; fd >= 0; --fd) {
           const float val = fmaf(w, tcol[fd], bperm_f(sg.first + fd * 4, a));
-          const bool take = (fd == LT - 1) || (val < best);
-          best = take ? val : best;
-          if (TRAIN) arg = take ? fd : arg;
+          if (TRAIN) {
+            const bool take = (fd == LT - 1) || (val < best);
+            best = take ? val : best;
+            arg = take ? fd : arg;
+          } else {
+            best = fminf(best, val);
+          }
         }
       } else {
 #pragma unroll 4
         for (int fd = L - 1; fd >= 0; --fd) {
           const float val = fmaf(w, tab[fd * L + l], bperm_f(sg.first + fd * 4, a));
-          const bool take = (fd == L - 1) || (val < best);
-          best = take ? val : best;
-          if (TRAIN) arg = take ? fd : arg;
+          if (TRAIN) {
+            const bool take = (fd == L - 1) || (val < best);
+            best = take ? val : best;
+            arg = take ? fd : arg;
+          } else {
+            best = fminf(best, val);
+          }
         }
       }
       const float nmin = seg_min(sg, on ? best : inf);  // MsgNormNaive, commonCUDA.cuh:92-129
