@@ -14,7 +14,8 @@
  *   msg_min_index   (n_iter, n_dir, B, H, W, L) uint8      msg_norm_index (n_iter, n_dir, B, H, W) uint8
  *   label_all       (n_iter, B, H, W) uint8
  *   context         ctx2d ? (L, L), entries [min(a,b)*L + max(a,b)] read : >= L floats, [|a-b|] read
- *   dcontext        same shape as context (zero-filled; only off-diagonal / k>=1 entries are written)
+ *   dcontext        same shape as context (zero-filled; only off-diagonal / k>=1 entries are written,
+ *                   unless MPL_F_DCONTEXT_SAME_LABEL is given)
  *
  * Return value: 0 on success, a negative MPL_E* code otherwise; mpl_last_error() then returns a
  * message for the calling thread.  On error nothing has been launched.
@@ -42,27 +43,47 @@ typedef struct mpl_shape {
   int width;
   int n_disp; /* labels, <= MPL_MAX_LABELS */
   int ctx2d;  /* 1: (L,L) context table (the reference selects it by n_disp == 21); needs L <= 64 */
-  int msg_uninit; /* forward calls only.  0: `msg` holds the initial messages (the reference's
-               * contract: the caller zero-fills it).  1: the contents of `msg` on entry are
-               * ignored; the messages start at zero and the library writes every element itself,
-               * which saves the caller's memset and the passes that would read the zeros back */
 } mpl_shape;
+
+/* Per-call flags, the `flags` argument of the forward and backward entry points (no counterpart in
+ * the reference).  0 is the reference's contract with the process defaults of mpl_set_option().
+ * A flag a call has no use for is ignored; unknown bits are rejected with MPL_EINVAL. */
+#define MPL_F_MSG_UNINIT 0x01u
+/* forward calls.  Without it `msg` holds the initial messages (the reference's contract: the
+ * caller zero-fills it).  With it the contents of `msg` on entry are ignored: the messages start at
+ * zero and the library writes every element itself, which saves the caller's memset and the passes
+ * that would read the zeros back. */
+#define MPL_F_PACKED_OFF 0x02u
+#define MPL_F_PACKED_ALWAYS 0x04u
+/* scans of at most 32 labels with several chains per wavefront: never / whenever the label count
+ * allows it, for this call (neither bit: the process default, see MPL_OPT_PACKED_SCANS). */
+#define MPL_F_FUSED_U_OFF 0x08u
+/* ISGMR forward: always run the pass that stores U (see MPL_OPT_FUSED_U). */
+#define MPL_F_DCONTEXT_SAME_LABEL 0x10u
+/* hard backward calls: dcontext also collects the pairs whose front label equals their own label
+ * (entry 0 of a 1-D table, the diagonal of a 2-D one), as the hard operator of the reference's
+ * TRWP_hard_soft build does (MPLayers/TRWP_hard_soft/TRWP_backward.cu:104-111, 188-195, 258-265);
+ * the TRWP and ISGMR builds skip them (MPLayers/TRWP/TRWP_backward.cu:111-112). */
+#define MPL_F_ALL 0x1fu
 
 /* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.
  * msg: initial messages in, final normalised messages out.  msg_min_index/msg_norm_index NULL =>
  * inference (no index stores).  label_all NULL => no per-iteration labels.  unary_update: scratch
  * plane (carries the running belief during the call).  cost_final doubles as scratch until the final aggregation. */
-int mpl_trwp_forward(const mpl_shape* shape, float rho, int n_iter, int enable_min_a_dir,
-                     const float* unary, const float* context, const float* edge_weights,
-                     float* msg, float* cost_final, uint8_t* msg_min_index,
-                     uint8_t* msg_norm_index, float* unary_update, uint8_t* label_all,
-                     void* stream);
+int mpl_trwp_forward(const mpl_shape* shape, unsigned flags, float rho, int n_iter,
+                     int enable_min_a_dir, const float* unary, const float* context,
+                     const float* edge_weights, float* msg, float* cost_final,
+                     uint8_t* msg_min_index, uint8_t* msg_norm_index, float* unary_update,
+                     uint8_t* label_all, void* stream);
 
 /* Replaces lib_*.TRWP.backward: MPLayers/TRWP/TRWP.cpp:285-318 -> TRWP_backward.cu:277-433.
  * dunary receives the gradient; dcontext and dedge_weights (zero-filled) accumulate; dmsg is
- * scratch (n_dir planes, any contents); dunary_update is accepted and unused. */
-int mpl_trwp_backward(const mpl_shape* shape, float rho, int n_iter, const float* context,
-                      const float* edge_weights, const float* dcost_final,
+ * scratch (n_dir planes, any contents); dunary_update is accepted and unused.
+ * dcontext and / or dedge_weights may be NULL when the caller has no use for that gradient (a fixed
+ * pairwise table, edge weights that are not learned): the reverse scans then leave that part of
+ * their step out; dunary is the same bit for bit. */
+int mpl_trwp_backward(const mpl_shape* shape, unsigned flags, float rho, int n_iter,
+                      const float* context, const float* edge_weights, const float* dcost_final,
                       const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
                       float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
                       void* stream);
@@ -70,19 +91,21 @@ int mpl_trwp_backward(const mpl_shape* shape, float rho, int n_iter, const float
 /* Replaces lib_*.ISGMR.forward: MPLayers/ISGMR/ISGMR.cpp:300-342 -> ISGMR_forward.cu:433-665.
  * msg_update: second message buffer (any contents); on return msg holds the final messages,
  * msg_update intermediate values; unary_update is accepted and unused. */
-int mpl_isgmr_forward(const mpl_shape* shape, int enable_sgm, float rho, int n_iter,
-                      int enable_min_a_dir, const float* unary, const float* context,
+int mpl_isgmr_forward(const mpl_shape* shape, unsigned flags, int enable_sgm, float rho,
+                      int n_iter, int enable_min_a_dir, const float* unary, const float* context,
                       const float* edge_weights, float* msg, float* cost_final,
                       uint8_t* msg_min_index, uint8_t* msg_norm_index, float* unary_update,
                       float* msg_update, uint8_t* label_all, void* stream);
 
 /* Replaces lib_*.ISGMR.backward: MPLayers/ISGMR/ISGMR.cpp:344-379 -> ISGMR_backward.cu:290-493.
  * dmsg_update and dmsg are scratch (n_dir planes each, any contents); dmsg may be NULL (the pass
- * then works in place in dmsg_update and moves somewhat more data); dunary_update is unused. */
-int mpl_isgmr_backward(const mpl_shape* shape, int enable_sgm, float rho, int n_iter,
-                       const float* context, const float* edge_weights, const float* dcost_final,
-                       const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
-                       float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
+ * then works in place in dmsg_update and moves somewhat more data); dunary_update is unused.
+ * dcontext and / or dedge_weights may be NULL, as for mpl_trwp_backward. */
+int mpl_isgmr_backward(const mpl_shape* shape, unsigned flags, int enable_sgm, float rho,
+                       int n_iter, const float* context, const float* edge_weights,
+                       const float* dcost_final, const uint8_t* msg_min_index,
+                       const uint8_t* msg_norm_index, float* dunary, float* dcontext,
+                       float* dedge_weights, float* dmsg, float* dunary_update,
                        float* dmsg_update, void* stream);
 
 /* Soft-weighted TRWP: replaces lib_*.TRWP_hard_soft.forward_soft, MPLayers/TRWP_hard_soft/TRWP.cpp:
@@ -91,19 +114,20 @@ int mpl_isgmr_backward(const mpl_shape* shape, int enable_sgm, float rho, int n_
  *   msg_edge_label (n_iter, n_dir, B, H, W, L, L) fp32: every dual of every pixel, kept for the
  *   backward pass (even directions [fd][cd], odd ones [cd][fd]); blocks of chain-start pixels are
  *   not written.  NULL together with msg_norm_index => inference. */
-int mpl_trwp_soft_forward(const mpl_shape* shape, float rho, int n_iter, const float* unary,
-                          const float* context, const float* edge_weights, float* msg,
-                          float* msg_edge_label, uint8_t* msg_norm_index, float* cost_final,
-                          float* unary_update, uint8_t* label_all, void* stream);
+int mpl_trwp_soft_forward(const mpl_shape* shape, unsigned flags, float rho, int n_iter,
+                          const float* unary, const float* context, const float* edge_weights,
+                          float* msg, float* msg_edge_label, uint8_t* msg_norm_index,
+                          float* cost_final, float* unary_update, uint8_t* label_all,
+                          void* stream);
 
 /* Replaces lib_*.TRWP_hard_soft.backward_soft, TRWP.cpp:351-383 (BackwardSoft) ->
  * TRWP_backward_soft.cu:422-548.  dcontext also receives the zero-offset / diagonal terms here
  * (the hard operator skips them).  dmsg is scratch (n_dir planes, any contents). */
-int mpl_trwp_soft_backward(const mpl_shape* shape, float rho, int n_iter, const float* dcost_final,
-                           const float* context, const float* edge_weights,
-                           const float* msg_edge_label, const uint8_t* msg_norm_index,
-                           float* dunary, float* dcontext, float* dedge_weights, float* dmsg,
-                           float* dunary_update, void* stream);
+int mpl_trwp_soft_backward(const mpl_shape* shape, unsigned flags, float rho, int n_iter,
+                           const float* dcost_final, const float* context,
+                           const float* edge_weights, const float* msg_edge_label,
+                           const uint8_t* msg_norm_index, float* dunary, float* dcontext,
+                           float* dedge_weights, float* dmsg, float* dunary_update, void* stream);
 
 /* Stand-alone softmin of stored blocks: replaces lib_*.TRWP_hard_soft.soft_weighted_message and
  * soft_weighted_message_back, TRWP.cpp:385-417 -> TRWP_swbp.cu:131-321.  message (n_trees, L, L)
@@ -226,7 +250,9 @@ int mpl_transpose(const float* src, float* dst, int batch, int64_t rows, int64_t
 /* Message of the last failed call on this thread ("" if none). */
 const char* mpl_last_error(void);
 
-/* Process-wide switches (no counterpart in the reference).
+/* Process-wide defaults of what the per-call flags MPL_F_PACKED_* and MPL_F_FUSED_U_OFF select
+ * (no counterpart in the reference).  A call that passes one of those flags is not affected by
+ * these; the values are read atomically once per call.
  * MPL_OPT_PACKED_SCANS (default 1): launches of at least 2048 chains with at most 32 labels, whose
  * planes stay below 2 GiB, are scanned with several chains per wavefront; 0 forces the
  * one-chain-per-wavefront kernels, 2 packs whenever the label count allows it (the results agree

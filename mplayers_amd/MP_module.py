@@ -53,19 +53,27 @@ def _forward_buffers(unary, args, n_dir, n_iter, with_message_tmp):
   return buf
 
 
-def _backward_buffers(dcost_final, message_index, with_message_tmp):
+def _backward_buffers(dcost_final, message_index, with_message_tmp, need_context=True,
+                      need_edge_weights=True):
   """Allocates the gradient tensors (MP_module.py:65-74, 139-150).  dedge_weights and
   dlabel_context accumulate and start at zero; dunary is written everywhere and the scratch
-  tensors are written before they are read."""
+  tensors are written before they are read.  A gradient autograd does not ask for (a fixed
+  pairwise table, no edge weights or ones that are not learned) is an empty tensor: the operators
+  then leave that part of the reverse scan out."""
   n_iter, n_dir, batch, cv, h, w, n_disp = message_index.size()
   buf = dict(
       dunary=dcost_final.new_empty(batch, cv, h, w, n_disp),
       dmessage=dcost_final.new_empty(n_dir, batch, cv, h, w, n_disp),
-      dunary_update=dcost_final.new_empty(0),
-      dedge_weights=dcost_final.new_zeros(n_dir, batch, cv, h, w))
+      dunary_update=dcost_final.new_empty(0))
+  if need_edge_weights:
+    buf["dedge_weights"] = dcost_final.new_zeros(n_dir, batch, cv, h, w)
+  else:
+    buf["dedge_weights"] = dcost_final.new_empty(0)
   if with_message_tmp:
     buf["dmessage_tmp"] = dcost_final.new_empty(n_dir, batch, cv, h, w, n_disp)
-  if n_disp == 21:
+  if not need_context:
+    buf["dlabel_context"] = dcost_final.new_empty(0)
+  elif n_disp == 21:
     buf["dlabel_context"] = dcost_final.new_zeros(n_disp, n_disp)
   else:
     buf["dlabel_context"] = dcost_final.new_zeros(n_disp)
@@ -98,12 +106,14 @@ class TRWPFunction(torch.autograd.Function):
     del ctx.intermediate_results
     dcost_final = dcost_final.contiguous()
     n_disp = message_index.size(6)
-    buf = _backward_buffers(dcost_final, message_index, with_message_tmp=False)
+    need_context = ctx.needs_input_grad[1]
+    need_edge_weights = enable_edge_weights and ctx.needs_input_grad[2]
+    buf = _backward_buffers(dcost_final, message_index, False, need_context, need_edge_weights)
     _ops_for(n_disp).TRWP.backward(rho, label_context, edge_weights, dcost_final, message_index,
                                    cost_index, buf["dunary"], buf["dlabel_context"],
                                    buf["dedge_weights"], buf["dmessage"], buf["dunary_update"])
-    dedge_weights = buf["dedge_weights"] if enable_edge_weights else None
-    return buf["dunary"], buf["dlabel_context"], dedge_weights, None
+    return (buf["dunary"], buf["dlabel_context"] if need_context else None,
+            buf["dedge_weights"] if need_edge_weights else None, None)
 
 
 class ISGMRFunction(torch.autograd.Function):
@@ -133,13 +143,15 @@ class ISGMRFunction(torch.autograd.Function):
     del ctx.intermediate_results
     dcost_final = dcost_final.contiguous()
     n_disp = message_index.size(6)
-    buf = _backward_buffers(dcost_final, message_index, with_message_tmp=True)
+    need_context = ctx.needs_input_grad[1]
+    need_edge_weights = enable_edge_weights and ctx.needs_input_grad[2]
+    buf = _backward_buffers(dcost_final, message_index, True, need_context, need_edge_weights)
     _ops_for(n_disp).ISGMR.backward(int(enable_sgm), rho, label_context, edge_weights,
                                     dcost_final, message_index, cost_index, buf["dunary"],
                                     buf["dlabel_context"], buf["dedge_weights"], buf["dmessage"],
                                     buf["dunary_update"], buf["dmessage_tmp"])
-    dedge_weights = buf["dedge_weights"] if enable_edge_weights else None
-    return buf["dunary"], buf["dlabel_context"], dedge_weights, None
+    return (buf["dunary"], buf["dlabel_context"] if need_context else None,
+            buf["dedge_weights"] if need_edge_weights else None, None)
 
 
 class MPModule(torch.nn.Module):

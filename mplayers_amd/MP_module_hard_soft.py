@@ -85,8 +85,13 @@ class TRWPFunction(torch.autograd.Function):
     dunary = dcost_final.new_empty(shape)
     scratch = dcost_final.new_empty((n_dir,) + shape)
     unused = dcost_final.new_empty(0)
-    dedge_weights = dcost_final.new_zeros((n_dir,) + shape[:-1])
-    dlabel_context = dcost_final.new_zeros((n_disp, n_disp) if args.enable_seg else (n_disp,))
+    # a gradient autograd does not ask for is an empty tensor: the operators leave it out
+    need_context = ctx.needs_input_grad[1]
+    need_edge_weights = saved["had_weights"] and ctx.needs_input_grad[2]
+    dedge_weights = (dcost_final.new_zeros((n_dir,) + shape[:-1]) if need_edge_weights
+                     else unused)
+    dlabel_context = (dcost_final.new_zeros((n_disp, n_disp) if args.enable_seg else (n_disp,))
+                      if need_context else unused)
     op = _operators(n_disp)
     if saved["soft"]:
       op.backward_soft(args.rho, dcost_final, saved["context"], saved["weights"], saved["blocks"],
@@ -94,8 +99,8 @@ class TRWPFunction(torch.autograd.Function):
     else:
       op.backward(args.rho, saved["context"], saved["weights"], dcost_final, saved["index"],
                   cost_index, dunary, dlabel_context, dedge_weights, scratch, unused)
-    return (dunary, dlabel_context, dedge_weights if saved["had_weights"] else None, None, None,
-            None)
+    return (dunary, dlabel_context if need_context else None,
+            dedge_weights if need_edge_weights else None, None)
 
 
 class MPModule(_HardModule):

@@ -18,8 +18,15 @@ KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combi
 class Shape(ctypes.Structure):
   """struct mpl_shape"""
   _fields_ = [("n_dir", ctypes.c_int), ("batch", ctypes.c_int), ("height", ctypes.c_int),
-              ("width", ctypes.c_int), ("n_disp", ctypes.c_int), ("ctx2d", ctypes.c_int),
-              ("msg_uninit", ctypes.c_int)]
+              ("width", ctypes.c_int), ("n_disp", ctypes.c_int), ("ctx2d", ctypes.c_int)]
+
+
+# per-call flags (MPL_F_* of include/mplayers_amd.h)
+F_MSG_UNINIT = 0x01
+F_PACKED_OFF = 0x02
+F_PACKED_ALWAYS = 0x04
+F_FUSED_U_OFF = 0x08
+F_DCONTEXT_SAME_LABEL = 0x10
 
 
 class KernelStat(ctypes.Structure):
@@ -40,14 +47,14 @@ def load():
         "libmplayers_hip.so is missing: build it with `python -m mplayers_amd._build` "
         "(hipcc --offload-arch=gfx950); there is no CPU or PyTorch fallback for these operators")
   lib = ctypes.CDLL(LIB_PATH)
-  vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+  vp, ci, cf, cu = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_uint
   sp = ctypes.POINTER(Shape)
-  lib.mpl_trwp_forward.argtypes = [sp, cf, ci, ci] + [vp] * 10
-  lib.mpl_trwp_backward.argtypes = [sp, cf, ci] + [vp] * 11
-  lib.mpl_isgmr_forward.argtypes = [sp, ci, cf, ci, ci] + [vp] * 11
-  lib.mpl_isgmr_backward.argtypes = [sp, ci, cf, ci] + [vp] * 12
-  lib.mpl_trwp_soft_forward.argtypes = [sp, cf, ci] + [vp] * 10
-  lib.mpl_trwp_soft_backward.argtypes = [sp, cf, ci] + [vp] * 11
+  lib.mpl_trwp_forward.argtypes = [sp, cu, cf, ci, ci] + [vp] * 10
+  lib.mpl_trwp_backward.argtypes = [sp, cu, cf, ci] + [vp] * 11
+  lib.mpl_isgmr_forward.argtypes = [sp, cu, ci, cf, ci, ci] + [vp] * 11
+  lib.mpl_isgmr_backward.argtypes = [sp, cu, ci, cf, ci] + [vp] * 12
+  lib.mpl_trwp_soft_forward.argtypes = [sp, cu, cf, ci] + [vp] * 10
+  lib.mpl_trwp_soft_backward.argtypes = [sp, cu, cf, ci] + [vp] * 11
   lib.mpl_soft_weighted_message.argtypes = [ci, ci, vp, vp, vp, vp]
   lib.mpl_soft_weighted_message_back.argtypes = [ci, ci, vp, vp, vp, vp, vp]
   lib.mpl_set_option.argtypes = [ci, ci]
@@ -64,6 +71,9 @@ def load():
   for name in SYMBOLS:
     getattr(lib, name).restype = ci
   lib.mpl_last_error.restype = ctypes.c_char_p
+  if lib.mpl_version() // 100 != 2:
+    raise RuntimeError("libmplayers_hip.so has ABI version %d, this package needs 2xx: rebuild it "
+                       "with `python -m mplayers_amd._build`" % lib.mpl_version())
   _lib = lib
   policy = os.environ.get("MPLAYERS_PACKED_SCANS")  # 0 | 1 | 2, see mpl_set_option
   if policy is not None:

@@ -11,6 +11,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -46,7 +47,10 @@ __global__ void __launch_bounds__(kWave) analyze_context_kernel(const float* __r
       lin = lin && (v == fminf(slope * (float)i, tail));
     }
     int k = (int)-wave_min(-(float)last_ne) + 1;  // c[k..L-1] == tail  (indices < 2^24: exact)
-    const bool ok = (tail == tail) && ballot(!below) == 0;
+    // a NaN tail disables both fast paths; tested on the bit pattern because the library is
+    // compiled without NaN semantics, where `tail == tail` may be folded to true
+    const bool tail_is_nan = (__builtin_bit_cast(unsigned, tail) & 0x7fffffffu) > 0x7f800000u;
+    const bool ok = !tail_is_nan && ballot(!below) == 0;
     const bool all_c0min = ballot(!c0min) == 0;
     const bool all_lin = ballot(!lin) == 0;
     if (k < 1) k = 1;  // a constant context: the centre tap alone is the band
@@ -547,12 +551,29 @@ void fill_dirs(const mpl_shape* s, int first, int count, int* dirs, int* prefix,
 
 int labels_per_lane(int L) { return (L + kWave - 1) / kWave; }
 
-bool g_packed_scans = true;  // mpl_set_option(MPL_OPT_PACKED_SCANS, ...)
-bool g_fused_u = true;       // mpl_set_option(MPL_OPT_FUSED_U, ...)
+// process defaults of the per-call choices (mpl_set_option); a call reads them once
+std::atomic<int> g_packed_scans{1};  // MPL_OPT_PACKED_SCANS: 0 off, 1 by chain count, 2 always
+std::atomic<int> g_fused_u{1};       // MPL_OPT_FUSED_U
 
-void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+// what one call does, from its flags and the process defaults
+struct CallOpts {
+  int packed;   // 0 off, 1 by chain count, 2 always
+  bool fused_u;
+};
+
+int read_flags(unsigned flags, const char* what, CallOpts* o) {
+  if (flags & ~MPL_F_ALL) return fail(MPL_EINVAL, "%s: unknown flag bits 0x%x", what, flags & ~MPL_F_ALL);
+  if ((flags & MPL_F_PACKED_OFF) && (flags & MPL_F_PACKED_ALWAYS))
+    return fail(MPL_EINVAL, "%s: MPL_F_PACKED_OFF and MPL_F_PACKED_ALWAYS exclude each other", what);
+  o->packed = (flags & MPL_F_PACKED_OFF) ? 0
+              : (flags & MPL_F_PACKED_ALWAYS) ? 2 : g_packed_scans.load(std::memory_order_relaxed);
+  o->fused_u = (flags & MPL_F_FUSED_U_OFF) ? false : g_fused_u.load(std::memory_order_relaxed) != 0;
+  return MPL_OK;
+}
+
+void launch_fwd(const SweepParams& p, bool train, bool jacobi, const CallOpts& o, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st);
-  if (g_packed_scans && launch_packed_fwd(p, train, jacobi, st)) return;
+  if (o.packed && launch_packed_fwd(p, train, jacobi, o.packed == 2, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_fwd<1>(p, train, jacobi, st); break;
     case 2: launch_sweep_fwd<2>(p, train, jacobi, st); break;
@@ -561,9 +582,9 @@ void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
   }
 }
 
-void launch_bwd(const BackParams& p, bool jacobi, hipStream_t st) {
+void launch_bwd(const BackParams& p, bool jacobi, const CallOpts& o, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st);
-  if (g_packed_scans && launch_packed_bwd(p, jacobi, st)) return;
+  if (o.packed && launch_packed_bwd(p, jacobi, o.packed == 2, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_bwd<1>(p, jacobi, st); break;
     case 2: launch_sweep_bwd<2>(p, jacobi, st); break;
@@ -632,18 +653,17 @@ extern "C" {
 
 const char* mpl_last_error(void) { return g_err; }
 
-int mpl_version(void) { return 100; }
+int mpl_version(void) { return 200; }
 
 int mpl_set_option(int option, int value) {
   if (option == MPL_OPT_PACKED_SCANS) {
     if (value < 0 || value > 2) return fail(MPL_EINVAL, "set_option: packed scans take 0, 1 or 2");
-    g_packed_scans = value != 0;
-    set_packed_policy(value == 2);
+    g_packed_scans.store(value, std::memory_order_relaxed);
     return MPL_OK;
   }
   if (option == MPL_OPT_FUSED_U) {
     if (value < 0 || value > 1) return fail(MPL_EINVAL, "set_option: fused U takes 0 or 1");
-    g_fused_u = value != 0;
+    g_fused_u.store(value, std::memory_order_relaxed);
     return MPL_OK;
   }
   return fail(MPL_EINVAL, "set_option: unknown option %d", option);
@@ -703,13 +723,16 @@ int mpl_selftest_wave_ops(int* out_host) {
   return MPL_OK;
 }
 
-int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a_dir,
-                     const float* unary, const float* context, const float* edge_weights,
-                     float* msg, float* cost_final, uint8_t* msg_min_index,
-                     uint8_t* msg_norm_index, float* unary_update, uint8_t* label_all,
-                     void* stream) {
+int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
+                     int enable_min_a_dir, const float* unary, const float* context,
+                     const float* edge_weights, float* msg, float* cost_final,
+                     uint8_t* msg_min_index, uint8_t* msg_norm_index, float* unary_update,
+                     uint8_t* label_all, void* stream) {
   int rc = check_shape(s, n_iter);
   if (rc) return rc;
+  CallOpts opts;
+  if ((rc = read_flags(flags, "trwp_forward", &opts)) != MPL_OK) return rc;
+  const bool msg_uninit = (flags & MPL_F_MSG_UNINIT) != 0;
   if (!unary || !context || !edge_weights || !msg || !cost_final || !unary_update)
     return fail(MPL_EINVAL, "trwp_forward: null tensor pointer");
   if ((msg_min_index == nullptr) != (msg_norm_index == nullptr))
@@ -724,8 +747,8 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   // (the first pair of sweeps reads `unary` in its place: Q = S - m_0 - m_1 = unary, too, and the
   // even sweep has nothing to store), no plane of initial messages is read (the descriptor's
   // flag stays 0), and the first sweep of every direction writes the zero of its chain starts.
-  const bool uninit = s->msg_uninit != 0 && desc != nullptr;
-  if (s->msg_uninit != 0 && !uninit) zero_fill(msg, (int64_t)s->n_dir * N, st);
+  const bool uninit = msg_uninit && desc != nullptr;
+  if (msg_uninit && !uninit) zero_fill(msg, (int64_t)s->n_dir * N, st);
   if (!uninit) {
     Timed timed(MPL_KERNEL_BELIEF, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
@@ -750,7 +773,7 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
         p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       }
-      launch_fwd(p, train, false, st);
+      launch_fwd(p, train, false, opts, st);
     }
     if (label_all) {
       Timed timed(MPL_KERNEL_LABEL, st);
@@ -766,13 +789,16 @@ int mpl_trwp_forward(const mpl_shape* s, float rho, int n_iter, int enable_min_a
   return launch_ok("trwp_forward");
 }
 
-int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
+int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float rho, int n_iter,
                       int enable_min_a_dir, const float* unary, const float* context,
                       const float* edge_weights, float* msg, float* cost_final,
                       uint8_t* msg_min_index, uint8_t* msg_norm_index, float* unary_update,
                       float* msg_update, uint8_t* label_all, void* stream) {
   int rc = check_shape(s, n_iter);
   if (rc) return rc;
+  CallOpts opts;
+  if ((rc = read_flags(flags, "isgmr_forward", &opts)) != MPL_OK) return rc;
+  const bool msg_uninit = (flags & MPL_F_MSG_UNINIT) != 0;
   if (!unary || !context || !edge_weights || !msg || !cost_final || !unary_update || !msg_update)
     return fail(MPL_EINVAL, "isgmr_forward: null tensor pointer");
   if ((msg_min_index == nullptr) != (msg_norm_index == nullptr))
@@ -792,14 +818,14 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   // Messages that start at zero by declaration: U_d = rho * unary in the first iteration, so at
   // rho = 1 its sweeps read `unary` itself and the pass that would store U is skipped (the
   // sweeps write every element of their output buffer, chain starts included).
-  const bool unary_as_u = s->msg_uninit != 0 && rho == 1.f;
+  const bool unary_as_u = msg_uninit && rho == 1.f;
   // Four directions at rho = 1: U of a pair of opposite directions is the unary plus the two
   // messages of the other pair, so the scans can form it on the fly (3 planes read per direction
   // instead of 1) and the pass that stores U (5 planes in, 2 out per iteration) is dropped; with
   // more directions the scans would read more than that pass moves.  (Not for the packed scans
   // of small label counts.)
-  const bool fuse_u = g_fused_u && s->n_dir == 4 && rho == 1.f && s->n_disp > 32;
-  if (s->msg_uninit != 0 && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
+  const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && s->n_disp > 32;
+  if (msg_uninit && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {
     // Jacobi over directions (ISGMR_forward.cu:506-622): every direction reads the old messages,
@@ -834,7 +860,7 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
     }
-    launch_fwd(p, train, true, st);
+    launch_fwd(p, train, true, opts, st);
     if (label_all) {
       Timed timed(MPL_KERNEL_LABEL, st);
       launch_labels(unary, nxt, s->n_dir, P, s->n_disp, factor, enable_min_a_dir, label_all + it * P, st);
@@ -850,16 +876,19 @@ int mpl_isgmr_forward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
   return launch_ok("isgmr_forward");
 }
 
-int mpl_trwp_backward(const mpl_shape* s, float rho, int n_iter, const float* context,
-                      const float* edge_weights, const float* dcost_final,
+int mpl_trwp_backward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
+                      const float* context, const float* edge_weights, const float* dcost_final,
                       const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
                       float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
                       void* stream) {
   (void)dunary_update;
   int rc = check_shape(s, n_iter);
   if (rc) return rc;
+  CallOpts opts;
+  if ((rc = read_flags(flags, "trwp_backward", &opts)) != MPL_OK) return rc;
+  // dcontext / dedge_weights may be null: gradients the caller has no use for
   if (!context || !edge_weights || !dcost_final || !msg_min_index || !msg_norm_index || !dunary ||
-      !dcontext || !dedge_weights || !dmsg)
+      !dmsg)
     return fail(MPL_EINVAL, "trwp_backward: null tensor pointer");
   hipStream_t st = (hipStream_t)stream;
   const int64_t P = (int64_t)s->batch * s->height * s->width;
@@ -879,6 +908,7 @@ int mpl_trwp_backward(const mpl_shape* s, float rho, int n_iter, const float* co
   p.ctx = context;
   p.dedge = dedge_weights;
   p.dctx = dcontext;
+  p.same_label = (flags & MPL_F_DCONTEXT_SAME_LABEL) ? 1 : 0;
   bool first = true;
   for (int it = n_iter - 1; it >= 0; --it) {
     for (int d = s->n_dir - 1; d >= 0; --d) {  // TRWP_backward.cu:337-424
@@ -891,14 +921,14 @@ int mpl_trwp_backward(const mpl_shape* s, float rho, int n_iter, const float* co
       p.skip_hi_store = (!(d & 1) && it == 0) ? 1 : 0;
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
-      launch_bwd(p, false, st);
+      launch_bwd(p, false, opts, st);
       first = false;
     }
   }
   return launch_ok("trwp_backward");
 }
 
-int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter,
+int mpl_isgmr_backward(const mpl_shape* s, unsigned flags, int enable_sgm, float rho, int n_iter,
                        const float* context, const float* edge_weights, const float* dcost_final,
                        const uint8_t* msg_min_index, const uint8_t* msg_norm_index, float* dunary,
                        float* dcontext, float* dedge_weights, float* dmsg, float* dunary_update,
@@ -906,8 +936,11 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
   (void)dunary_update;
   int rc = check_shape(s, n_iter);
   if (rc) return rc;
+  CallOpts opts;
+  if ((rc = read_flags(flags, "isgmr_backward", &opts)) != MPL_OK) return rc;
+  // dcontext / dedge_weights may be null: gradients the caller has no use for
   if (!context || !edge_weights || !dcost_final || !msg_min_index || !msg_norm_index || !dunary ||
-      !dcontext || !dedge_weights || !dmsg_update)
+      !dmsg_update)
     return fail(MPL_EINVAL, "isgmr_backward: null tensor pointer");
   // The reverse scans write X_k = dU_k into dmsg_update; the recombined gradients gu_k of the next
   // (earlier) iteration go to dmsg when the caller passes it, so that at rho == 1 one plane per
@@ -937,6 +970,7 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
   p.ctx = context;
   p.dedge = dedge_weights;
   p.dctx = dcontext;
+  p.same_label = (flags & MPL_F_DCONTEXT_SAME_LABEL) ? 1 : 0;
   fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
   for (int it = n_iter - 1; it >= 0; --it) {
     const bool first = (it == n_iter - 1);
@@ -945,7 +979,7 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
     p.gu_pair_share = first ? 0 : pair_share;
     p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
     p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
-    launch_bwd(p, true, st);
+    launch_bwd(p, true, opts, st);
     Timed timed(MPL_KERNEL_COMBINE, st);
     const bool v4 = (N % 4 == 0) && aligned16(dmsg_update) && aligned16(gu_buf) &&
                     aligned16(dcost_final) && aligned16(dunary);
@@ -956,12 +990,15 @@ int mpl_isgmr_backward(const mpl_shape* s, int enable_sgm, float rho, int n_iter
 }
 
 // ---- soft-weighted TRWP ------------------------------------------------------------------------
-int mpl_trwp_soft_forward(const mpl_shape* s, float rho, int n_iter, const float* unary,
-                          const float* context, const float* edge_weights, float* msg,
-                          float* msg_edge_label, uint8_t* msg_norm_index, float* cost_final,
-                          float* unary_update, uint8_t* label_all, void* stream) {
+int mpl_trwp_soft_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
+                          const float* unary, const float* context, const float* edge_weights,
+                          float* msg, float* msg_edge_label, uint8_t* msg_norm_index,
+                          float* cost_final, float* unary_update, uint8_t* label_all,
+                          void* stream) {
   int rc = check_shape(s, n_iter);
   if (rc) return rc;
+  CallOpts opts;
+  if ((rc = read_flags(flags, "trwp_soft_forward", &opts)) != MPL_OK) return rc;
   if (s->n_disp > kWave)
     return fail(MPL_EINVAL, "trwp_soft_forward: at most %d labels (one per lane; the stored "
                 "duals take n_disp^2 floats per pixel, direction and iteration), got %d", kWave,
@@ -974,7 +1011,7 @@ int mpl_trwp_soft_forward(const mpl_shape* s, float rho, int n_iter, const float
   const int64_t P = (int64_t)s->batch * s->height * s->width;
   const int64_t N = P * s->n_disp;
   const bool train = msg_edge_label != nullptr;
-  if (s->msg_uninit != 0) zero_fill(msg, (int64_t)s->n_dir * N, st);
+  if (flags & MPL_F_MSG_UNINIT) zero_fill(msg, (int64_t)s->n_dir * N, st);
   {
     Timed timed(MPL_KERNEL_BELIEF, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
@@ -1010,18 +1047,20 @@ int mpl_trwp_soft_forward(const mpl_shape* s, float rho, int n_iter, const float
   return launch_ok("trwp_soft_forward");
 }
 
-int mpl_trwp_soft_backward(const mpl_shape* s, float rho, int n_iter, const float* dcost_final,
-                           const float* context, const float* edge_weights,
-                           const float* msg_edge_label, const uint8_t* msg_norm_index,
-                           float* dunary, float* dcontext, float* dedge_weights, float* dmsg,
-                           float* dunary_update, void* stream) {
+int mpl_trwp_soft_backward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
+                           const float* dcost_final, const float* context,
+                           const float* edge_weights, const float* msg_edge_label,
+                           const uint8_t* msg_norm_index, float* dunary, float* dcontext,
+                           float* dedge_weights, float* dmsg, float* dunary_update, void* stream) {
   (void)dunary_update;
   int rc = check_shape(s, n_iter);
   if (rc) return rc;
+  CallOpts opts;
+  if ((rc = read_flags(flags, "trwp_soft_backward", &opts)) != MPL_OK) return rc;
   if (s->n_disp > kWave)
     return fail(MPL_EINVAL, "trwp_soft_backward: at most %d labels, got %d", kWave, s->n_disp);
   if (!context || !edge_weights || !dcost_final || !msg_edge_label || !msg_norm_index || !dunary ||
-      !dcontext || !dedge_weights || !dmsg)
+      !dmsg)
     return fail(MPL_EINVAL, "trwp_soft_backward: null tensor pointer");
   hipStream_t st = (hipStream_t)stream;
   const int64_t P = (int64_t)s->batch * s->height * s->width;

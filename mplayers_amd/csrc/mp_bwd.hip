@@ -51,8 +51,12 @@ struct PixB {
 };
 
 // SMALL: one label per lane and at most kSmallL labels (see small_l below)
-template <int R, bool VEC, bool MASK, bool JACOBI, bool SMALL>
+// GRAD: bit 0 = dedge_weights is wanted, bit 1 = dcontext is wanted (a caller with a fixed pairwise
+// table or edge weights that are not learned passes null for them; that part of the step is then
+// not compiled in: no dedge read-modify-write, no context products, no histogram gathers)
+template <int R, bool VEC, bool MASK, bool JACOBI, bool SMALL, int GRAD>
 __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
+  constexpr bool DE = (GRAD & 1) != 0, DC = (GRAD & 2) != 0;
   extern __shared__ float smem[];
   const int L = p.L;
   // 2-D context tables exist for at most 64 labels, i.e. only with one label per lane
@@ -76,6 +80,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const int dir = ch.dir;
   const int n = ch.n;
 
+  const bool same = DC && p.same_label != 0;
   for (int i = lane; i < n_ctx; i += kWave) {
     ctx_s[i] = p.ctx[i];
     hist_s[i] = 0.f;
@@ -117,7 +122,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const int img_bytes_p = (int)(HW * 4 > 0x7fffffff ? 0x7fffffff : HW * 4);
   const rsrc_t dInorm = make_rsrc(p.idx_norm + (int64_t)dir * P + img_p, (int)HW);
   const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P + img_p, img_bytes_p);
-  const rsrc_t dDe = make_rsrc(p.dedge + (int64_t)dir * P + img_p, img_bytes_p);
+  const rsrc_t dDe = make_rsrc(DE ? p.dedge + (int64_t)dir * P + img_p : nullptr, DE ? img_bytes_p : 0);
   const float rho = p.rho;
   const int lab0 = R * lane;
   const int foff = lab0 * 4;
@@ -153,7 +158,9 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
                         pp * (unsigned)L, r.fd);
     r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, (int)pp, 0, 0);
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
-    r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dDe, (int)(pp * 4u), 0, 0));
+    r.de = 0.f;
+    if (DE)
+      r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dDe, (int)(pp * 4u), 0, 0));
     ld_t -= 1;
     ld_p -= ch.pstep;
     return r;
@@ -161,8 +168,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 
   // memory instructions per step: label vectors, indices, norm index, weight, dedge in;
   // label vectors and dedge out
-  constexpr int kOps = (JACOBI ? 1 : 3) * vec_ops(R, VEC) + byte_ops(R, VEC) + 3 +
-                       (JACOBI ? 1 : 3) * vec_ops(R, VEC) + 1;
+  constexpr int kOps = (JACOBI ? 1 : 3) * vec_ops(R, VEC) + byte_ops(R, VEC) + 2 + (DE ? 1 : 0) +
+                       (JACOBI ? 1 : 3) * vec_ops(R, VEC) + (DE ? 1 : 0);
   constexpr int D = ring_depth(kOps);
   PixB<R> ring[D];
 #pragma unroll
@@ -212,15 +219,15 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           // this lane's own pair: dedge and dcontext (TRWP_backward.cu:109-112)
           const int ao = fd > cd ? fd - cd : cd - fd;
           const int ci = !valid[0] ? 0 : (ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
-          const float de = ctx_s[ci] * g;
-          if (valid[0] && cd != fd) pair_s[cd * L + fd] = fmaf(w, g, pair_s[cd * L + fd]);
+          const float de = DE ? ctx_s[ci] * g : 0.f;
+          if (DC && valid[0] && (same || cd != fd)) pair_s[cd * L + fd] = fmaf(w, g, pair_s[cd * L + fd]);
           // dU[q, f] = sum of g[c] over the labels c that point at f: one source label per trip
           // (fully unrolled for the next size bucket: lanes past L carry g = 0)
           if (L <= 8)
             scn[0] = gather_by_target<8>(g, fd, lane);
           else
             scn[0] = gather_by_target<16>(g, fd, lane);
-          det = wave_sum(de);
+          if (DE) det = wave_sum(de);
         } else {
         // the two popular targets: where the first and the last label point
         const int f0 = __builtin_amdgcn_readlane(px.fd[0], 0);
@@ -249,8 +256,10 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           off[j] = (c0 | c1) ? kPopular : d;
           any_left |= !(c0 | c1) & (ao > near_max) & valid[j];
           // dedge_weights[cur] += ctx(cd, fd) * value
-          const int ci = !valid[j] ? 0 : (ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
-          de = fmaf(ctx_s[ci], gv[j], de);
+          if (DE) {
+            const int ci = !valid[j] ? 0 : (ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
+            de = fmaf(ctx_s[ci], gv[j], de);
+          }
         }
         const float s0sum = wave_sum(p0);
         // nothing belongs to the second class when both popular targets coincide (the usual case)
@@ -288,12 +297,21 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           const float own = (off[j] == 0) ? gv[j] : 0.f;
           scn[j] = own + tp[j] + tn[j] + (cd == f0 ? s0sum : 0.f) + (cd == f1 ? s1sum : 0.f);
         }
-        // dcontext += edge_weight * value where cd != fd (TRWP_backward.cu:111-112)
-        if (!ctx2d) {
+        // dcontext += edge_weight * value where cd != fd (TRWP_backward.cu:111-112); with `same`
+        // also where cd == fd (TRWP_hard_soft/TRWP_backward.cu:110)
+        if (!DC) {
+        } else if (!ctx2d) {
+          // bin 0, labels outside the popular classes that point at themselves
+          if (same) {  // wave-uniform
+            float own_sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < R; ++j) own_sum += (off[j] == 0) ? gv[j] : 0.f;
+            near_acc[0] = fmaf(w, own_sum, near_acc[0]);
+          }
 #pragma unroll
           for (int o = 1; o <= kNear; ++o) near_acc[o] = fmaf(w, near_t[o], near_acc[o]);
           // popular classes: bin |cd - f| is reached from labels f + k and f - k; gather through LDS
-          // (bin 0 collects the popular label's own value twice; it is never flushed)
+          // (bin 0 collects the popular label's own value twice: halved when it is flushed)
 #pragma unroll
           for (int j = 0; j < R; ++j)
             if (valid[j]) g0_s[L + lab0 + j] = (px.fd[j] == f0) ? w * gv[j] : 0.f;
@@ -318,7 +336,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
           for (int j = 0; j < R; ++j) {
             const int cd = lab0 + j, fd = px.fd[j];
-            if (valid[j] && cd != fd)
+            if (valid[j] && (same || cd != fd))
               atomicAdd(&hist_s[cd < fd ? cd * L + fd : fd * L + cd], w * gv[j]);
           }
         }
@@ -329,7 +347,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
             const int ao = off[j] < 0 ? -off[j] : off[j];
             if (valid[j] && off[j] != kPopular && ao > near_max) {
               atomicAdd(&sc_s[px.fd[j]], gv[j]);
-              if (!ctx2d) atomicAdd(&hist_s[ao], w * gv[j]);
+              if (DC && !ctx2d) atomicAdd(&hist_s[ao], w * gv[j]);
             }
           }
           __syncthreads();
@@ -337,7 +355,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           for (int j = 0; j < R; ++j)
             if (valid[j]) scn[j] += atomicExch(&sc_s[lab0 + j], 0.f);  // read and clear
         }
-        det = wave_sum(de);
+        if (DE) det = wave_sum(de);
         }
       }
       // pixel-local part of UpdateUnaryKernelBack with dU[pix] = sc; nothing is stored for t < 0
@@ -362,30 +380,33 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
         buf_store<R, VEC>(make_rsrc(bHi, p.skip_hi_store ? 0 : nrec), foff, so, hin);
       }
       // each pixel receives over exactly one edge per direction: plain read-modify-write
-      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
-                                            t >= 1 ? (int)(sp * 4u) : kDeadOffset, 0, 0);
+      if (DE)
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
+                                              t >= 1 ? (int)(sp * 4u) : kDeadOffset, 0, 0);
 #pragma unroll
       for (int j = 0; j < R; ++j) sc[j] = scn[j];
       st_p -= ch.pstep;
     }
   }
+  if (!DC) return;
   __syncthreads();
   if (small_l) {
-    // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D)
+    // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D); the pairs
+    // with cd == fd (bin 0 / the diagonal) were only collected when the caller asked for them
     if (!ctx2d) {
-      if (lane >= 1 && lane < L) {
+      if (lane < L) {
         float acc = 0.f;
         for (int c = 0; c < L; ++c) {
           if (c + lane < L) acc += pair_s[c * L + c + lane];
-          if (c - lane >= 0) acc += pair_s[c * L + c - lane];
+          if (lane >= 1 && c - lane >= 0) acc += pair_s[c * L + c - lane];
         }
         if (acc != 0.f) atomicAdd(&p.dctx[lane], acc);
       }
     } else {
       for (int i = lane; i < L * L; i += kWave) {
         const int c = i / L, f = i - c * L;
-        if (c >= f) continue;  // the (f, c) entry is added here; the diagonal never accumulates
-        const float v = pair_s[i] + pair_s[f * L + c];
+        if (c > f) continue;  // the (f, c) entry is added here
+        const float v = pair_s[i] + (c < f ? pair_s[f * L + c] : 0.f);
         if (v != 0.f) atomicAdd(&p.dctx[i], v);
       }
     }
@@ -403,27 +424,43 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
       const float v = wave_sum(near_acc[k]);
       if (lane == 0 && k < L && v != 0.f) atomicAdd(&p.dctx[k], v);
     }
+    if (same) {
+      // bin 0: the popular labels that point at themselves were gathered twice into the
+      // accumulator of label 0 (x + x, exact), the others were summed per lane
+      const float v = wave_sum(near_acc[0] + (lane == 0 ? 0.5f * hist_reg[0] : 0.f));
+      if (lane == 0 && v != 0.f) atomicAdd(&p.dctx[0], v);
+    }
   }
 }
 
-template <int R, bool VEC, bool MASK>
-void launch_vm(const BackParams& p, bool jacobi, hipStream_t st) {
+template <int R, bool VEC, bool MASK, int GRAD>
+void launch_vmg(const BackParams& p, bool jacobi, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = sizeof(float) * (kMaxL + 6 * p.L + 2 * (p.ctx2d ? p.L * p.L : p.L) +
                                       ((R == 1 && p.L <= kSmallL) ? p.L * p.L : 0));
   if constexpr (R == 1) {
     if (p.L <= kSmallL) {
       if (jacobi)
-        sweep_bwd_kernel<R, VEC, MASK, true, true><<<blocks, kWave, lds, st>>>(p);
+        sweep_bwd_kernel<R, VEC, MASK, true, true, GRAD><<<blocks, kWave, lds, st>>>(p);
       else
-        sweep_bwd_kernel<R, VEC, MASK, false, true><<<blocks, kWave, lds, st>>>(p);
+        sweep_bwd_kernel<R, VEC, MASK, false, true, GRAD><<<blocks, kWave, lds, st>>>(p);
       return;
     }
   }
   if (jacobi)
-    sweep_bwd_kernel<R, VEC, MASK, true, false><<<blocks, kWave, lds, st>>>(p);
+    sweep_bwd_kernel<R, VEC, MASK, true, false, GRAD><<<blocks, kWave, lds, st>>>(p);
   else
-    sweep_bwd_kernel<R, VEC, MASK, false, false><<<blocks, kWave, lds, st>>>(p);
+    sweep_bwd_kernel<R, VEC, MASK, false, false, GRAD><<<blocks, kWave, lds, st>>>(p);
+}
+
+template <int R, bool VEC, bool MASK>
+void launch_vm(const BackParams& p, bool jacobi, hipStream_t st) {
+  switch ((p.dedge != nullptr ? 1 : 0) | (p.dctx != nullptr ? 2 : 0)) {
+    case 0: launch_vmg<R, VEC, MASK, 0>(p, jacobi, st); break;
+    case 1: launch_vmg<R, VEC, MASK, 1>(p, jacobi, st); break;
+    case 2: launch_vmg<R, VEC, MASK, 2>(p, jacobi, st); break;
+    default: launch_vmg<R, VEC, MASK, 3>(p, jacobi, st); break;
+  }
 }
 
 }  // namespace

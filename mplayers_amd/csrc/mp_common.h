@@ -470,8 +470,10 @@ struct BackParams {
   const float* ctx;
   const uint8_t* idx_min;   // (n_dir_total, N) of this iteration
   const uint8_t* idx_norm;  // (n_dir_total, P)
-  float* dedge;             // (n_dir_total, P) accumulates
-  float* dctx;              // accumulates
+  float* dedge;             // (n_dir_total, P) accumulates; null: not wanted, that part of the step is left out
+  float* dctx;              // accumulates; null: not wanted
+  int same_label;           // dctx also collects the pairs with cd == fd (the hard operator of the
+                            // reference's TRWP_hard_soft build, TRWP_hard_soft/TRWP_backward.cu:104-111)
   const float* edge_label;  // soft TRWP: (n_dir_total, P, L, L) duals of this iteration
   int pack;                 // packed scans (mp_pack.hip): chains per wavefront
 };
@@ -490,9 +492,9 @@ void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 // The launchers return false, without launching, when the problem does not qualify.
 constexpr int kPackedMaxL = 32;
 constexpr int kPackedMinChains = 2048;  // two wavefronts per SIMD of the 256 CUs when unpacked
-void set_packed_policy(bool always);  // tests: pack whatever the number of chains
-bool launch_packed_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st);
-bool launch_packed_bwd(const BackParams& p, bool jacobi, hipStream_t st);
+// always: pack whatever the number of chains (tests and comparisons)
+bool launch_packed_fwd(const SweepParams& p, bool train, bool jacobi, bool always, hipStream_t st);
+bool launch_packed_bwd(const BackParams& p, bool jacobi, bool always, hipStream_t st);
 
 // soft-weighted TRWP (mp_soft.hip): one direction per launch, L <= 64
 void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st);

@@ -274,8 +274,10 @@ struct PixPB {
   float w, de;
 };
 
-template <bool JACOBI, int LT>
+// GRAD: bit 0 = dedge_weights is wanted, bit 1 = dcontext is wanted
+template <bool JACOBI, int LT, int GRAD>
 __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
+  constexpr bool DE = (GRAD & 1) != 0, DC = (GRAD & 2) != 0;
   extern __shared__ float smem[];
   const int L = LT > 0 ? LT : p.L;
   const int G = p.pack;
@@ -284,14 +286,16 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
   const int lane = threadIdx.x;
   const PackedChains ch = locate_packed(p, lane, L, G);
   const Seg sg = make_seg(lane, L, G);
-  fill_table(p.ctx, L, p.ctx2d, lane, tab);
-  for (int i = lane; i < G * L * L; i += kWave) pairs[i] = 0.f;
+  if (DE) fill_table(p.ctx, L, p.ctx2d, lane, tab);
+  if (DC)
+    for (int i = lane; i < G * L * L; i += kWave) pairs[i] = 0.f;
   __syncthreads();
 
   const int64_t P = (int64_t)p.B * p.H * p.W;
   const int64_t N = P * L;
   const int dir = ch.dir;
   const int plane_bytes = (int)(N * 4);
+  const bool same = p.same_label != 0;
   const bool read_h = !JACOBI && !p.first_touch;
   const bool inv_from_a = !JACOBI && p.inv_from_a;
   const int gdir = p.gu_pair_share ? (dir & ~1) : dir;
@@ -305,7 +309,7 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
   const rsrc_t dImin = make_rsrc(p.idx_min + (int64_t)dir * N, (int)N);
   const rsrc_t dInorm = make_rsrc(p.idx_norm + (int64_t)dir * P, (int)P);
   const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P, (int)(P * 4));
-  const rsrc_t dDe = make_rsrc(p.dedge + (int64_t)dir * P, (int)(P * 4));
+  const rsrc_t dDe = make_rsrc(DE ? p.dedge + (int64_t)dir * P : nullptr, DE ? (int)(P * 4) : 0);
   const float rho = p.rho;
   const int l = sg.l;
   const bool on = ch.on;
@@ -330,14 +334,16 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
     r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, act ? ld_pix : kDeadOffset, 0, 0);
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
                                         dW, act ? ld_pix * 4 : kDeadOffset, 0, 0));
-    r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                         dDe, (act && l == 0) ? ld_pix * 4 : kDeadOffset, 0, 0));
+    r.de = 0.f;
+    if (DE)
+      r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                           dDe, (act && l == 0) ? ld_pix * 4 : kDeadOffset, 0, 0));
     ld_pix -= ch.pstep;
     ld_t -= 1;
     return r;
   };
 
-  constexpr int kOps = (JACOBI ? 1 : 3) + 4 + (JACOBI ? 1 : 3) + 1;
+  constexpr int kOps = (JACOBI ? 1 : 3) + 3 + (DE ? 1 : 0) + (JACOBI ? 1 : 3) + (DE ? 1 : 0);
   constexpr int D = ring_depth(kOps);
   PixPB ring[D];
 #pragma unroll
@@ -379,8 +385,9 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
       // dedge_weights[p] += ctx(cd, fd) * g;  dcontext[(cd, fd)] += w * g for cd != fd
       // (TRWP_backward.cu:109-112)
       const int fdc = edge ? fd : 0;
-      const float det = seg_sum(sg, tab[fdc * L + l] * g);
-      if (edge && fdc != l) my_pairs[fdc] = fmaf(px.w, g, my_pairs[fdc]);
+      float det = 0.f;
+      if (DE) det = seg_sum(sg, tab[fdc * L + l] * g);
+      if (DC && edge && (same || fdc != l)) my_pairs[fdc] = fmaf(px.w, g, my_pairs[fdc]);
       const unsigned eo = here ? (unsigned)(st_pix * L + l) * 4u : (unsigned)kDeadOffset;
       if (JACOBI) {
         stf(dAo, eo, sc);
@@ -390,30 +397,34 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
         stf(dHdOut, eo, -an);          // g_dir = 0 after its sweep
         stf(dHiOut, eo, px.hi - sc);   // g_inv -= dU
       }
-      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
-                                            (edge && l == 0) ? st_pix * 4 : kDeadOffset, 0, 0);
+      if (DE)
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
+                                              (edge && l == 0) ? st_pix * 4 : kDeadOffset, 0, 0);
       sc = here ? scn : 0.f;
       st_pix -= ch.pstep;
     }
   }
+  if (!DC) return;
   __syncthreads();
-  // fold the pair tables of all chain slots into dcontext's bins
+  // fold the pair tables of all chain slots into dcontext's bins (the pairs with cd == fd were
+  // only collected when the caller asked for them)
   if (!p.ctx2d) {
-    if (lane >= 1 && lane < L) {
+    if (lane < L) {
       float acc = 0.f;
       for (int g2 = 0; g2 < G; ++g2)
         for (int c = 0; c < L; ++c) {
           if (c + lane < L) acc += pairs[g2 * L * L + c * L + c + lane];
-          if (c - lane >= 0) acc += pairs[g2 * L * L + c * L + c - lane];
+          if (lane >= 1 && c - lane >= 0) acc += pairs[g2 * L * L + c * L + c - lane];
         }
       if (acc != 0.f) atomicAdd(&p.dctx[lane], acc);
     }
   } else {
     for (int i = lane; i < L * L; i += kWave) {
       const int c = i / L, f = i - c * L;
-      if (c >= f) continue;
+      if (c > f) continue;
       float v = 0.f;
-      for (int g2 = 0; g2 < G; ++g2) v += pairs[g2 * L * L + i] + pairs[g2 * L * L + f * L + c];
+      for (int g2 = 0; g2 < G; ++g2)
+        v += pairs[g2 * L * L + i] + (c < f ? pairs[g2 * L * L + f * L + c] : 0.f);
       if (v != 0.f) atomicAdd(&p.dctx[i], v);
     }
   }
@@ -441,25 +452,21 @@ Params with_wave_prefix(const Params& p, int G) {
 
 }  // namespace
 
-bool g_pack_always = false;  // set_packed_policy
-
-int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains) {
+int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool always) {
   if (L > kPackedMaxL) return 0;
   if ((int64_t)B * H * W * L * 4 >= (int64_t)kDeadOffset) return 0;  // 32-bit plane offsets
   // A packed step issues fewer instructions per chain but has the longer dependent chain (its
   // reductions go through ds_bpermute): it pays once every SIMD of the 256 CUs would otherwise
   // hold two or more wavefronts (measured: 516 chains of 129 pixels and 21 labels per launch are
   // 25 % faster unpacked, 2064 chains 15-40 % faster packed).
-  if (chains < (g_pack_always ? 1 : kPackedMinChains)) return 0;
+  if (chains < (always ? 1 : kPackedMinChains)) return 0;
   int G = kWave / L;
   return G > 16 ? 16 : G;
 }
 
-void set_packed_policy(bool always) { g_pack_always = always; }
-
-bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, hipStream_t st) {
+bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, bool always, hipStream_t st) {
   if (p0.u_fused) return false;  // (set for more than 32 labels only)
-  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0));
+  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0), always);
   if (G < 2) return false;
   const SweepParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
@@ -486,23 +493,33 @@ bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, hipStream
   return true;
 }
 
-bool launch_packed_bwd(const BackParams& p0, bool jacobi, hipStream_t st) {
-  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0));
+bool launch_packed_bwd(const BackParams& p0, bool jacobi, bool always, hipStream_t st) {
+  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0), always);
   if (G < 2) return false;
   const BackParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = sizeof(float) * p.L * p.L * (1 + G);
-  if (p.L == 21) {
-    if (jacobi)
-      packed_bwd_kernel<true, 21><<<blocks, kWave, lds, st>>>(p);
-    else
-      packed_bwd_kernel<false, 21><<<blocks, kWave, lds, st>>>(p);
-  } else {
-    if (jacobi)
-      packed_bwd_kernel<true, 0><<<blocks, kWave, lds, st>>>(p);
-    else
-      packed_bwd_kernel<false, 0><<<blocks, kWave, lds, st>>>(p);
+#define MPL_PACKED_BWD(GRAD)                                                  \
+  do {                                                                        \
+    if (p.L == 21) {                                                          \
+      if (jacobi)                                                             \
+        packed_bwd_kernel<true, 21, GRAD><<<blocks, kWave, lds, st>>>(p);     \
+      else                                                                    \
+        packed_bwd_kernel<false, 21, GRAD><<<blocks, kWave, lds, st>>>(p);    \
+    } else {                                                                  \
+      if (jacobi)                                                             \
+        packed_bwd_kernel<true, 0, GRAD><<<blocks, kWave, lds, st>>>(p);      \
+      else                                                                    \
+        packed_bwd_kernel<false, 0, GRAD><<<blocks, kWave, lds, st>>>(p);     \
+    }                                                                         \
+  } while (0)
+  switch ((p.dedge != nullptr ? 1 : 0) | (p.dctx != nullptr ? 2 : 0)) {
+    case 0: MPL_PACKED_BWD(0); break;
+    case 1: MPL_PACKED_BWD(1); break;
+    case 2: MPL_PACKED_BWD(2); break;
+    default: MPL_PACKED_BWD(3); break;
   }
+#undef MPL_PACKED_BWD
   return true;
 }
 

@@ -238,7 +238,9 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
   const int img_bytes_p = (int)(HW * 4 > 0x7fffffff ? 0x7fffffff : HW * 4);
   const rsrc_t dInorm = make_rsrc(p.idx_norm + (int64_t)dir * P + img_p, (int)HW);
   const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P + img_p, img_bytes_p);
-  const rsrc_t dDe = make_rsrc(p.dedge + (int64_t)dir * P + img_p, img_bytes_p);
+  // a gradient the caller does not want (null): its reads return 0 and its stores are dropped
+  const rsrc_t dDe = make_rsrc(p.dedge != nullptr ? p.dedge + (int64_t)dir * P + img_p : nullptr,
+                               p.dedge != nullptr ? img_bytes_p : 0);
   const float rho = p.rho;
   const int foff = lane * 4;
   const bool valid = lane < L;
@@ -381,6 +383,7 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
       st_p -= ch.pstep;
     }
   }
+  if (p.dctx == nullptr) return;
   if (LT > 0 && valid) {
 #pragma unroll
     for (int fd = 0; fd < LT; ++fd) hist[fd * L + lane] = hreg[fd];

@@ -37,6 +37,12 @@ def _context_numel(L, ctx2d):
   return L * L if ctx2d else L
 
 
+def _wanted(t):
+  """An output gradient the caller has no use for is passed as None or as an empty tensor, the
+  reference's way of switching an output off (TRWP_forward.cu:406-408)."""
+  return t is not None and t.numel() > 0
+
+
 class _Op(object):
   """Shared plumbing of the two operator namespaces."""
 
@@ -86,15 +92,16 @@ class TRWP(object):
 
   @staticmethod
   def forward(rho, n_iter, enable_min_a_dir, unary, context, edge_weights, msg, cost_final,
-              msg_min_index, msg_norm_index, unary_update, label_all, msg_uninit=False):
+              msg_min_index, msg_norm_index, unary_update, label_all, msg_uninit=False, flags=0):
     """msg_uninit (not in the reference): True declares that `msg` holds no initial messages --
-    they start at zero and the library writes every element, so the caller need not clear it."""
+    they start at zero and the library writes every element, so the caller need not clear it.
+    flags (not in the reference): further per-call MPL_F_* bits of the C ABI."""
     lib = _lib.load()
     shape, _, _ = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
                                      msg_norm_index, unary_update, label_all, n_iter)
-    shape.msg_uninit = int(bool(msg_uninit))
+    flags = int(flags) | (_lib.F_MSG_UNINIT if msg_uninit else 0)
     with torch.cuda.device(unary.device):
-      rc = lib.mpl_trwp_forward(shape, float(rho), int(n_iter), int(enable_min_a_dir),
+      rc = lib.mpl_trwp_forward(shape, flags, float(rho), int(n_iter), int(enable_min_a_dir),
                                 _ptr(unary), _ptr(context), _ptr(edge_weights), _ptr(msg),
                                 _ptr(cost_final), _ptr(msg_min_index), _ptr(msg_norm_index),
                                 _ptr(unary_update), _ptr(label_all), _Op._stream(unary))
@@ -102,7 +109,9 @@ class TRWP(object):
 
   @staticmethod
   def backward(rho, context, edge_weights, dcost_final, msg_min_index, msg_norm_index, dunary,
-               dcontext, dedge_weights, dmsg, dunary_update):
+               dcontext, dedge_weights, dmsg, dunary_update, flags=0):
+    """dcontext / dedge_weights: None or an empty tensor when that gradient is not wanted (not in
+    the reference, which always computes both); flags: per-call MPL_F_* bits of the C ABI."""
     lib = _lib.load()
     shape, n_iter, P, L, ctx2d = _Op._shape_from_index(msg_min_index)
     N = P * L
@@ -113,11 +122,13 @@ class TRWP(object):
     _check("msg_min_index", msg_min_index, u8, n_iter * shape.n_dir * N)
     _check("msg_norm_index", msg_norm_index, u8, n_iter * shape.n_dir * P)
     _check("dunary", dunary, f32, N)
-    _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
-    _check("dedge_weights", dedge_weights, f32, shape.n_dir * P)
+    if _wanted(dcontext):
+      _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
+    if _wanted(dedge_weights):
+      _check("dedge_weights", dedge_weights, f32, shape.n_dir * P)
     _check("dmsg", dmsg, f32, shape.n_dir * N)
     with torch.cuda.device(dcost_final.device):
-      rc = lib.mpl_trwp_backward(shape, float(rho), int(n_iter), _ptr(context),
+      rc = lib.mpl_trwp_backward(shape, int(flags), float(rho), int(n_iter), _ptr(context),
                                  _ptr(edge_weights), _ptr(dcost_final), _ptr(msg_min_index),
                                  _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
                                  _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),
@@ -131,15 +142,15 @@ class ISGMR(object):
   @staticmethod
   def forward(enable_sgm, rho, n_iter, enable_min_a_dir, unary, context, edge_weights, msg,
               cost_final, msg_min_index, msg_norm_index, unary_update, msg_update, label_all,
-              msg_uninit=False):
-    """msg_uninit (not in the reference): see TRWP.forward."""
+              msg_uninit=False, flags=0):
+    """msg_uninit, flags (not in the reference): see TRWP.forward."""
     lib = _lib.load()
     shape, _, N = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
                                      msg_norm_index, unary_update, label_all, n_iter)
-    shape.msg_uninit = int(bool(msg_uninit))
+    flags = int(flags) | (_lib.F_MSG_UNINIT if msg_uninit else 0)
     _check("msg_update", msg_update, torch.float32, shape.n_dir * N)
     with torch.cuda.device(unary.device):
-      rc = lib.mpl_isgmr_forward(shape, int(enable_sgm), float(rho), int(n_iter),
+      rc = lib.mpl_isgmr_forward(shape, flags, int(enable_sgm), float(rho), int(n_iter),
                                  int(enable_min_a_dir), _ptr(unary), _ptr(context),
                                  _ptr(edge_weights), _ptr(msg), _ptr(cost_final),
                                  _ptr(msg_min_index), _ptr(msg_norm_index), _ptr(unary_update),
@@ -148,7 +159,9 @@ class ISGMR(object):
 
   @staticmethod
   def backward(enable_sgm, rho, context, edge_weights, dcost_final, msg_min_index,
-               msg_norm_index, dunary, dcontext, dedge_weights, dmsg, dunary_update, dmsg_update):
+               msg_norm_index, dunary, dcontext, dedge_weights, dmsg, dunary_update, dmsg_update,
+               flags=0):
+    """dcontext / dedge_weights / flags: see TRWP.backward."""
     lib = _lib.load()
     shape, n_iter, P, L, ctx2d = _Op._shape_from_index(msg_min_index)
     N = P * L
@@ -159,15 +172,18 @@ class ISGMR(object):
     _check("msg_min_index", msg_min_index, u8, n_iter * shape.n_dir * N)
     _check("msg_norm_index", msg_norm_index, u8, n_iter * shape.n_dir * P)
     _check("dunary", dunary, f32, N)
-    _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
-    _check("dedge_weights", dedge_weights, f32, shape.n_dir * P)
+    if _wanted(dcontext):
+      _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
+    if _wanted(dedge_weights):
+      _check("dedge_weights", dedge_weights, f32, shape.n_dir * P)
     _check("dmsg_update", dmsg_update, f32, shape.n_dir * N)
     # dmsg is optional scratch: used when it has the reference's full size, ignored otherwise
     if not (isinstance(dmsg, torch.Tensor) and dmsg.is_cuda and dmsg.is_contiguous() and
             dmsg.dtype == f32 and dmsg.numel() >= shape.n_dir * N):
       dmsg = None
     with torch.cuda.device(dcost_final.device):
-      rc = lib.mpl_isgmr_backward(shape, int(enable_sgm), float(rho), int(n_iter), _ptr(context),
+      rc = lib.mpl_isgmr_backward(shape, int(flags), int(enable_sgm), float(rho), int(n_iter),
+                                  _ptr(context),
                                   _ptr(edge_weights), _ptr(dcost_final), _ptr(msg_min_index),
                                   _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
                                   _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),
@@ -182,7 +198,17 @@ class TRWP_hard_soft(object):
   `soft_weighted_message` / `soft_weighted_message_back`."""
 
   forward = TRWP.forward
-  backward = TRWP.backward
+
+  @staticmethod
+  def backward(rho, context, edge_weights, dcost_final, msg_min_index, msg_norm_index, dunary,
+               dcontext, dedge_weights, dmsg, dunary_update, flags=0):
+    """The hard backward of this build differs from TRWP.backward in one point: dcontext also
+    collects the pairs whose front label equals their own (entry 0 of a 1-D table, the diagonal of
+    a 2-D one): TRWP_hard_soft/TRWP_backward.cu:110,194,264 have no `current_d != front_d` guard
+    (TRWP/TRWP_backward.cu:111-112 has)."""
+    TRWP.backward(rho, context, edge_weights, dcost_final, msg_min_index, msg_norm_index, dunary,
+                  dcontext, dedge_weights, dmsg, dunary_update,
+                  flags=int(flags) | _lib.F_DCONTEXT_SAME_LABEL)
 
   @staticmethod
   def forward_soft(rho, n_iter, unary, context, edge_weights, msg, msg_edge_label, msg_norm_index,
@@ -203,7 +229,7 @@ class TRWP_hard_soft(object):
     if label_all.numel() > 0:
       _check("label_all", label_all, u8, n_iter * P)
     with torch.cuda.device(unary.device):
-      rc = lib.mpl_trwp_soft_forward(shape, float(rho), int(n_iter), _ptr(unary), _ptr(context),
+      rc = lib.mpl_trwp_soft_forward(shape, 0, float(rho), int(n_iter), _ptr(unary), _ptr(context),
                                      _ptr(edge_weights), _ptr(msg), _ptr(msg_edge_label),
                                      _ptr(msg_norm_index), _ptr(cost_final), _ptr(unary_update),
                                      _ptr(label_all), _Op._stream(unary))
@@ -228,11 +254,13 @@ class TRWP_hard_soft(object):
     _check("msg_edge_label", msg_edge_label, f32, n_iter * n_dir * N * L)
     _check("msg_norm_index", msg_norm_index, u8, n_iter * n_dir * P)
     _check("dunary", dunary, f32, N)
-    _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
-    _check("dedge_weights", dedge_weights, f32, n_dir * P)
+    if _wanted(dcontext):
+      _check("dcontext", dcontext, f32, _context_numel(L, ctx2d))
+    if _wanted(dedge_weights):
+      _check("dedge_weights", dedge_weights, f32, n_dir * P)
     _check("dmsg", dmsg, f32, n_dir * N)
     with torch.cuda.device(dcost_final.device):
-      rc = lib.mpl_trwp_soft_backward(shape, float(rho), int(n_iter), _ptr(dcost_final),
+      rc = lib.mpl_trwp_soft_backward(shape, 0, float(rho), int(n_iter), _ptr(dcost_final),
                                       _ptr(context), _ptr(edge_weights), _ptr(msg_edge_label),
                                       _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
                                       _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),

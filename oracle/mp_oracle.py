@@ -74,7 +74,8 @@ def forward(mode, unary, context, edge_weights, n_dir, n_iter, rho, training=Tru
   """Restated ForwardCUDA of TRWP (TRWP_forward.cu:378-560) or ISGMR (ISGMR_forward.cu:433-665).
 
   Returns a dict with msg, cost_final, msg_min_index, msg_norm_index, label_all and, when
-  want_gaps, gap_min / gap_norm (second best minus best of every argmin, for tie-aware checks).
+  want_gaps, gap_min / gap_norm / gap_label (second best minus best of every argmin and of every
+  saved label, for tie-aware checks).
   """
   unary = np.ascontiguousarray(unary)
   sfx, creal = _real(unary.dtype)
@@ -94,30 +95,34 @@ def forward(mode, unary, context, edge_weights, n_dir, n_iter, rho, training=Tru
   label = np.zeros((n_iter, b, cv, h, w), dtype=np.uint8) if saving_label else None
   gmin = np.full((n_iter, n_dir, b, cv, h, w, L), np.inf, dtype=dt) if want_gaps else None
   gnorm = np.full((n_iter, n_dir, b, cv, h, w), np.inf, dtype=dt) if want_gaps else None
+  glabel = np.full((n_iter, b, cv, h, w), np.inf, dtype=dt) if (want_gaps and saving_label) \
+      else None
   out = dict(msg=msg, cost_final=cost, msg_min_index=imin, msg_norm_index=inorm, label_all=label,
-             gap_min=gmin, gap_norm=gnorm)
+             gap_min=gmin, gap_norm=gnorm, gap_label=glabel)
   if mode == "TRWP":
     fn = getattr(lib(), "mpo_trwp_forward_" + sfx)
     fn(ctypes.byref(g), creal(rho), int(n_iter), int(enable_min_a_dir), _ptr(unary),
        _ptr(context), _ptr(edge_weights), _ptr(msg), _ptr(cost), _ptr(imin), _ptr(inorm),
-       _ptr(label), _ptr(gmin), _ptr(gnorm))
+       _ptr(label), _ptr(gmin), _ptr(gnorm), _ptr(glabel))
   elif mode in ("ISGMR", "SGM"):
     fn = getattr(lib(), "mpo_isgmr_forward_" + sfx)
     msg_update = np.zeros_like(msg)
     fn(ctypes.byref(g), int(enable_sgm), creal(rho), int(n_iter), int(enable_min_a_dir),
        _ptr(unary), _ptr(context), _ptr(edge_weights), _ptr(msg), _ptr(msg_update), _ptr(cost),
-       _ptr(imin), _ptr(inorm), _ptr(label), _ptr(gmin), _ptr(gnorm))
+       _ptr(imin), _ptr(inorm), _ptr(label), _ptr(gmin), _ptr(gnorm), _ptr(glabel))
   else:
     raise ValueError(mode)
   return out
 
 
 def backward(mode, context, edge_weights, dcost_final, msg_min_index, msg_norm_index, rho,
-             enable_sgm=False, ctx2d=None):
+             enable_sgm=False, ctx2d=None, same_label=False):
   """Restated BackwardCUDA (TRWP_backward.cu:277-433, ISGMR_backward.cu:290-493).
 
   Returns (dunary, dcontext, dedge_weights); dcontext is (L, L) when ctx2d else (L,), as
   allocated by the reference's Function.backward (MP_module.py:65-74).
+  same_label (TRWP only): the hard backward of the TRWP_hard_soft build, whose dcontext also
+  collects the pairs with current_d == front_d (TRWP_hard_soft/TRWP_backward.cu:110,194,264).
   """
   dcost_final = np.ascontiguousarray(dcost_final)
   sfx, creal = _real(dcost_final.dtype)
@@ -137,8 +142,9 @@ def backward(mode, context, edge_weights, dcost_final, msg_min_index, msg_norm_i
     fn = getattr(lib(), "mpo_trwp_backward_" + sfx)
     fn(ctypes.byref(g), creal(rho), int(n_iter), _ptr(context), _ptr(edge_weights),
        _ptr(dcost_final), _ptr(msg_min_index), _ptr(msg_norm_index), _ptr(dunary),
-       _ptr(dcontext), _ptr(dedge))
+       _ptr(dcontext), _ptr(dedge), int(bool(same_label)))
   elif mode in ("ISGMR", "SGM"):
+    assert not same_label
     fn = getattr(lib(), "mpo_isgmr_backward_" + sfx)
     fn(ctypes.byref(g), int(enable_sgm), creal(rho), int(n_iter), _ptr(context),
        _ptr(edge_weights), _ptr(dcost_final), _ptr(msg_min_index), _ptr(msg_norm_index),
@@ -177,7 +183,7 @@ def refcpu_forward(mode, unary, context, n_dir, n_iter, rho, n_threads=16, ctx2d
 
 
 def forward_soft(unary, context, edge_weights, n_dir, n_iter, rho, training=True,
-                 saving_label=False, ctx2d=None):
+                 saving_label=False, ctx2d=None, want_gaps=False):
   """Restated ForwardCUDASoft (TRWP_hard_soft/TRWP_forward_soft.cu:378-559).
 
   Returns a dict with msg, cost_final, msg_edge_label (n_iter, n_dir, B, cv, H, W, L, L),
@@ -196,10 +202,13 @@ def forward_soft(unary, context, edge_weights, n_dir, n_iter, rho, training=True
   mel = np.zeros((n_iter, n_dir, b, cv, h, w, L, L), dtype=dt) if training else None
   inorm = np.zeros((n_iter, n_dir, b, cv, h, w), dtype=np.uint8) if training else None
   label = np.zeros((n_iter, b, cv, h, w), dtype=np.uint8) if saving_label else None
+  glabel = np.full((n_iter, b, cv, h, w), np.inf, dtype=dt) if (want_gaps and saving_label) \
+      else None
   fn = getattr(lib(), "mpo_trwp_soft_forward_" + sfx)
   fn(ctypes.byref(g), creal(rho), int(n_iter), _ptr(unary), _ptr(context), _ptr(edge_weights),
-     _ptr(msg), _ptr(cost), _ptr(mel), _ptr(inorm), _ptr(label))
-  return dict(msg=msg, cost_final=cost, msg_edge_label=mel, msg_norm_index=inorm, label_all=label)
+     _ptr(msg), _ptr(cost), _ptr(mel), _ptr(inorm), _ptr(label), _ptr(glabel))
+  return dict(msg=msg, cost_final=cost, msg_edge_label=mel, msg_norm_index=inorm, label_all=label,
+              gap_label=glabel)
 
 
 def backward_soft(context, edge_weights, dcost_final, msg_edge_label, msg_norm_index, rho,

@@ -151,17 +151,24 @@ static void FN(cost_aggregate)(const mpo_geom* g, int enable_min_a_dir, REAL una
 }
 
 /* ---- CalLabelKernel: TRWP_forward.cu:8-29 (lowest label wins ties) ---------------------- */
-static void FN(cal_label)(const mpo_geom* g, const REAL* cost, uint8_t* label) {
+/* gap (optional diagnostic): second smallest cost minus the smallest, per pixel               */
+static void FN(cal_label)(const mpo_geom* g, const REAL* cost, uint8_t* label, REAL* gap) {
   int64_t P = mpo_pixels(g);
   for (int64_t p = 0; p < P; ++p) {
-    REAL mn = cost[p * g->L];
+    REAL mn = cost[p * g->L], second = (REAL)INFINITY;
     int arg = 0;
-    for (int l = 1; l < g->L; ++l)
-      if (cost[p * g->L + l] < mn) {
-        mn = cost[p * g->L + l];
+    for (int l = 1; l < g->L; ++l) {
+      REAL c = cost[p * g->L + l];
+      if (c < mn) {
+        second = mn;
+        mn = c;
         arg = l;
+      } else if (c < second) {
+        second = c;
       }
+    }
     label[p] = (uint8_t)arg;
+    if (gap) gap[p] = second - mn;
   }
 }
 
@@ -170,7 +177,7 @@ int FN(mpo_trwp_forward)(const mpo_geom* g, REAL rho, int n_iter, int enable_min
                          const REAL* unary, const REAL* context, const REAL* edge_weights,
                          REAL* msg, REAL* cost_final, uint8_t* msg_min_index,
                          uint8_t* msg_norm_index, uint8_t* label_all, REAL* gap_min,
-                         REAL* gap_norm) {
+                         REAL* gap_norm, REAL* gap_label) {
   int64_t N = mpo_plane(g), P = mpo_pixels(g);
   REAL* U = (REAL*)malloc(sizeof(REAL) * N);
   for (int it = 0; it < n_iter; ++it) {
@@ -184,7 +191,8 @@ int FN(mpo_trwp_forward)(const mpo_geom* g, REAL rho, int n_iter, int enable_min
     }
     if (label_all) {
       FN(cost_aggregate)(g, enable_min_a_dir, 1, unary, msg, cost_final);
-      FN(cal_label)(g, cost_final, label_all + (int64_t)it * P);
+      FN(cal_label)(g, cost_final, label_all + (int64_t)it * P,
+                    gap_label ? gap_label + (int64_t)it * P : NULL);
     }
   }
   FN(cost_aggregate)(g, enable_min_a_dir, 1, unary, msg, cost_final);
@@ -198,7 +206,7 @@ int FN(mpo_isgmr_forward)(const mpo_geom* g, int enable_sgm, REAL rho, int n_ite
                           int enable_min_a_dir, const REAL* unary, const REAL* context,
                           const REAL* edge_weights, REAL* msg, REAL* msg_update, REAL* cost_final,
                           uint8_t* msg_min_index, uint8_t* msg_norm_index, uint8_t* label_all,
-                          REAL* gap_min, REAL* gap_norm) {
+                          REAL* gap_min, REAL* gap_norm, REAL* gap_label) {
   int64_t N = mpo_plane(g), P = mpo_pixels(g);
   REAL* U = (REAL*)malloc(sizeof(REAL) * N);
   REAL factor = enable_sgm ? (REAL)g->n_dir : (REAL)1;
@@ -214,7 +222,8 @@ int FN(mpo_isgmr_forward)(const mpo_geom* g, int enable_sgm, REAL rho, int n_ite
     memcpy(msg, msg_update, sizeof(REAL) * N * g->n_dir); /* ISGMR_forward.cu:621-622 */
     if (label_all) {
       FN(cost_aggregate)(g, enable_min_a_dir, factor, unary, msg_update, cost_final);
-      FN(cal_label)(g, cost_final, label_all + (int64_t)it * P);
+      FN(cal_label)(g, cost_final, label_all + (int64_t)it * P,
+                    gap_label ? gap_label + (int64_t)it * P : NULL);
     }
   }
   FN(cost_aggregate)(g, enable_min_a_dir, factor, unary, msg_update, cost_final);
@@ -224,9 +233,12 @@ int FN(mpo_isgmr_forward)(const mpo_geom* g, int enable_sgm, REAL rho, int n_ite
 
 /* ---- scan-back kernels: TRWP_backward.cu:49-275 (ISGMR_backward.cu:62-288 identical) ---- */
 /* steps negated (common.cpp:89-92); front = current + negated step                          */
+/* same_label: the hard kernels of the TRWP_hard_soft build, which add to dcontext without    */
+/* the `current_d != front_d` guard (TRWP_hard_soft/TRWP_backward.cu:110,194,264)             */
 static void FN(sweep_back)(const mpo_geom* g, int dir, REAL rho, const REAL* context,
                            const REAL* w_dir, const uint8_t* idx_min, const uint8_t* idx_norm,
-                           REAL* dmsg_dir, REAL* dU, REAL* dcontext, REAL* dedge_dir) {
+                           REAL* dmsg_dir, REAL* dU, REAL* dcontext, REAL* dedge_dir,
+                           int same_label) {
   int L = g->L, H = g->H, W = g->W;
   int hs, ws;
   mpo_dir_step(dir, &hs, &ws);
@@ -258,7 +270,7 @@ static void FN(sweep_back)(const mpo_geom* g, int dir, REAL rho, const REAL* con
           dU[pf * L + fd] += v;
           dmsg_dir[pf * L + fd] += rho * v;
           dedge_dir[pc] += context[co] * v;
-          if (cd != fd) dcontext[co] += w_dir[pc] * v;
+          if (same_label || cd != fd) dcontext[co] += w_dir[pc] * v;
         }
       }
     }
@@ -285,7 +297,7 @@ static void FN(update_unary_back)(const mpo_geom* g, int dir, REAL rho, const RE
 int FN(mpo_trwp_backward)(const mpo_geom* g, REAL rho, int n_iter, const REAL* context,
                           const REAL* edge_weights, const REAL* dcost_final,
                           const uint8_t* msg_min_index, const uint8_t* msg_norm_index,
-                          REAL* dunary, REAL* dcontext, REAL* dedge_weights) {
+                          REAL* dunary, REAL* dcontext, REAL* dedge_weights, int same_label) {
   int64_t N = mpo_plane(g), P = mpo_pixels(g);
   REAL* dmsg = (REAL*)malloc(sizeof(REAL) * N * g->n_dir);
   REAL* dU = (REAL*)calloc(N, sizeof(REAL));
@@ -299,7 +311,7 @@ int FN(mpo_trwp_backward)(const mpo_geom* g, REAL rho, int n_iter, const REAL* c
       int64_t io = ((int64_t)it * g->n_dir + d);
       FN(sweep_back)(g, d, rho, context, edge_weights + (int64_t)d * P, msg_min_index + io * N,
                      msg_norm_index + io * P, dmsg + (int64_t)d * N, dU, dcontext,
-                     dedge_weights + (int64_t)d * P);
+                     dedge_weights + (int64_t)d * P, same_label);
       FN(update_unary_back)(g, d, rho, dU, dunary, dmsg);
       memset(dU, 0, sizeof(REAL) * N);                    /* :421 */
       memset(dmsg + (int64_t)d * N, 0, sizeof(REAL) * N); /* :422 */
@@ -331,7 +343,7 @@ int FN(mpo_isgmr_backward)(const mpo_geom* g, int enable_sgm, REAL rho, int n_it
       int64_t io = ((int64_t)it * g->n_dir + d);
       FN(sweep_back)(g, d, rho, context, edge_weights + (int64_t)d * P, msg_min_index + io * N,
                      msg_norm_index + io * P, dmsg_update + (int64_t)d * N, dU, dcontext,
-                     dedge_weights + (int64_t)d * P);
+                     dedge_weights + (int64_t)d * P, 0);
       FN(update_unary_back)(g, d, rho, dU, dunary, dmsg);
       memset(dU, 0, sizeof(REAL) * N);
       memset(dmsg_update + (int64_t)d * N, 0, sizeof(REAL) * N);
@@ -442,7 +454,7 @@ static void FN(sweep_soft)(const mpo_geom* g, int dir, REAL rho, const REAL* U, 
 int FN(mpo_trwp_soft_forward)(const mpo_geom* g, REAL rho, int n_iter, const REAL* unary,
                               const REAL* context, const REAL* edge_weights, REAL* msg,
                               REAL* cost_final, REAL* msg_edge_label, uint8_t* msg_norm_index,
-                              uint8_t* label_all) {
+                              uint8_t* label_all, REAL* gap_label) {
   int64_t N = mpo_plane(g), P = mpo_pixels(g);
   REAL* U = (REAL*)malloc(sizeof(REAL) * N);
   for (int it = 0; it < n_iter; ++it) {
@@ -455,7 +467,8 @@ int FN(mpo_trwp_soft_forward)(const mpo_geom* g, REAL rho, int n_iter, const REA
     }
     if (label_all) {
       FN(cost_aggregate)(g, 0, 1, unary, msg, cost_final); /* CostAggregateKernelSoft :142-159 */
-      FN(cal_label)(g, cost_final, label_all + (int64_t)it * P); /* CalLabelKernelSoft :119-140 */
+      FN(cal_label)(g, cost_final, label_all + (int64_t)it * P, /* CalLabelKernelSoft :119-140 */
+                    gap_label ? gap_label + (int64_t)it * P : NULL);
     }
   }
   FN(cost_aggregate)(g, 0, 1, unary, msg, cost_final);

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
   for name in names:
     assert hasattr(lib, name), name
   assert sorted(_lib.SYMBOLS) == names
-  assert lib.mpl_version() >= 100
+  assert lib.mpl_version() // 100 == 2
 
 
 def test_chain_counts_match_reference_tree_counts(oracle):
@@ -45,9 +45,10 @@ def test_shape_validation_answers_before_any_launch():
   one = ctypes.c_void_p(8)  # never dereferenced: validation fails first
 
   def fwd(shape, n_iter=1):
-    return lib.mpl_trwp_forward(shape, 0.5, n_iter, 0, one, one, one, one, one, None, None, one,
-                                None, None)
+    return lib.mpl_trwp_forward(shape, flags, 0.5, n_iter, 0, one, one, one, one, one, None, None,
+                                one, None, None)
 
+  flags = 0
   assert fwd(_lib.Shape(4, 1, 4, 4, 257, 0)) == -1
   assert b"n_disp" in lib.mpl_last_error()
   assert fwd(_lib.Shape(3, 1, 4, 4, 8, 0)) == -1
@@ -57,9 +58,16 @@ def test_shape_validation_answers_before_any_launch():
   assert b"2-D context" in lib.mpl_last_error()
   assert fwd(_lib.Shape(4, 1, 4, 4, 8, 0), n_iter=0) == -1
   assert fwd(_lib.Shape(4, 1, 40000, 40000, 8, 0)) == -1  # one image above 4 GiB
-  assert lib.mpl_isgmr_backward(_lib.Shape(4, 1, 4, 4, 8, 0), 0, 1.0, 1, one, one, one, one, one,
-                                one, one, one, None, None, None, None) == -1
+  assert lib.mpl_isgmr_backward(_lib.Shape(4, 1, 4, 4, 8, 0), 0, 0, 1.0, 1, one, one, one, one,
+                                one, one, one, one, None, None, None, None) == -1
   assert b"null" in lib.mpl_last_error()
+  # per-call flags: unknown bits and contradictory choices are refused
+  flags = 0x8000
+  assert fwd(_lib.Shape(4, 1, 4, 4, 8, 0)) == -1
+  assert b"flag" in lib.mpl_last_error()
+  flags = _lib.F_PACKED_OFF | _lib.F_PACKED_ALWAYS
+  assert fwd(_lib.Shape(4, 1, 4, 4, 8, 0)) == -1
+  assert b"exclude" in lib.mpl_last_error()
 
 
 def test_operators_refuse_cpu_tensors_loudly():

@@ -33,15 +33,16 @@ def test_config_matches_oracle(gpu, oracle, name, mode, scale, n_iter):
   train = cfg["training"]
   print("config", name, mode, unary.shape, "n_iter", n_iter, flush=True)
   ref = oracle.forward(mode, unary, ctx, ew, cfg["n_dir"], n_iter, cfg["rho"], training=train,
-                       want_gaps=train, saving_label=True)
+                       want_gaps=True, saving_label=True)
   got = gpu.gpu_forward(mode, unary, ctx, ew, cfg["n_dir"], n_iter, cfg["rho"], training=train,
                         saving_label=True)
   gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=ref["cost_final"])
   gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
-  assert (got["label_all"][-1] != ref["label_all"][-1]).mean() < 0.01
+  tol = 2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max()))
+  n_bad = gpu.assert_labels_match_off_ties(got["label_all"], ref["label_all"], ref["gap_label"], tol)
+  assert n_bad <= 1e-3 * ref["label_all"].size
   if not train:
     return
-  tol = 2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max()))
   n_bad = gpu.assert_indices_match_off_ties(got["msg_min_index"], ref["msg_min_index"],
                                             ref["gap_min"], tol, "msg_min_index")
   assert n_bad <= 1e-3 * ref["msg_min_index"].size
@@ -111,10 +112,11 @@ def test_module_forward_backward(gpu, oracle, mode, L, train_mode):
   en = np.ascontiguousarray(ew[:, None].transpose(2, 0, 1, 3, 4))
   dn = np.ascontiguousarray(dcost.transpose(0, 1, 3, 4, 2))
   rho = 0.5 if mode == "TRWP" else 1.0
-  ref = oracle.forward(mode, un, ctx, en, n_dir, n_iter, rho, saving_label=True)
+  ref = oracle.forward(mode, un, ctx, en, n_dir, n_iter, rho, saving_label=True, want_gaps=True)
   gpu.assert_values_close(cost.detach().cpu().numpy().transpose(0, 1, 3, 4, 2), ref["cost_final"],
                           what="module cost")
-  assert (labels.cpu().numpy() != ref["label_all"]).mean() < 0.01
+  gpu.assert_labels_match_off_ties(labels.cpu().numpy(), ref["label_all"], ref["gap_label"],
+                                   2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max())))
   du, dc, de = oracle.backward(mode, ctx.astype(np.float64), en.astype(np.float64),
                                dn.astype(np.float64), ref["msg_min_index"], ref["msg_norm_index"], rho)
   assert np.abs(u.grad.cpu().numpy().transpose(0, 1, 3, 4, 2) - du).max() <= 1e-4 * max(1, np.abs(du).max())

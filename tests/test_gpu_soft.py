@@ -73,12 +73,14 @@ def test_forward_soft_matches_oracle(gpu, oracle, n_dir, B, H, W, L, kind, n_ite
   ew = (0.2 + rng.random((n_dir, B, 1, H, W))).astype(np.float32)
   rho = 0.5
   print("case", n_dir, B, H, W, L, kind, n_iter, training, flush=True)
-  ref = oracle.forward_soft(unary, ctx, ew, n_dir, n_iter, rho, training=training, saving_label=True)
+  ref = oracle.forward_soft(unary, ctx, ew, n_dir, n_iter, rho, training=training, saving_label=True,
+                            want_gaps=True)
   got = gpu_forward_soft(unary, ctx, ew, n_dir, n_iter, rho, training=training, saving_label=True)
   belief = ref["cost_final"]
   gpu.assert_values_close(got["msg"], ref["msg"], rel=2e-5, what="msg", belief=belief)
   gpu.assert_values_close(got["cost_final"], ref["cost_final"], rel=2e-5, what="cost")
-  assert (got["label_all"] != ref["label_all"]).mean() <= 0.02
+  gpu.assert_labels_match_off_ties(got["label_all"], ref["label_all"], ref["gap_label"],
+                                   4e-5 * max(1.0, float(np.abs(belief).max())))
   if training:
     gpu.assert_values_close(got["msg_edge_label"], ref["msg_edge_label"], rel=2e-5, what="duals",
                             belief=belief)
@@ -165,13 +167,101 @@ def test_module_soft_forward_backward(gpu, oracle, L, train_mode):
                                     cost_index.cpu().numpy(), 0.5)
   assert np.abs(u.grad.cpu().numpy().transpose(0, 1, 3, 4, 2) - du).max() <= 1e-4 * max(1, np.abs(du).max())
   assert np.abs(e.grad.cpu().numpy()[:, None].transpose(2, 0, 1, 3, 4) - de).max() <= 1e-4 * max(1, np.abs(de).max())
-  assert mod.label_context.grad is None or True  # the parameter may be a plain tensor
+  if train_mode:
+    # the learned context: its gradient is the oracle's dcontext pulled back through the
+    # re-parameterisation of MP_module_hard_soft.py:148-163 (term weight first, then 2 * sigmoid,
+    # the diagonal pinned)
+    lc = torch.from_numpy(mod.label_context.detach().cpu().numpy().astype(np.float64)).requires_grad_(True)
+    eff = lc * args.mpnet_term_weight
+    loc, diag = mod.label_context_loc, mod.label_context_diag_loc
+    eff[loc] = 2 * torch.sigmoid(eff[loc].flatten())
+    eff[tuple(diag) if isinstance(diag, list) else diag] = args.mpnet_diag_value
+    eff.backward(torch.from_numpy(dc))
+    got_lc = mod.label_context.grad.cpu().numpy()
+    assert np.abs(lc.grad.numpy()).max() > 1e-3
+    assert np.abs(got_lc - lc.grad.numpy()).max() <= 1e-4 * max(1, np.abs(lc.grad.numpy()).max())
+  else:
+    assert mod.label_context.grad is None  # a fixed table: not a learnable parameter
   # hard mode through the same surface equals the plain TRWP module
   args.mpnet_enable_soft = False
   cost_h = mod(u.detach(), e.detach())[0]
   hard = oracle.forward("TRWP", un, ctx, en, n_dir, n_iter, 0.5)
   gpu.assert_values_close(cost_h.detach().cpu().numpy().transpose(0, 1, 3, 4, 2), hard["cost_final"],
                           what="hard mode")
+
+
+@pytest.mark.parametrize("L,n_dir", [(21, 4), (9, 8), (70, 4), (16, 4), (192, 4)])
+def test_module_hard_mode_backward_collects_same_label_terms(gpu, oracle, L, n_dir):
+  """mpnet_enable_soft = False with a context learned as it is (mpnet_smoothness_train = 'on'):
+  the module calls TRWP_hard_soft.backward (MP_module_hard_soft.py:95), whose dcontext also
+  collects the pairs with equal labels (TRWP_hard_soft/TRWP_backward.cu:110,194,264), so entry 0
+  of a 1-D table / the diagonal of a 2-D one get their gradient; TRWP.backward leaves them 0."""
+  import torch
+  from mplayers_amd import lib_stereo
+  from mplayers_amd.MP_module_hard_soft import MPModule
+  rng = np.random.default_rng(L + n_dir)
+  B, H, W, n_iter = 2, 6, 7, 2
+  args = argparse.Namespace(mpnet_mrf_mode="TRWP", mpnet_enable_soft=False, mpnet_max_iter=n_iter,
+                            mpnet_n_dirs=n_dir, n_classes=L, mpnet_term_weight=1.0,
+                            mpnet_smoothness_train="on", mpnet_smoothness_mode="TL",
+                            mpnet_smoothness_trunct_value=3, mpnet_smoothness_trunct_loc=-1,
+                            mpnet_diag_value=0.0, enable_symmetric=True, enable_cuda=True)
+  mod = MPModule(args, enable_create_label_context=True).cuda().train()
+  assert mod.label_context.requires_grad
+  with torch.no_grad():  # a table whose same-label entries matter
+    if L == 21:
+      mod.label_context.copy_(torch.from_numpy(
+          (np.triu(rng.random((L, L)), 1) + np.diag(0.1 + 0.3 * rng.random(L))).astype(np.float32)))
+    else:
+      mod.label_context[0] = 0.2
+  unary = rng.standard_normal((B, 1, L, H, W)).astype(np.float32)
+  ew = (0.1 + 0.9 * rng.random((B, n_dir, H, W))).astype(np.float32)
+  dcost = rng.standard_normal((B, 1, L, H, W)).astype(np.float32)
+  u = torch.from_numpy(unary).cuda().requires_grad_(True)
+  e = torch.from_numpy(ew).cuda().requires_grad_(True)
+  print("case", L, n_dir, flush=True)
+  cost = mod(u, e)[0]
+  cost.backward(torch.from_numpy(dcost).cuda())
+  torch.cuda.synchronize()
+  ctx = mod.label_context.detach().cpu().numpy()
+  un = np.ascontiguousarray(unary.transpose(0, 1, 3, 4, 2))
+  en = np.ascontiguousarray(ew[:, None].transpose(2, 0, 1, 3, 4))
+  dn = np.ascontiguousarray(dcost.transpose(0, 1, 3, 4, 2))
+  ref = oracle.forward("TRWP", un, ctx, en, n_dir, n_iter, 0.5)
+  gpu.assert_values_close(cost.detach().cpu().numpy().transpose(0, 1, 3, 4, 2), ref["cost_final"],
+                          what="hard mode cost")
+  du, dc, de = oracle.backward("TRWP", ctx.astype(np.float64), en.astype(np.float64),
+                               dn.astype(np.float64), ref["msg_min_index"], ref["msg_norm_index"],
+                               0.5, same_label=True)
+  same = np.diag(dc) if L == 21 else dc[:1]
+  assert np.abs(same).max() > 1e-2  # the terms the guarded operator drops are not small
+  got = mod.label_context.grad.cpu().numpy()
+  assert np.abs(got - dc).max() <= 1e-4 * max(1, np.abs(dc).max()), np.abs(got - dc).max()
+  assert np.abs(u.grad.cpu().numpy().transpose(0, 1, 3, 4, 2) - du).max() <= 1e-4 * max(1, np.abs(du).max())
+  assert np.abs(e.grad.cpu().numpy()[:, None].transpose(2, 0, 1, 3, 4) - de).max() <= 1e-4 * max(1, np.abs(de).max())
+  # the two operator namespaces on the oracle's indices: they differ in those entries only
+  t8 = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+  res = {}
+  for name, op in (("TRWP", lib_stereo.TRWP), ("TRWP_hard_soft", lib_stereo.TRWP_hard_soft)):
+    dctx = torch.zeros(ctx.shape, device="cuda")
+    dunary = torch.empty(un.shape, device="cuda")
+    dedge = torch.zeros(en.shape, device="cuda")
+    op.backward(0.5, t8(ctx), t8(en), t8(dn), t8(ref["msg_min_index"]), t8(ref["msg_norm_index"]),
+                dunary, dctx, dedge, torch.empty((n_dir,) + un.shape, device="cuda"),
+                torch.empty(0, device="cuda"))
+    torch.cuda.synchronize()
+    res[name] = (dunary.cpu().numpy(), dctx.cpu().numpy(), dedge.cpu().numpy())
+  assert np.array_equal(res["TRWP"][0], res["TRWP_hard_soft"][0])
+  assert np.array_equal(res["TRWP"][2], res["TRWP_hard_soft"][2])
+  guarded, full = res["TRWP"][1], res["TRWP_hard_soft"][1]
+  if L == 21:
+    assert np.all(np.diag(guarded) == 0)
+    off = ~np.eye(L, dtype=bool)
+    assert np.abs(guarded[off] - full[off]).max() <= 1e-5 * max(1, np.abs(full).max())
+  else:
+    assert guarded[0] == 0
+    assert np.abs(guarded[1:] - full[1:]).max() <= 1e-5 * max(1, np.abs(full).max())
+  assert np.abs(full - dc).max() <= 1e-4 * max(1, np.abs(dc).max())
 
 
 def test_soft_refuses_more_than_64_labels(gpu):

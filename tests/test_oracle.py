@@ -216,6 +216,50 @@ def test_backward_matches_finite_differences(oracle, mode, rho, n_dir, ctx2d):
   assert abs(du.sum() - factor * dcost.sum()) < 1e-9
 
 
+@pytest.mark.parametrize("n_dir,ctx2d", [(4, False), (8, True), (16, True), (8, False)])
+def test_hard_soft_backward_collects_the_same_label_terms(oracle, n_dir, ctx2d):
+  """The hard backward of the reference's TRWP_hard_soft build drops the `current_d != front_d`
+  guard (TRWP_hard_soft/TRWP_backward.cu:110 against TRWP/TRWP_backward.cu:111-112): entry 0 of a
+  1-D table / the diagonal of a 2-D one then receive their true gradient, which finite differences
+  of the forward pass pin; every other output is what the guarded backward gives."""
+  rng = np.random.default_rng(11)
+  B, H, W, L, n_iter, rho = 1, 4, 5, 3, 2, 0.5
+  unary, ctx, ew = _rand_problem(rng, n_dir, B, H, W, L, ctx2d)
+  if ctx2d:
+    ctx = ctx + np.diag(0.2 + rng.random(L))  # a diagonal that matters
+  else:
+    ctx[0] = 0.3
+  dcost = rng.standard_normal(unary.shape)
+
+  def loss(c):
+    o = oracle.forward("TRWP", unary, c, ew, n_dir, n_iter, rho, training=False, ctx2d=ctx2d)
+    return float((o["cost_final"] * dcost).sum())
+
+  out = oracle.forward("TRWP", unary, ctx, ew, n_dir, n_iter, rho, ctx2d=ctx2d)
+  args = ("TRWP", ctx, ew, dcost, out["msg_min_index"], out["msg_norm_index"], rho)
+  du0, dc0, de0 = oracle.backward(*args, ctx2d=ctx2d)
+  du1, dc1, de1 = oracle.backward(*args, ctx2d=ctx2d, same_label=True)
+  assert np.array_equal(du0, du1) and np.array_equal(de0, de1)
+  eps = 1e-6
+  entries = [(i, j) for i in range(L) for j in range(i, L)] if ctx2d else [(k,) for k in range(L)]
+  seen_nonzero = False
+  for idx in entries:
+    hi, lo = ctx.copy(), ctx.copy()
+    hi[idx] += eps
+    lo[idx] -= eps
+    g = (loss(hi) - loss(lo)) / (2 * eps)
+    assert abs(g - dc1[idx]) < 1e-6, idx
+    same = (idx[0] == idx[1]) if ctx2d else (idx[0] == 0)
+    if same:
+      assert dc0[idx] == 0
+      seen_nonzero |= abs(dc1[idx]) > 1e-3
+    else:
+      assert dc0[idx] == dc1[idx]
+  assert seen_nonzero  # the guarded operator really loses something
+  if ctx2d:
+    assert np.all(np.tril(dc1, -1) == 0)
+
+
 @pytest.mark.parametrize("n_dir", [4, 8])
 def test_isgmr_flip_and_transpose_permute_directions(oracle, n_dir):
   rng = np.random.default_rng(21)
