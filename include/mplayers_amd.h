@@ -196,6 +196,18 @@ int mpl_edge_shift(int mode, const float* image, int batch, int channels, int he
                    int n_dirs, float sigma, float threshold, float penalty, float* out,
                    double* dir_sums, void* stream);
 
+/* mpl_edge_shift for callers that cannot allocate or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results as mpl_edge_shift without dir_sums: the per-direction
+ * sums of CUE_BINARY live in a static device array of the library (MPL_MAX_DIRS doubles, 128
+ * bytes on every GPU the library runs on, held until the process ends), whose address is resolved
+ * on the first call on a device.  The call allocates nothing; n_dirs beyond MPL_MAX_DIRS is refused
+ * with MPL_EINVAL.  All calls on one GPU share that array (it is cleared by a kernel at the start
+ * of each call): calls that overlap on one GPU, on different streams, race. */
+int mpl_edge_shift_static(int mode, const float* image, int batch, int channels, int height,
+                          int width, int n_dirs, float sigma, float threshold, float penalty,
+                          float* out, void* stream);
+
 /* Stereo data term, the layers' upstream in the reference's energy-minimisation driver: replaces
  * computeDSI (MPLayers/aux/aux.cpp:5-98) as called by compute_all_terms
  * (MPLayers/aux/auxPy.cpp:22,62-66: birchfield = 1, squared_diffs = 0, trunc_diffs = 255).

@@ -7,7 +7,8 @@ LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hi
 
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
            "mpl_selftest_wave_ops", "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
-           "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_trwp_soft_forward",
+           "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_edge_shift_static",
+           "mpl_trwp_soft_forward",
            "mpl_trwp_soft_backward", "mpl_soft_weighted_message", "mpl_soft_weighted_message_back", "mpl_set_option",
            "mpl_stereo_data_cost", "mpl_gradient_cues", "mpl_mrf_energy", "mpl_probe_copy", "mpl_transpose")
 
@@ -59,6 +60,7 @@ def load():
   lib.mpl_soft_weighted_message_back.argtypes = [ci, ci, vp, vp, vp, vp, vp]
   lib.mpl_set_option.argtypes = [ci, ci]
   lib.mpl_edge_shift.argtypes = [ci, vp, ci, ci, ci, ci, ci, cf, cf, cf, vp, vp, vp]
+  lib.mpl_edge_shift_static.argtypes = [ci, vp, ci, ci, ci, ci, ci, cf, cf, cf, vp, vp]
   lib.mpl_stereo_data_cost.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, ci, vp, vp]
   lib.mpl_gradient_cues.argtypes = [vp, ci, ci, ci, ci, cf, vp, vp, vp]
   lib.mpl_mrf_energy.argtypes = [sp, ci, vp, vp, vp, vp, vp, vp]

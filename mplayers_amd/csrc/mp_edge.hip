@@ -10,6 +10,8 @@
 // value is read once; the image is small next to the n_dirs output planes, so the kernel is bound
 // by its writes.
 
+#include <mutex>
+
 #include "mp_common.h"
 
 using namespace mpl;
@@ -158,35 +160,20 @@ int blocks_for(int64_t n) {
   return (int)b;
 }
 
-int edge_fail(const char* msg) { return fail(MPL_EINVAL, "%s", msg); }
-
-}  // namespace
-
-extern "C" {
-
-int mpl_edge_shift(int mode, const float* image, int batch, int channels, int height, int width,
-                   int n_dirs, float sigma, float threshold, float penalty, float* out,
-                   double* dir_sums, void* stream) {
-  if (image == nullptr || out == nullptr) return edge_fail("edge_shift: null tensor pointer");
-  if (batch < 1 || channels < 1 || height < 1 || width < 1)
-    return edge_fail("edge_shift: batch/channels/height/width must be positive");
-  if (n_dirs < 0 || n_dirs > kMaxDirs) return edge_fail("edge_shift: n_dirs must be in [0, 16]");
-  if (mode < 0 || mode >= MPL_EDGE_MODES) return edge_fail("edge_shift: unknown mode");
-  if ((int64_t)height * width > 0x7fffffff) return edge_fail("edge_shift: more than 2^31 pixels");
+// the body of both entry points; sums: 16 doubles of device scratch (kernel_cue_binary only)
+int edge_shift_run(const char* who, int mode, const float* image, int batch, int channels,
+                   int height, int width, int n_dirs, float sigma, float threshold, float penalty,
+                   float* out, double* sums, hipStream_t st) {
+  if (n_dirs == 0) return MPL_OK;
   const bool reduce = mode == MPL_EDGE_SUPERPIXEL || mode == MPL_EDGE_CUE_REAL ||
                       mode == MPL_EDGE_CUE_BINARY || mode == MPL_EDGE_THRESHOLD;
-  if (reduce && batch != 1)
-    return edge_fail("edge_shift: the channel-reducing modes take one image (batch == 1)");
-  if (mode == MPL_EDGE_CUE_BINARY && dir_sums == nullptr)
-    return edge_fail("edge_shift: kernel_cue_binary needs the dir_sums scratch (16 doubles)");
-  if (n_dirs == 0) return MPL_OK;
-  hipStream_t st = (hipStream_t)stream;
   const int64_t HW = (int64_t)height * width;
   if (!reduce) {
     edge_shift_channel_kernel<<<blocks_for((int64_t)batch * channels * HW), 256, 0, st>>>(
         image, mode, n_dirs, batch, channels, height, width, out);
   } else {
-    double* sums = (mode == MPL_EDGE_CUE_BINARY) ? dir_sums : nullptr;
+    if (mode != MPL_EDGE_CUE_BINARY) sums = nullptr;
+    // cleared by a kernel, not a memset node: the call may be captured into a graph
     if (sums != nullptr) zero_sums_kernel<<<1, kWave, 0, st>>>(sums, kMaxDirs);
     edge_shift_reduce_kernel<<<blocks_for(HW), 256, 0, st>>>(image, mode, n_dirs, channels, height,
                                                             width, sigma, threshold, penalty, out,
@@ -196,8 +183,88 @@ int mpl_edge_shift(int mode, const float* image, int batch, int channels, int he
           n_dirs, channels, height, width, sums, out);
   }
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(MPL_ELAUNCH, "edge_shift: %s", hipGetErrorString(e));
+  if (e != hipSuccess) return fail(MPL_ELAUNCH, "%s: %s", who, hipGetErrorString(e));
   return MPL_OK;
+}
+
+int edge_shift_check(const char* who, int mode, const float* image, int batch, int channels,
+                     int height, int width, int n_dirs, const float* out) {
+  if (image == nullptr || out == nullptr) return fail(MPL_EINVAL, "%s: null tensor pointer", who);
+  if (batch < 1 || channels < 1 || height < 1 || width < 1)
+    return fail(MPL_EINVAL, "%s: batch/channels/height/width must be positive", who);
+  if (n_dirs < 0 || n_dirs > kMaxDirs)
+    return fail(MPL_EINVAL, "%s: n_dirs must be in [0, %d], got %d", who, kMaxDirs, n_dirs);
+  if (mode < 0 || mode >= MPL_EDGE_MODES) return fail(MPL_EINVAL, "%s: unknown mode %d", who, mode);
+  if ((int64_t)height * width > 0x7fffffff) return fail(MPL_EINVAL, "%s: more than 2^31 pixels", who);
+  const bool reduce = mode == MPL_EDGE_SUPERPIXEL || mode == MPL_EDGE_CUE_REAL ||
+                      mode == MPL_EDGE_CUE_BINARY || mode == MPL_EDGE_THRESHOLD;
+  if (reduce && batch != 1)
+    return fail(MPL_EINVAL, "%s: the channel-reducing modes take one image (batch == 1)", who);
+  return MPL_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Library-owned scratch of mpl_edge_shift_static: the per-direction sums of kernel_cue_binary, one
+// double per direction of the 16-direction table (128 bytes).  Every GPU the library runs on holds
+// its own copy of this array, at its own address, until the process ends.  In host code the name
+// is only a handle for hipGetSymbolAddress: kernels and fills take the resolved device pointer.
+// ------------------------------------------------------------------------------------------------
+constexpr int kStaticSums = MPL_MAX_DIRS;  // the most directions one call can ask for
+static __device__ __align__(256) double scratch[kStaticSums];
+
+constexpr int kMaxDevices = 64;
+double* g_scratch_ptr[kMaxDevices];  // resolved address of `scratch` per device, null until asked
+std::mutex g_scratch_mu;
+
+// address of this device's copy of `scratch`; resolved once per device, with that device current
+int static_sums(const char* who, double** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MPL_ELAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(MPL_EINVAL, "%s: device ordinal %d outside [0, %d)", who, dev, kMaxDevices);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    double* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(MPL_ELAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", who, dev,
+                  hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MPL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mpl_edge_shift(int mode, const float* image, int batch, int channels, int height, int width,
+                   int n_dirs, float sigma, float threshold, float penalty, float* out,
+                   double* dir_sums, void* stream) {
+  int rc = edge_shift_check("edge_shift", mode, image, batch, channels, height, width, n_dirs, out);
+  if (rc != MPL_OK) return rc;
+  if (mode == MPL_EDGE_CUE_BINARY && dir_sums == nullptr)
+    return fail(MPL_EINVAL, "edge_shift: kernel_cue_binary needs the dir_sums scratch (16 doubles)");
+  return edge_shift_run("edge_shift", mode, image, batch, channels, height, width, n_dirs, sigma,
+                        threshold, penalty, out, dir_sums, (hipStream_t)stream);
+}
+
+int mpl_edge_shift_static(int mode, const float* image, int batch, int channels, int height,
+                          int width, int n_dirs, float sigma, float threshold, float penalty,
+                          float* out, void* stream) {
+  const char* who = "edge_shift_static";
+  if (n_dirs > kStaticSums)
+    return fail(MPL_EINVAL, "%s: %d directions asked for, the library's static scratch holds the "
+                "sums of at most %d", who, n_dirs, kStaticSums);
+  int rc = edge_shift_check(who, mode, image, batch, channels, height, width, n_dirs, out);
+  if (rc != MPL_OK) return rc;
+  double* sums = nullptr;
+  if ((rc = static_sums(who, &sums)) != MPL_OK) return rc;
+  // the array keeps the previous call's sums: edge_shift_run clears it before it accumulates
+  return edge_shift_run(who, mode, image, batch, channels, height, width, n_dirs, sigma, threshold,
+                        penalty, out, sums, (hipStream_t)stream);
 }
 
 }  // extern "C"
