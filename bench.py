@@ -22,15 +22,32 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per launch of the scan kernels at the full-size large configuration, measured with
+# HBM bytes per launch of the scan kernels at the full-size large configuration were measured with
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (one counter per run) and scaled by what the
-# same counters read for a plain device copy of one plane (FETCH_SIZE x2.0, WRITE_SIZE x1.0); the
-# summary of those runs is kept under profiles/.  Counters cannot be read from inside this script.
-MEASURED_TRAFFIC_BYTES = {
-    ("C5", 1.0, True): {"fwd_sweep": 10.57e9, "bwd_sweep": 11.65e9,
-                        # ISGMR: scan + its element-wise companion pass
-                        "fwd_sweep_all": 43.98e9 + 29.95e9, "bwd_sweep_all": 47.13e9 + 30.41e9},
-}
+# same counters read for a plain device copy of one plane; counters cannot be read from inside this
+# script, so the figure is taken from the committed summary of those runs: the table row whose
+# first cell names the kernel kind ("bwd_sweep", ...), column "HBM GB / launch".
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "c5_trwp_isgmr_hbm_traffic.md")
+
+
+def measured_traffic_bytes(kind, cfg_name, scale, training):
+  """HBM bytes per launch of kernel `kind` from the committed counter summary; None when the
+  summary is absent or covers another workload."""
+  if (cfg_name, scale, training) != ("C5", 1.0, True) or not os.path.exists(TRAFFIC_SUMMARY):
+    return None
+  col = None
+  for line in open(TRAFFIC_SUMMARY):
+    cells = [c.strip() for c in line.strip().strip("|").split("|")]
+    if col is None:
+      if "HBM GB / launch" in cells:
+        col = cells.index("HBM GB / launch")
+      continue
+    if cells and cells[0].strip("`") == kind and col < len(cells):
+      try:
+        return float(cells[col]) * 1e9
+      except ValueError:
+        return None
+  return None
 
 
 def parse():
@@ -61,10 +78,15 @@ def parse():
   ap.add_argument("--edge-probe", action="store_true",
                   help="also time the edge-weight producer on an image of the workload's size "
                        "(reported under \"edge_weights\")")
-  ap.add_argument("--caller-clears-messages", action="store_true",
-                  help="the reference's contract: the step zero-fills `msg` and the operators read "
-                       "it as initial messages (default: msg_uninit=1, the library starts the "
-                       "messages at zero itself and the step does not touch `msg` beforehand)")
+  ap.add_argument("--msg-uninit", action="store_true",
+                  help="headline under the library's MPL_F_MSG_UNINIT extension: the library starts "
+                       "the messages at zero itself and the step does not touch `msg` beforehand "
+                       "(default: the reference's operator contract, the step zero-fills `msg` "
+                       "inside the timed region and the operators read it as initial messages; the "
+                       "other contract is timed over the same number of steps and reported beside it)")
+  ap.add_argument("--dunary-only", action="store_true",
+                  help="backward without dcontext and dedge_weights (a fixed pairwise table and "
+                       "edge weights that are not learned); not the headline workload")
   ap.add_argument("--graph-probe", action="store_true",
                   help="also capture one step in a HIP graph and time its replays (the library only "
                        "launches kernels, so a step is capturable; reported under \"graph_replay\")")
@@ -74,12 +96,27 @@ def parse():
   return ap.parse_args()
 
 
-def cpu_baseline(cfg, budget_s=15.0):
+def host_cpu():
+  """Model name and logical CPU count of this host, and the thread share the harness grants."""
+  model = "unknown"
+  try:
+    for line in open("/proc/cpuinfo"):
+      if line.startswith("model name"):
+        model = line.split(":", 1)[1].strip()
+        break
+  except OSError:
+    pass
+  share = os.environ.get("OMP_NUM_THREADS")
+  return model, os.cpu_count(), int(share) if share and share.isdigit() else None
+
+
+def cpu_baseline(cfg, budget_s=12.0):
   """Times the reference's CPU forward path (built from the reference sources into oracle/_ref)
   or, where that build is absent, the oracle's restatement of the same loop nest, on a crop of
   the workload: full-width rows, one iteration, unit edge weights (that path ignores them),
   forward only (the reference has no CPU backward).  A short calibration run sizes the crop so
-  that the timed run takes about budget_s seconds."""
+  that the timed run takes about budget_s seconds.  The reference hard-codes 16 OpenMP threads;
+  the restatement is timed a second time on every core this process may use."""
   import numpy as np
   from oracle import mp_oracle, ref_cpu
   L, n_dir, W = cfg["L"], cfg["n_dir"], cfg["W"]
@@ -94,25 +131,43 @@ def cpu_baseline(cfg, budget_s=15.0):
   table = np.ascontiguousarray(np.broadcast_to(table, (n_dir, L, L)), dtype=np.float32)
   kind = "reference" if ref_cpu.available() else "port"
 
-  def run(rows):
+  def run(rows, which, n_threads):
     unary = cfg["unary"][:1, :, :rows, :, :].contiguous().numpy()
     t0 = time.perf_counter()
-    if kind == "reference":
+    if which == "reference":
       ref_cpu.forward(mode, unary, table, n_dir, 1, cfg["rho"])
     else:
-      mp_oracle.refcpu_forward(mode, unary, table, n_dir, 1, cfg["rho"], n_threads=threads,
+      mp_oracle.refcpu_forward(mode, unary, table, n_dir, 1, cfg["rho"], n_threads=n_threads,
                                context_per_dir=True, ctx2d=(L == 21))
     return time.perf_counter() - t0
 
   rows0 = min(cfg["H"], 4)
-  dt0 = run(rows0)
+  dt0 = run(rows0, kind, threads)
   rows = int(max(rows0, min(cfg["H"], rows0 * budget_s / max(dt0, 1e-3))))
-  dt = run(rows) if rows > rows0 else dt0
+  dt = run(rows, kind, threads) if rows > rows0 else dt0
   units = rows * W * L * 1
-  return {"value": units / dt, "unit": "pixel*label*iter/s", "cores": threads, "kind": kind,
-          "sample": "%s forward only (the reference has no CPU backward), first %d rows x %d "
-                    "columns of %s, %d labels, %d directions, 1 iteration, unit edge weights, "
-                    "%.1f s" % (mode, rows, W, cfg["name"], L, n_dir, dt)}
+  model, nproc, share = host_cpu()
+  # every core this process may use: the affinity mask, capped by the harness's thread share
+  try:
+    usable = len(os.sched_getaffinity(0))
+  except AttributeError:
+    usable = nproc or threads
+  all_cores = min(usable, share) if share else usable
+  dt_all = run(rows, "port", all_cores)
+  out = {"value": units / dt, "unit": "pixel*label*iter/s", "cores": threads, "kind": kind,
+         "sample": "%s forward only (the reference has no CPU backward), first %d rows x %d "
+                   "columns of %s, %d labels, %d directions, 1 iteration, unit edge weights, "
+                   "%.1f s" % (mode, rows, W, cfg["name"], L, n_dir, dt),
+         "host_cpu": model, "nproc": nproc, "usable_cores": usable, "thread_share": share,
+         "all_cores": {"kind": "port", "cores": all_cores, "value": units / dt_all,
+                       "seconds": round(dt_all, 2),
+                       "note": "the restatement of the same loop nest (oracle/mp_oracle.c) on every "
+                               "core this process may use; the reference's own build cannot change "
+                               "its 16 threads"},
+         "compile_flags": {"reference": "g++ -O2 -std=c++17 -fopenmp (oracle/build_ref.py, the "
+                                        "reference's sources compiled in place)",
+                           "port": "gcc -O2 -ffp-contract=off -fopenmp (oracle/Makefile)"}}
+  return out
 
 
 def peak_probe(H, W, L, dev, reps=5):
@@ -274,13 +329,20 @@ def main():
   else:
     imin = inorm = empty
 
-  uninit = not a.caller_clears_messages
+  uninit = bool(a.msg_uninit)
+  if training and a.dunary_only:
+    dedge = dctx = torch.empty(0, **f32)
 
   def step(uninit=uninit):
     for alg in algs:
       rho = 1.0 if alg == "ISGMR" else 0.5
       if alg == "SOFT" or not uninit:
         msg.zero_()
+      if training and not a.dunary_only:
+        # the accumulating gradients must arrive zero-filled (the reference's caller allocates
+        # them with new_zeros on every call, MP_module.py:65-74)
+        dedge.zero_()
+        dctx.zero_()
       if alg == "SOFT":
         lib_stereo.TRWP_hard_soft.forward_soft(rho, n_iter, unary, context, edge, msg, soft_blocks,
                                                inorm, cost, belief, empty)
@@ -350,7 +412,8 @@ def main():
       kernels[kind]["companion_pass"] = companion
       kernels[kind]["companion_avg_ms"] = stats[companion][1] / n
   dominant = max(kernels, key=lambda k: kernels[k]["total_ms"])
-  traffic = MEASURED_TRAFFIC_BYTES.get((cfg["name"], a.scale, training), {}).get(dominant)
+  traffic = None if a.dunary_only else measured_traffic_bytes(dominant, cfg["name"], a.scale,
+                                                              training)
   roofline = {"bound": "hbm", "kernel": dominant, "achieved": kernels[dominant]["achieved_GBs"],
               "peak": HBM_PEAK_GBS, "unit": "GB/s",
               "frac": kernels[dominant]["achieved_GBs"] / HBM_PEAK_GBS, "traffic": traffic,
@@ -370,9 +433,14 @@ def main():
                                              "fwd+bwd" if training else "fwd", B, H, W, L, n_dir,
                                              n_iter),
                  "scale": a.scale,
-                 "initial_messages": ("zero by declaration (msg_uninit): the library writes every "
-                                      "element itself" if uninit else
-                                      "tensor cleared by the caller inside the timed step")},
+                 "initial_messages": ("zero by declaration (MPL_F_MSG_UNINIT): the library writes "
+                                      "every element itself" if uninit else
+                                      "the reference's operator contract: `msg` cleared by the "
+                                      "caller inside the timed step and read as initial messages"),
+                 "gradients": ("none" if not training else
+                               "dunary only" if a.dunary_only else
+                               "dunary, dcontext, dedge_weights (the two accumulating ones cleared "
+                               "inside the timed step)")},
       "roofline": roofline,
       "whole_step_frac_of_hbm_roofline": whole,
       "contract_bytes_per_unit": contract,
@@ -381,21 +449,23 @@ def main():
       "other_kernels_ms": {k: round(stats[k][1], 3) for k in stats if k not in kernels},
 
   }
-  if uninit and "SOFT" not in algs:
-    # the same step under the reference's contract, for comparison: `msg` zero-filled by the
-    # caller inside the step and read back by the operators as initial messages
-    n_ref = min(3, a.steps)
-    step(uninit=False)
+  if "SOFT" not in algs:
+    # the same step under the other contract for the initial messages, over the same number of
+    # steps: zero by declaration (the library's extension, what its nn.Module passes) when the
+    # headline is the reference's operator contract, and the other way round
+    for _ in range(min(2, a.warmup)):
+      step(uninit=not uninit)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(n_ref):
-      step(uninit=False)
+    for _ in range(a.steps):
+      step(uninit=not uninit)
     torch.cuda.synchronize()
-    ref_ms = (time.perf_counter() - t0) / n_ref * 1e3
-    out["caller_cleared_messages"] = {"ms_per_step": ref_ms, "steps": n_ref,
-                                      "value": units_per_step / (ref_ms * 1e-3)}
-  if a.peak_probe:
-    out["measured_stream_rates"] = peak_probe(H, W, L, dev)
+    alt_ms = (time.perf_counter() - t0) / a.steps * 1e3
+    out["msg_uninit" if not uninit else "caller_cleared_messages"] = {
+        "ms_per_step": alt_ms, "steps": a.steps, "value": units_per_step / (alt_ms * 1e-3)}
+  if a.peak_probe or (cfg["name"] == "C5" and a.scale == 1.0):
+    # what this GPU sustains for traffic of the kernels' shapes, next to the published 8 TB/s
+    out["measured_stream_rates"] = peak_probe(H, W, L, dev, reps=5 if a.peak_probe else 2)
   if a.module_probe and training:
     out["module_surface"] = module_probe(cfg, algs, unary, edge, dcost)
   if a.edge_probe:

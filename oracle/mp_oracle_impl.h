@@ -38,6 +38,7 @@ static void FN(update_unary)(const mpo_geom* g, int dir, REAL rho, const REAL* u
                              const REAL* msg, REAL* U) {
   int64_t N = mpo_plane(g);
   int inv = dir ^ 1; /* common.cpp:23-26 */
+#pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < N; ++i) {
     REAL v = unary[i];
     for (int k = 0; k < g->n_dir; ++k) v += msg[(int64_t)k * N + i];
@@ -104,29 +105,35 @@ static void FN(sweep)(const mpo_geom* g, int dir, REAL rho, const REAL* U, const
   int hs, ws;
   mpo_dir_step(dir, &hs, &ws);
   int n_trees = mpo_n_trees(dir, H, W);
-  REAL* prev = (REAL*)malloc(sizeof(REAL) * L);
-  REAL* tmp = (REAL*)malloc(sizeof(REAL) * L);
-  for (int bv = 0; bv < g->B; ++bv) {
-    int64_t pix_base = (int64_t)bv * H * W;
-    for (int tree = 0; tree < n_trees; ++tree) {
-      int h0, w0, n_roll;
-      mpo_tree_start(dir, hs, ws, H, W, tree, &h0, &w0, &n_roll);
-      for (int l = 0; l < L; ++l) prev[l] = 0; /* shared vector zeroed per block */
-      for (int i = 0; i <= n_roll; ++i) {
-        int ch = h0 + i * hs, cw = w0 + i * ws;
-        int fh = ch - hs, fw = cw - ws;
-        if (ch < 0 || ch >= H || cw < 0 || cw >= W || fh < 0 || fh >= H || fw < 0 || fw >= W)
-          continue;
-        int64_t pc = pix_base + (int64_t)ch * W + cw;
-        int64_t pf = pix_base + (int64_t)fh * W + fw;
-        FN(pixel_step)(L, g->ctx2d, rho, U + pf * L, context, w_dir[pc], prev, tmp, m_out + pc * L,
-                       idx_min ? idx_min + pc * L : NULL, idx_norm ? idx_norm + pc : NULL,
-                       gap_min ? gap_min + pc * L : NULL, gap_norm ? gap_norm + pc : NULL);
+  /* chains ("trees", one block each in the reference) are independent: one thread per chain */
+#pragma omp parallel
+  {
+    REAL* prev = (REAL*)malloc(sizeof(REAL) * L);
+    REAL* tmp = (REAL*)malloc(sizeof(REAL) * L);
+#pragma omp for collapse(2) schedule(dynamic, 4)
+    for (int bv = 0; bv < g->B; ++bv) {
+      for (int tree = 0; tree < n_trees; ++tree) {
+        int64_t pix_base = (int64_t)bv * H * W;
+        int h0, w0, n_roll;
+        mpo_tree_start(dir, hs, ws, H, W, tree, &h0, &w0, &n_roll);
+        for (int l = 0; l < L; ++l) prev[l] = 0; /* shared vector zeroed per block */
+        for (int i = 0; i <= n_roll; ++i) {
+          int ch = h0 + i * hs, cw = w0 + i * ws;
+          int fh = ch - hs, fw = cw - ws;
+          if (ch < 0 || ch >= H || cw < 0 || cw >= W || fh < 0 || fh >= H || fw < 0 || fw >= W)
+            continue;
+          int64_t pc = pix_base + (int64_t)ch * W + cw;
+          int64_t pf = pix_base + (int64_t)fh * W + fw;
+          FN(pixel_step)(L, g->ctx2d, rho, U + pf * L, context, w_dir[pc], prev, tmp,
+                         m_out + pc * L, idx_min ? idx_min + pc * L : NULL,
+                         idx_norm ? idx_norm + pc : NULL, gap_min ? gap_min + pc * L : NULL,
+                         gap_norm ? gap_norm + pc : NULL);
+        }
       }
     }
+    free(prev);
+    free(tmp);
   }
-  free(prev);
-  free(tmp);
 }
 
 /* ---- CostAggregateKernel: TRWP_forward.cu:31-58, ISGMR_forward.cu:69-99 --------------- */
