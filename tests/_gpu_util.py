@@ -13,7 +13,11 @@ def _t(a, dtype=torch.float32):
 
 
 def gpu_forward(mode, unary, context, edge_weights, n_dir, n_iter, rho, training=True,
-                saving_label=False, enable_min_a_dir=False, enable_sgm=False, msg_init=None):
+                saving_label=False, enable_min_a_dir=False, enable_sgm=False, msg_init=None,
+                ops=None):
+  """ops: a namespace with TRWP / ISGMR operator modules in the reference's calling convention
+  (default: mplayers_amd.lib_stereo, the ctypes operators)."""
+  ops = lib_stereo if ops is None else ops
   unary = _t(unary)
   b, cv, h, w, L = unary.shape
   context = _t(context)
@@ -28,12 +32,12 @@ def gpu_forward(mode, unary, context, edge_weights, n_dir, n_iter, rho, training
   inorm = unary.new_zeros(n_iter, n_dir, b, cv, h, w, **u8) if training else torch.empty(0, **u8)
   label = unary.new_zeros(n_iter, b, cv, h, w, **u8) if saving_label else torch.empty(0, **u8)
   if mode == "TRWP":
-    lib_stereo.TRWP.forward(rho, n_iter, int(enable_min_a_dir), unary, context, edge_weights, msg,
-                            cost, imin, inorm, scratch, label)
+    ops.TRWP.forward(rho, n_iter, int(enable_min_a_dir), unary, context, edge_weights, msg,
+                     cost, imin, inorm, scratch, label)
   else:
     msg_update = torch.zeros_like(msg)
-    lib_stereo.ISGMR.forward(int(enable_sgm), rho, n_iter, int(enable_min_a_dir), unary, context,
-                             edge_weights, msg, cost, imin, inorm, scratch, msg_update, label)
+    ops.ISGMR.forward(int(enable_sgm), rho, n_iter, int(enable_min_a_dir), unary, context,
+                      edge_weights, msg, cost, imin, inorm, scratch, msg_update, label)
   torch.cuda.synchronize()
   return dict(msg=msg.cpu().numpy(), cost_final=cost.cpu().numpy(),
               msg_min_index=imin.cpu().numpy() if training else None,
@@ -44,9 +48,12 @@ def gpu_forward(mode, unary, context, edge_weights, n_dir, n_iter, rho, training
 
 def gpu_backward(mode, context, edge_weights, dcost, msg_min_index, msg_norm_index, rho,
                  enable_sgm=False, garbage_scratch=False, flags=0, want_dctx=True, want_dedge=True,
-                 hard_soft=False):
+                 hard_soft=False, ops=None):
   """want_dctx / want_dedge False: that gradient is passed as an empty tensor (not wanted) and
-  comes back as None.  hard_soft: the TRWP_hard_soft namespace's hard backward."""
+  comes back as None.  hard_soft: the TRWP_hard_soft namespace's hard backward.  ops: as for
+  gpu_forward (such operators take the reference's arguments only: no flags)."""
+  kw = dict(flags=flags) if ops is None else {}
+  ops = lib_stereo if ops is None else ops
   n_iter, n_dir, b, cv, h, w, L = msg_min_index.shape
   context = _t(context)
   if edge_weights is None:
@@ -63,13 +70,13 @@ def gpu_backward(mode, context, edge_weights, dcost, msg_min_index, msg_norm_ind
   dctx = (dcost.new_zeros(L, L) if L == 21 else dcost.new_zeros(L)) if want_dctx else \
       dcost.new_empty(0)
   if mode == "TRWP":
-    op = lib_stereo.TRWP_hard_soft if hard_soft else lib_stereo.TRWP
+    op = ops.TRWP_hard_soft if hard_soft else ops.TRWP
     op.backward(rho, context, edge_weights, dcost, imin, inorm, dunary, dctx, dedge, dmsg,
-                dunary_update, flags=flags)
+                dunary_update, **kw)
   else:
     dmsg_update = make(n_dir, b, cv, h, w, L)
-    lib_stereo.ISGMR.backward(int(enable_sgm), rho, context, edge_weights, dcost, imin, inorm,
-                              dunary, dctx, dedge, dmsg, dunary_update, dmsg_update, flags=flags)
+    ops.ISGMR.backward(int(enable_sgm), rho, context, edge_weights, dcost, imin, inorm,
+                       dunary, dctx, dedge, dmsg, dunary_update, dmsg_update, **kw)
   torch.cuda.synchronize()
   return (dunary.cpu().numpy(), dctx.cpu().numpy() if want_dctx else None,
           dedge.cpu().numpy() if want_dedge else None)
