@@ -110,7 +110,8 @@ int mpl_isgmr_backward(const mpl_shape* shape, unsigned flags, int enable_sgm, f
 
 /* Soft-weighted TRWP: replaces lib_*.TRWP_hard_soft.forward_soft, MPLayers/TRWP_hard_soft/TRWP.cpp:
  * 313-349 (ForwardSoft) -> TRWP_forward_soft.cu:378-559.  The min over front labels becomes the
- * expectation of the dual under softmin weights.  n_disp <= 64.
+ * expectation of the dual under softmin weights.  n_disp <= MPL_MAX_LABELS as for the reference's
+ * stereo build (TRWP.cpp:336-340); 2-D context tables up to 64 labels.
  *   msg_edge_label (n_iter, n_dir, B, H, W, L, L) fp32: every dual of every pixel, kept for the
  *   backward pass (even directions [fd][cd], odd ones [cd][fd]); blocks of chain-start pixels are
  *   not written.  NULL together with msg_norm_index => inference. */

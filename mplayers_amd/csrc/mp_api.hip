@@ -999,10 +999,6 @@ int mpl_trwp_soft_forward(const mpl_shape* s, unsigned flags, float rho, int n_i
   if (rc) return rc;
   CallOpts opts;
   if ((rc = read_flags(flags, "trwp_soft_forward", &opts)) != MPL_OK) return rc;
-  if (s->n_disp > kWave)
-    return fail(MPL_EINVAL, "trwp_soft_forward: at most %d labels (one per lane; the stored "
-                "duals take n_disp^2 floats per pixel, direction and iteration), got %d", kWave,
-                s->n_disp);
   if (!unary || !context || !edge_weights || !msg || !cost_final || !unary_update)
     return fail(MPL_EINVAL, "trwp_soft_forward: null tensor pointer");
   if ((msg_edge_label == nullptr) != (msg_norm_index == nullptr))
@@ -1057,8 +1053,6 @@ int mpl_trwp_soft_backward(const mpl_shape* s, unsigned flags, float rho, int n_
   if (rc) return rc;
   CallOpts opts;
   if ((rc = read_flags(flags, "trwp_soft_backward", &opts)) != MPL_OK) return rc;
-  if (s->n_disp > kWave)
-    return fail(MPL_EINVAL, "trwp_soft_backward: at most %d labels, got %d", kWave, s->n_disp);
   if (!context || !edge_weights || !dcost_final || !msg_edge_label || !msg_norm_index || !dunary ||
       !dmsg)
     return fail(MPL_EINVAL, "trwp_soft_backward: null tensor pointer");

@@ -11,8 +11,8 @@
 //     ddual[cd, fd] = g[cd] * prob * (1 - dual + soft[cd])
 //     dU[q, fd] += sum_cd ddual;  dedge[p] += sum ctx * ddual;  dcontext[ctx index] += w[p] * ddual
 //
-// Mapping: one wavefront per chain, one label per lane (L <= 64), pixel planes prefetched through a
-// register ring as in the hard kernels.  The (L, L) block goes through LDS so that global memory
+// Mapping (up to 64 labels; the kernels for more are further down): one wavefront per chain, one
+// label per lane, pixel planes prefetched through a register ring as in the hard kernels.  The (L, L) block goes through LDS so that global memory
 // sees it as T = ceil(L*L/64) coalesced dword accesses per lane; T is a template bucket so that the
 // number of memory instructions per step is a compile-time constant.
 
@@ -410,6 +410,389 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// More than 64 labels (up to 256, the label count the reference's stereo build accepts for
+// ForwardSoft, TRWP_hard_soft/TRWP.cpp:336-340): R = ceil(L / 64) labels per lane, lane i owning
+// labels i, i + 64, ...  A pixel's block of duals (L * L floats, up to 256 KB) does not fit in LDS,
+// so it moves through a tile of kFc front labels at a time, tile[cd * kTs + fc], with an odd row
+// stride: a lane reads and writes the row of its own label without bank conflicts, and the wave
+// moves the tile to and from global memory in runs of kFc consecutive floats whatever the stored
+// layout is (even directions [fd][cd], odd ones [cd][fd]).  1-D contexts only (2-D tables exist
+// for at most 64 labels).  A step costs L * L exponentials, which dwarfs the latency of its loads:
+// no prefetch ring here, the loads of a pixel are issued where they are needed.
+// ------------------------------------------------------------------------------------------------
+constexpr int kFc = 32;        // front labels per chunk of the tile
+constexpr int kTs = kFc + 1;   // row stride of the tile (odd: conflict-free rows and columns)
+
+// largest label among the lanes' labels (lane + 64 * j) whose predicate is set; dflt when none is
+template <int R>
+__device__ __forceinline__ int last_label_strided(const bool (&pred)[R], int dflt) {
+  int best = dflt;
+  bool found = false;
+#pragma unroll
+  for (int j = R - 1; j >= 0; --j) {
+    const uint64_t m = ballot(pred[j]);
+    if (!found && m != 0) {
+      best = kWave * j + 63 - __builtin_clzll(m);
+      found = true;
+    }
+  }
+  return best;
+}
+
+// tile[cd * kTs + fc] <-> block entry (cd, fd = f0 + fc), nf = number of front labels in the chunk
+template <int R>
+__device__ __forceinline__ void tile_from_global(const float* __restrict__ blk, bool even, int L,
+                                                 int f0, int nf, int lane, float* tile) {
+  if (even) {  // stored [fd][cd]: consecutive lanes, consecutive labels
+    for (int fc = 0; fc < nf; ++fc) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        const int cd = lane + kWave * j;
+        if (cd < L) tile[cd * kTs + fc] = __builtin_nontemporal_load(blk + (int64_t)(f0 + fc) * L + cd);
+      }
+    }
+  } else {     // stored [cd][fd]: two rows of kFc front labels per wave access
+    const int col = lane & (kFc - 1), sub = lane >> 5;
+    for (int r0 = 0; r0 < L; r0 += 2) {
+      const int row = r0 + sub;
+      if (row < L && col < nf) tile[row * kTs + col] = __builtin_nontemporal_load(blk + (int64_t)row * L + f0 + col);
+    }
+  }
+}
+
+template <int R>
+__device__ __forceinline__ void tile_to_global_rows(float* __restrict__ blk, int L, int f0, int nf,
+                                                    int lane, const float* tile) {
+  const int col = lane & (kFc - 1), sub = lane >> 5;
+  for (int r0 = 0; r0 < L; r0 += 2) {
+    const int row = r0 + sub;
+    if (row < L && col < nf) __builtin_nontemporal_store(tile[row * kTs + col], blk + (int64_t)row * L + f0 + col);
+  }
+}
+
+template <int R, bool TRAIN>
+__global__ void __launch_bounds__(kWave) soft_wide_fwd_kernel(const SweepParams p) {
+  extern __shared__ float smem[];
+  const int L = p.L;
+  float* a_s = smem;              // kMaxL
+  float* ctx_s = a_s + kMaxL;     // kMaxL
+  float* tile = ctx_s + kMaxL;    // L * kTs (training, odd directions)
+  const int lane = threadIdx.x;
+  const ChainCtx ch = locate_chain(p);
+  if (ch.n < 2) return;  // nothing to write
+  for (int i = lane; i < L; i += kWave) ctx_s[i] = p.ctx[i];
+  __syncthreads();
+
+  const int64_t HW = (int64_t)p.H * p.W;
+  const int64_t P = (int64_t)p.B * HW;
+  const int64_t N = P * L;
+  const int dir = ch.dir;
+  const bool even = (dir & 1) == 0;
+  const int64_t img_p = (int64_t)ch.bv * HW;
+  const float* __restrict__ bS = p.belief + img_p * L;
+  const float* __restrict__ bMd = p.msg_in + (int64_t)dir * N + img_p * L;
+  const float* __restrict__ bMi = p.msg_in + (int64_t)(dir ^ 1) * N + img_p * L;
+  float* __restrict__ bMo = p.msg_out + (int64_t)dir * N + img_p * L;
+  float* __restrict__ bSo = p.belief_out + img_p * L;
+  const float* __restrict__ bW = p.edge + (int64_t)dir * P + img_p;
+  float* __restrict__ bBlk = TRAIN ? p.edge_label + ((int64_t)dir * P + img_p) * L * L : nullptr;
+  uint8_t* __restrict__ bInorm = TRAIN ? p.idx_norm + (int64_t)dir * P + img_p : nullptr;
+  const float rho = p.rho;
+  const float inf = INFINITY;
+
+  int cd[R], cdc[R];
+  bool valid[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    cd[j] = lane + kWave * j;
+    valid[j] = cd[j] < L;
+    cdc[j] = valid[j] ? cd[j] : L - 1;  // keeps the table reads of idle lanes in range
+  }
+
+  float prev[R], uf[R];
+  {
+    const int64_t e0 = (int64_t)ch.pix0 * L;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      prev[j] = 0.f;
+      uf[j] = inf;
+      if (valid[j]) uf[j] = fmaf(bS[e0 + cd[j]] - bMd[e0 + cd[j]], rho, -bMi[e0 + cd[j]]);
+    }
+  }
+  for (int t = 1; t < ch.n; ++t) {
+    const int pix = ch.pix0 + t * ch.pstep;
+    const int64_t e = (int64_t)pix * L;
+    const float w = uniform_f(bW[pix]);
+    float tt[R], un[R], a[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      tt[j] = 0.f;
+      un[j] = inf;
+      if (valid[j]) {
+        const float mi = bMi[e + cd[j]];
+        tt[j] = bS[e + cd[j]] - bMd[e + cd[j]];
+        un[j] = fmaf(tt[j], rho, -mi);  // UpdateUnaryKernelSoft, TRWP_forward_soft.cu:161-181
+      }
+      a[j] = fmaf(rho, prev[j], uf[j]);
+      if (valid[j]) a_s[cd[j]] = a[j];
+    }
+    __syncthreads();
+    // pass 1: minimum of the duals of each of the lane's labels (TRWP_forward_soft.cu:69-80)
+    float mn[R], se[R], sd[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      mn[j] = inf;
+      se[j] = sd[j] = 0.f;
+    }
+#pragma unroll 2
+    for (int fd = 0; fd < L; ++fd) {
+      const float af = a_s[fd];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        const int k = cdc[j] - fd;
+        mn[j] = fminf(mn[j], fmaf(w, ctx_s[k < 0 ? -k : k], af));
+      }
+    }
+    // pass 2: softmin weights and the expected dual (:81-97); the block leaves chunk by chunk
+    float* blk = TRAIN ? bBlk + (int64_t)pix * L * L : nullptr;
+    for (int f0 = 0; f0 < L; f0 += kFc) {
+      const int nf = L - f0 < kFc ? L - f0 : kFc;
+      for (int fc = 0; fc < nf; ++fc) {
+        const int fd = f0 + fc;
+        const float af = a_s[fd];
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const int k = cdc[j] - fd;
+          const float dual = fmaf(w, ctx_s[k < 0 ? -k : k], af);
+          const float ex = fast_exp(mn[j] - dual);
+          se[j] += ex;
+          sd[j] = fmaf(ex, dual, sd[j]);
+          if (TRAIN && valid[j]) {
+            if (even)
+              __builtin_nontemporal_store(dual, blk + (int64_t)fd * L + cd[j]);  // [fd][cd]
+            else
+              tile[cd[j] * kTs + fc] = dual;
+          }
+        }
+      }
+      if (TRAIN && !even) {  // [cd][fd]: rows of the chunk, kFc consecutive floats each
+        __syncthreads();
+        tile_to_global_rows<R>(blk, L, f0, nf, lane, tile);
+        __syncthreads();
+      }
+    }
+    float soft[R], lo = inf;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      soft[j] = sd[j] / se[j];
+      lo = fminf(lo, valid[j] ? soft[j] : inf);
+    }
+    const float nmin = wave_min(lo);
+    bool pr[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const float m = soft[j] - nmin;
+      pr[j] = valid[j] && (soft[j] == nmin);
+      if (valid[j]) {
+        __builtin_nontemporal_store(m, bMo + e + cd[j]);
+        __builtin_nontemporal_store(tt[j] + m, bSo + e + cd[j]);
+      }
+      prev[j] = valid[j] ? m : 0.f;
+      uf[j] = un[j];
+    }
+    if (TRAIN) {
+      const int nidx = last_label_strided<R>(pr, L - 1);  // largest label on ties
+      if (lane == 0) bInorm[pix] = (uint8_t)nidx;
+    }
+    __syncthreads();  // a_s is rewritten by the next step
+  }
+}
+
+template <int R>
+__global__ void __launch_bounds__(kWave) soft_wide_bwd_kernel(const BackParams p) {
+  extern __shared__ float smem[];
+  const int L = p.L;
+  float* ctx_s = smem;           // kMaxL
+  float* tile = ctx_s + kMaxL;   // L * kTs
+  const int lane = threadIdx.x;
+  const int64_t HW = (int64_t)p.H * p.W;
+  const int64_t P = (int64_t)p.B * HW;
+  const int64_t N = P * L;
+  const ChainCtx ch = locate_chain(p);
+  const int dir = ch.dir;
+  const bool even = (dir & 1) == 0;
+  const int n = ch.n;
+  for (int i = lane; i < L; i += kWave) ctx_s[i] = p.ctx[i];
+  __syncthreads();
+
+  const int64_t img_p = (int64_t)ch.bv * HW;
+  const bool read_h = !p.first_touch;
+  const float* __restrict__ bA = p.a_in + img_p * L;
+  float* __restrict__ bAo = p.a_out + img_p * L;
+  float* __restrict__ bHd = p.h + (int64_t)dir * N + img_p * L;
+  float* __restrict__ bHi = p.h + (int64_t)(dir ^ 1) * N + img_p * L;
+  const float* __restrict__ bBlk = p.edge_label + ((int64_t)dir * P + img_p) * L * L;
+  const uint8_t* __restrict__ bInorm = p.idx_norm + (int64_t)dir * P + img_p;
+  const float* __restrict__ bW = p.edge + (int64_t)dir * P + img_p;
+  float* __restrict__ bDe = p.dedge != nullptr ? p.dedge + (int64_t)dir * P + img_p : nullptr;
+  const float rho = p.rho;
+  const float inf = INFINITY;
+
+  int cd[R], cdc[R];
+  bool valid[R];
+  float sc[R], hist[R];  // dU of the current pixel; dcontext bins lane + 64 * j
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    cd[j] = lane + kWave * j;
+    valid[j] = cd[j] < L;
+    cdc[j] = valid[j] ? cd[j] : L - 1;
+    sc[j] = hist[j] = 0.f;
+  }
+  const int col = lane & (kFc - 1), sub = lane >> 5;
+
+  for (int t = n - 1; t >= 0; --t) {
+    const int pix = ch.pix0 + t * ch.pstep;
+    const int64_t e = (int64_t)pix * L;
+    float a[R], hd[R], hi[R], scn[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      a[j] = hd[j] = hi[j] = scn[j] = 0.f;
+      if (valid[j]) {
+        a[j] = bA[e + cd[j]];
+        if (read_h) {
+          hd[j] = bHd[e + cd[j]];
+          hi[j] = bHi[e + cd[j]];
+        }
+      }
+    }
+    float det = 0.f;
+    if (t >= 1) {  // the chain start (t == 0) has no incoming edge
+      const float w = uniform_f(bW[pix]);
+      const int nidx = uniform_i((int)bInorm[pix]);
+      float g[R], part = 0.f;
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        g[j] = valid[j] ? fmaf(rho, sc[j], a[j] + hd[j]) : 0.f;
+        part += g[j];
+      }
+      const float tot = wave_sum(part);  // back norm, TRWP_backward_soft.cu:52-63
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+        if (cd[j] == nidx) g[j] -= tot;
+      const float* blk = bBlk + (int64_t)pix * L * L;
+      // pass A: softmin statistics of each of the lane's labels (:83-105), chunk by chunk with a
+      // running minimum (the sums are rescaled when a chunk lowers it)
+      float mn[R], se[R], sd[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        mn[j] = inf;
+        se[j] = sd[j] = 0.f;
+      }
+      for (int f0 = 0; f0 < L; f0 += kFc) {
+        const int nf = L - f0 < kFc ? L - f0 : kFc;
+        tile_from_global<R>(blk, even, L, f0, nf, lane, tile);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const float* row = tile + cdc[j] * kTs;
+          float cm = inf;
+          for (int fc = 0; fc < nf; ++fc) cm = fminf(cm, row[fc]);
+          const float mnew = fminf(mn[j], cm);
+          const float scale = fast_exp(mnew - mn[j]);  // 0 for the first chunk (mn = +inf)
+          float s1 = se[j] * scale, s2 = sd[j] * scale;
+          for (int fc = 0; fc < nf; ++fc) {
+            const float x = row[fc];
+            const float ex = fast_exp(mnew - x);
+            s1 += ex;
+            s2 = fmaf(ex, x, s2);
+          }
+          se[j] = s1;
+          sd[j] = s2;
+          mn[j] = mnew;
+        }
+        __syncthreads();
+      }
+      float gs[R], soft1[R], de = 0.f;
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        const float inv = 1.f / se[j];
+        soft1[j] = fmaf(sd[j], inv, 1.f);
+        gs[j] = g[j] * inv;
+      }
+      // pass B: ddual = g * prob * (1 - dual + soft) (:110-113) replaces the duals in the tile;
+      // its column sums are dU[q, fd], its diagonal sums the dcontext bins
+#pragma unroll
+      for (int jc = 0; jc < R; ++jc) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int f0 = kWave * jc + kFc * half;
+          if (f0 < L) {  // wave-uniform
+            const int nf = L - f0 < kFc ? L - f0 : kFc;
+            tile_from_global<R>(blk, even, L, f0, nf, lane, tile);
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+              if (valid[j]) {
+                float* row = tile + cd[j] * kTs;
+                for (int fc = 0; fc < nf; ++fc) {
+                  const float x = row[fc];
+                  const float dd = gs[j] * fast_exp(mn[j] - x) * (soft1[j] - x);
+                  const int k = cd[j] - (f0 + fc);
+                  de = fmaf(ctx_s[k < 0 ? -k : k], dd, de);
+                  row[fc] = dd;
+                }
+              }
+            }
+            __syncthreads();
+            // dU[q, f0 + col]: every lane adds up half of the rows of its column
+            float cs = 0.f;
+            if (col < nf)
+              for (int r = sub; r < L; r += 2) cs += tile[r * kTs + col];
+            cs += __shfl_xor(cs, 32);
+            if (sub == half) scn[jc] += cs;  // label f0 + col = lane + 64 * jc
+            // dcontext[k] += w * ddual over |cd - fd| == k (the pairs with k == 0 included,
+            // TRWP_backward_soft.cu:116-126): lane + 64 * j owns bin k
+            if (p.dctx != nullptr) {
+#pragma unroll
+              for (int j = 0; j < R; ++j) {
+                const int k = cd[j];
+                if (k < L) {
+                  float acc = 0.f;
+                  for (int fc = 0; fc < nf; ++fc) {
+                    const int fd = f0 + fc;
+                    if (fd + k < L) acc += tile[(fd + k) * kTs + fc];
+                    if (k > 0 && fd - k >= 0) acc += tile[(fd - k) * kTs + fc];
+                  }
+                  hist[j] = fmaf(w, acc, hist[j]);
+                }
+              }
+            }
+            __syncthreads();
+          }
+        }
+      }
+      det = wave_sum(de);
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      if (valid[j]) {
+        const float an = fmaf(rho, sc[j], a[j]);  // g_k += rho*dU for every k, dunary too
+        bAo[e + cd[j]] = an;
+        bHd[e + cd[j]] = -an;             // g_dir = 0 after its sweep
+        bHi[e + cd[j]] = hi[j] - sc[j];   // g_inv -= dU
+      }
+      sc[j] = scn[j];
+    }
+    if (t >= 1 && bDe != nullptr && lane == 0) bDe[pix] += det;
+  }
+  if (p.dctx != nullptr) {
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+      if (valid[j] && hist[j] != 0.f) atomicAdd(&p.dctx[cd[j]], hist[j]);
+  }
+}
+
 // Stand-alone softmin of stored blocks (SoftWeightedMessageKernel / ...BackKernel,
 // TRWP_hard_soft/TRWP_swbp.cu:131-254): message (n_trees, L, L) laid out [fd][cd];
 //   out[tree, cd] = sum_fd prob * message - min_cd(...),  prob = softmax_fd(-message[:, cd])
@@ -510,6 +893,25 @@ int tile_bucket(int L) {
 void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
   if (blocks <= 0) return;
+  if (p.L > kWave) {  // several labels per lane
+    const size_t wide_lds = sizeof(float) * (2 * kMaxL + (train ? p.L * kTs : 0));
+    const int R = (p.L + kWave - 1) / kWave;
+#define MPL_SOFT_WIDE_FWD(RR)                                                       \
+  do {                                                                              \
+    if (train)                                                                      \
+      soft_wide_fwd_kernel<RR, true><<<blocks, kWave, wide_lds, st>>>(p);           \
+    else                                                                            \
+      soft_wide_fwd_kernel<RR, false><<<blocks, kWave, wide_lds, st>>>(p);          \
+  } while (0)
+    if (R == 2)
+      MPL_SOFT_WIDE_FWD(2);
+    else if (R == 3)
+      MPL_SOFT_WIDE_FWD(3);
+    else
+      MPL_SOFT_WIDE_FWD(4);
+#undef MPL_SOFT_WIDE_FWD
+    return;
+  }
   const int LL = p.L * p.L;
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (LL + (train ? (LL > kWave * T ? LL : kWave * T) : 0));
@@ -535,6 +937,17 @@ void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st) {
 void launch_soft_bwd(const BackParams& p, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
   if (blocks <= 0) return;
+  if (p.L > kWave) {  // several labels per lane
+    const size_t wide_lds = sizeof(float) * (kMaxL + p.L * kTs);
+    const int R = (p.L + kWave - 1) / kWave;
+    if (R == 2)
+      soft_wide_bwd_kernel<2><<<blocks, kWave, wide_lds, st>>>(p);
+    else if (R == 3)
+      soft_wide_bwd_kernel<3><<<blocks, kWave, wide_lds, st>>>(p);
+    else
+      soft_wide_bwd_kernel<4><<<blocks, kWave, wide_lds, st>>>(p);
+    return;
+  }
   const int LL = p.L * p.L;
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (2 * LL + kWave * T + p.L * (p.L | 1));

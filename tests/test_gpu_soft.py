@@ -21,6 +21,13 @@ CASES = [
     (4, 1, 1, 9, 8, "tl2", 2),
     (4, 1, 9, 1, 8, "tl2", 2),
     (2, 3, 3, 12, 3, "tl2", 3),
+    # more than 64 labels (the stereo build accepts up to 256, TRWP_hard_soft/TRWP.cpp:336-340):
+    # several labels per lane, the duals move through LDS in chunks of 32 front labels
+    (4, 1, 4, 5, 65, "tl3", 2),         # one label in the second register, one 1-label chunk
+    (4, 2, 3, 4, 96, "dense1d", 1),     # chunks end on a label boundary
+    (8, 1, 4, 4, 130, "tl3", 1),        # three labels per lane, diagonals too
+    (4, 1, 3, 3, 200, "dense1d", 2),    # four labels per lane, partial last chunk
+    (4, 1, 2, 3, 256, "tl3", 1),        # every lane holds four labels
 ]
 
 
@@ -264,12 +271,14 @@ def test_module_hard_mode_backward_collects_same_label_terms(gpu, oracle, L, n_d
   assert np.abs(full - dc).max() <= 1e-4 * max(1, np.abs(dc).max())
 
 
-def test_soft_refuses_more_than_64_labels(gpu):
+def test_soft_accepts_what_the_reference_accepts(gpu):
+  """Up to 256 labels (MAX_DISPARITY of the stereo build); beyond that the call is refused before
+  anything is launched (the reference prints a message and returns zero-filled outputs)."""
   import torch
   from mplayers_amd import lib_stereo
-  L = 65
+  L = 257
   u = torch.zeros(1, 1, 2, 2, L, device="cuda")
-  with pytest.raises(RuntimeError):
+  with pytest.raises(RuntimeError, match="n_disp"):
     lib_stereo.TRWP_hard_soft.forward_soft(
         0.5, 1, u, torch.zeros(L, device="cuda"), torch.ones(4, 1, 1, 2, 2, device="cuda"),
         torch.zeros(4, 1, 1, 2, 2, L, device="cuda"), torch.empty(0), torch.empty(0, dtype=torch.uint8),
