@@ -415,6 +415,11 @@ __global__ void __launch_bounds__(kWave) selftest_kernel(int* out) {
   for (int special = 0; special < 64; special += 9)  // the minimum sits in every row and bank
     if (wave_min(y + (lane == special ? -100.f : 0.f)) != (float)((special * 37 + 11) % 64) - 100.f)
       ok = 0;
+  if (wave_min_fast(y) != 0.f) ok = 0;
+  for (int special = 0; special < 64; special += 7)
+    if (wave_min_fast(y + (lane == special ? -100.f : 0.f)) != (float)((special * 37 + 11) % 64) - 100.f)
+      ok = 0;
+  if (wave_min_fast(lane < 21 ? (float)(30 - lane) : INFINITY) != 10.f) ok = 0;
   if (wave_sum((float)lane) != 2016.f) ok = 0;
   bool pr[2] = {lane == 5 || lane == 40, lane == 40};
   if (last_label<2>(pr, -1) != 81) ok = 0;
@@ -494,7 +499,7 @@ int check_shape(const mpl_shape* s, int n_iter) {
   int64_t P = (int64_t)s->batch * s->height * s->width;
   if (P > 0x7fffffff) return fail(MPL_EINVAL, "more than 2^31 pixels");
   // pixels are addressed with 32-bit byte offsets from the first pixel of their batch item
-  if ((int64_t)s->height * s->width * s->n_disp * 4 > 0xffffffffll)
+  if ((int64_t)s->height * s->width * s->n_disp * 4 > kMaxImageBytes)
     return fail(MPL_EINVAL, "one batch item (height*width*n_disp floats) must stay below 4 GiB");
   int64_t max_blocks = 0;
   for (int d = 0; d < s->n_dir; ++d)

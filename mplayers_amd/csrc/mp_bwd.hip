@@ -131,21 +131,53 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
   for (int j = 0; j < R; ++j) valid[j] = MASK ? (lab0 + j < L) : true;
 
+  // VEC: one descriptor per plane for the whole kernel, covering the batch item's image; a lane
+  // reaches its labels of a pixel through its vector offset, a lane without labels (or a step that
+  // must not store) through an offset no descriptor covers: one multiply, one add and one select
+  // per pixel instead of a descriptor formed per access.  Planes that are not to be read or stored
+  // get an empty descriptor.
+  const bool lane_ok = !MASK || lab0 < L;
+  const int img_bytes = (int)(unsigned)(HW * L * 4);
+  const rsrc_t rA = make_rsrc(bA, img_bytes);
+  const rsrc_t rAo = make_rsrc(bAo, img_bytes);
+  const rsrc_t rHdIn = make_rsrc(bHd, (!JACOBI && read_h) ? img_bytes : 0);
+  const rsrc_t rHiIn = make_rsrc(bHi, (!JACOBI && read_h && !inv_from_a) ? img_bytes : 0);
+  const rsrc_t rHdOut = make_rsrc(bHd, (JACOBI || p.skip_hd_store) ? 0 : img_bytes);
+  const rsrc_t rHiOut = make_rsrc(bHi, (JACOBI || p.skip_hi_store) ? 0 : img_bytes);
+  const rsrc_t rImin = make_rsrc(bImin, (int)(HW * L));
   // loads run from the last pixel of the chain down to the first; past it the first is refetched
+  // (VEC: the prefetch simply runs on; what lies there is another pixel or reads as 0)
   int ld_t = n - 1;
   int ld_p = ch.pix0 + (n - 1) * ch.pstep;
-  auto load_next = [&]() {
+  auto load_next = [&]() __attribute__((always_inline)) {
     PixB<R> r;
-    const unsigned pp = (unsigned)uniform_i(ld_t >= 0 ? ld_p : ch.pix0);
+    const unsigned pp = (unsigned)uniform_i((VEC || ld_t >= 0) ? ld_p : ch.pix0);
     const unsigned so = pp * (unsigned)vbytes;
-    const int nrec = (int)(so + (unsigned)vbytes);
-    buf_load<R, VEC>(make_rsrc(bA, nrec), foff, so, r.a);
+    if constexpr (VEC) {
+      const int vo = (int)(lane_ok ? so + (unsigned)foff : kDeadWide);
+      buf_load<R, true>(rA, vo, 0u, r.a);
+      if (!JACOBI) {
+        // before the first write of these planes they count as zero (empty descriptor); the sweep
+        // that ran just before this one was the opposite direction's and left h_inv = -A
+        buf_load<R, true>(rHdIn, vo, 0u, r.hd);
+        buf_load<R, true>(rHiIn, vo, 0u, r.hi);
+      }
+      buf_load_u8<R, true>(rImin, (int)(lane_ok ? pp * (unsigned)L + (unsigned)lab0 : kDeadWide), 0u,
+                           r.fd);
+    } else {
+      const int nrec = (int)(so + (unsigned)vbytes);
+      buf_load<R, VEC>(make_rsrc(bA, nrec), foff, so, r.a);
+      if (!JACOBI) {
+        // before the first write of these planes they count as zero: an empty descriptor reads 0
+        buf_load<R, VEC>(make_rsrc(bHd, read_h ? nrec : 0), foff, so, r.hd);
+        // the sweep that ran just before this one was the opposite direction's: it left
+        // h_inv = -A everywhere, so the plane need not be read (empty descriptor, no traffic)
+        buf_load<R, VEC>(make_rsrc(bHi, (read_h && !inv_from_a) ? nrec : 0), foff, so, r.hi);
+      }
+      buf_load_u8<R, VEC>(make_rsrc(bImin, (int)(pp * (unsigned)L + (unsigned)L)), lab0,
+                          pp * (unsigned)L, r.fd);
+    }
     if (!JACOBI) {
-      // before the first write of these planes they count as zero: an empty descriptor reads 0
-      buf_load<R, VEC>(make_rsrc(bHd, read_h ? nrec : 0), foff, so, r.hd);
-      // the sweep that ran just before this one was the opposite direction's: it left
-      // h_inv = -A everywhere, so the plane need not be read (empty descriptor, no traffic)
-      buf_load<R, VEC>(make_rsrc(bHi, (read_h && !inv_from_a) ? nrec : 0), foff, so, r.hi);
       if (inv_from_a) {
 #pragma unroll
         for (int j = 0; j < R; ++j) r.hi[j] = -r.a[j];
@@ -154,8 +186,6 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
       for (int j = 0; j < R; ++j) r.hd[j] = r.hi[j] = 0.f;
     }
-    buf_load_u8<R, VEC>(make_rsrc(bImin, (int)(pp * (unsigned)L + (unsigned)L)), lab0,
-                        pp * (unsigned)L, r.fd);
     r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, (int)pp, 0, 0);
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
     r.de = 0.f;
@@ -171,7 +201,9 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   constexpr int kOps = (JACOBI ? 1 : 3) * vec_ops(R, VEC) + byte_ops(R, VEC) + 2 + (DE ? 1 : 0) +
                        (JACOBI ? 1 : 3) * vec_ops(R, VEC) + (DE ? 1 : 0);
   constexpr int D = ring_depth(kOps);
-  PixB<R> ring[D];
+  // two banks of D pixels in flight, consumed in turn: after 2 D steps every value sits in the
+  // register it started in (a single bank ends the loop in one register move per value in flight)
+  PixB<R> ring[D], ring2[D];
 #pragma unroll
   for (int u = 0; u < D; ++u) ring[u] = load_next();
 
@@ -185,14 +217,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const int last_lane = (L - 1) / R, last_reg = (L - 1) % R;
 
   int st_p = ch.pix0 + (n - 1) * ch.pstep;
-  for (int s0 = 0; s0 < n; s0 += D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      const int t = n - 1 - (s0 + u);
-      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
-      wait_vmem<(D - 1) * kOps>();
-      const PixB<R> px = ring[u];
-      ring[u] = load_next();
+  auto step = [&](const PixB<R>& px, const int t) __attribute__((always_inline)) {
       float scn[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) scn[j] = 0.f;
@@ -362,8 +387,12 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
       const unsigned sp = (unsigned)uniform_i(st_p);
       const unsigned so = sp * (unsigned)vbytes;
       const int nrec = t >= 0 ? (int)(so + (unsigned)vbytes) : 0;
+      const int vo = (int)((lane_ok && t >= 0) ? so + (unsigned)foff : kDeadWide);
       if (JACOBI) {
-        buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, sc);
+        if constexpr (VEC)
+          buf_store<R, true>(rAo, vo, 0u, sc);
+        else
+          buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, sc);
       } else {
         float an[R], hdn[R], hin[R];
 #pragma unroll
@@ -372,12 +401,18 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           hdn[j] = -an[j];                    // g_dir = 0 after its sweep
           hin[j] = px.hi[j] - sc[j];          // g_inv -= dU
         }
-        buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, an);
         // h_dir = -A is only read by the next launch when that one sweeps the opposite
         // direction, which derives it from A instead: nothing is stored then (nor after the last
         // sweeps of the pass, whose h planes nobody reads)
-        buf_store<R, VEC>(make_rsrc(bHd, p.skip_hd_store ? 0 : nrec), foff, so, hdn);
-        buf_store<R, VEC>(make_rsrc(bHi, p.skip_hi_store ? 0 : nrec), foff, so, hin);
+        if constexpr (VEC) {
+          buf_store<R, true>(rAo, vo, 0u, an);
+          buf_store<R, true>(rHdOut, vo, 0u, hdn);
+          buf_store<R, true>(rHiOut, vo, 0u, hin);
+        } else {
+          buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, an);
+          buf_store<R, VEC>(make_rsrc(bHd, p.skip_hd_store ? 0 : nrec), foff, so, hdn);
+          buf_store<R, VEC>(make_rsrc(bHi, p.skip_hi_store ? 0 : nrec), foff, so, hin);
+        }
       }
       // each pixel receives over exactly one edge per direction: plain read-modify-write
       if (DE)
@@ -386,6 +421,23 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 #pragma unroll
       for (int j = 0; j < R; ++j) sc[j] = scn[j];
       st_p -= ch.pstep;
+  };
+  for (int s0 = 0; s0 < n; s0 += 2 * D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
+      const PixB<R> px = ring[u];
+      ring2[u] = load_next();
+      step(px, n - 1 - (s0 + u));
+    }
+    if (s0 + D >= n) break;  // wave-uniform
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      wait_vmem<(D - 1) * kOps>();
+      const PixB<R> px = ring2[u];
+      ring[u] = load_next();
+      step(px, n - 1 - (s0 + D + u));
     }
   }
   if (!DC) return;

@@ -124,6 +124,25 @@ __device__ __forceinline__ float wave_min_f32(float x) {
   return readlane_f(x, 63);
 }
 
+// The float minimum with each lane shift folded into the min instruction, which the compiler does
+// not emit by itself: v_min_f32 with a DPP source, in place, so that a lane without a source keeps
+// its own value.  No conversions to integer keys and back: 6 instructions and the read-out.  (A
+// DPP operand written by the instruction before needs two wait states, which the compiler cannot
+// see inside the statement: each one carries its own.)
+__device__ __forceinline__ float wave_min_fast(float x) {
+#define MPL_MIN_DPP(CTRL) \
+  asm("s_nop 1\n\tv_min_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf" : "+v"(x))
+  MPL_MIN_DPP("row_shr:1 row_mask:0xf");
+  MPL_MIN_DPP("row_shr:2 row_mask:0xf");
+  MPL_MIN_DPP("row_shr:4 row_mask:0xf");
+  MPL_MIN_DPP("row_shr:8 row_mask:0xf");
+  MPL_MIN_DPP("row_bcast:15 row_mask:0xa");
+  MPL_MIN_DPP("row_bcast:31 row_mask:0xc");
+#undef MPL_MIN_DPP
+  asm("s_nop 1" : "+v"(x));
+  return readlane_f(x, 63);
+}
+
 // sum over the 64 lanes, returned wave-uniform
 __device__ __forceinline__ float wave_sum(float x) {
   x += dpp_f<0x111>(0.f, x);
@@ -231,6 +250,9 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, int bytes) {
 #endif
 
 constexpr int kDeadOffset = 0x7ffffff0;  // a vector offset no descriptor covers: access suppressed
+// the same for descriptors that cover a whole image (up to kMaxImageBytes, beyond 2 GiB)
+constexpr unsigned kDeadWide = 0xfffffff0u;
+constexpr int64_t kMaxImageBytes = 0xffffffc0ll;
 
 // R consecutive floats at vector byte offset `off` (range-checked) + scalar byte offset `so`.
 // VEC: one R-dword access (used when every lane's block lies entirely inside or entirely outside

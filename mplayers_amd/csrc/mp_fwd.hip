@@ -386,24 +386,54 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // (at a chain start, where no message is written, the plane is converted with the old values)
   const bool pair_first = !JACOBI && p.pair_q && (dir & 1) == 0;
   const bool pair_second = !JACOBI && p.pair_q && (dir & 1) == 1;
+  // VEC: one descriptor per plane for the whole kernel, covering the batch item's image; a lane
+  // reaches its labels of a pixel through its vector offset, and a lane without labels (or a step
+  // that must not store) through an offset no descriptor covers.  Nothing but one multiply, one
+  // add and one select per pixel is then spent on addressing (descriptors formed per access cost
+  // some eight scalar instructions each, which a chain-starved launch -- one wavefront per SIMD,
+  // every instruction an issue slot of its own -- cannot hide).  Planes that are not to be read
+  // (all-zero initial messages, the odd sweep's own old messages) or stored get an empty descriptor.
+  const bool lane_ok = !MASK || lab0 < L;
+  const int img_bytes = (int)(unsigned)(HW * L * 4);
+  const rsrc_t rS = make_rsrc(bS, img_bytes);
+  const rsrc_t rMd0 = make_rsrc(bMd, md_zero ? 0 : img_bytes);  // chain start
+  const rsrc_t rMd = make_rsrc(bMd, (md_zero || pair_second) ? 0 : img_bytes);
+  const rsrc_t rMi = make_rsrc(bMi, mi_zero ? 0 : img_bytes);
+  const rsrc_t rMo = make_rsrc(bMo, img_bytes);
+  const rsrc_t rSo = make_rsrc(bSo, (JACOBI || p.skip_s_store) ? 0 : img_bytes);
+  const rsrc_t rImin = make_rsrc(bImin, TRAIN ? (int)(HW * L) : 0);
   // loads of the next pixel; past the end of the chain the last pixel is fetched again
   const int last_p = ch.pix0 + (n - 1) * ch.pstep;
   int ld_p = ch.pix0;
   int ld_t = 0;
-  auto load_next = [&]() {
+  auto load_next = [&](const bool first = false) __attribute__((always_inline)) {
     PixF<R> r;
-    const unsigned pp = (unsigned)uniform_i(ld_t < n ? ld_p : last_p);
+    // VEC: the prefetch simply runs on past the end of the chain: what lies there is another pixel
+    // of the image or outside the descriptors (reads as 0), and no step uses it
+    const unsigned pp = (unsigned)uniform_i((VEC || ld_t < n) ? ld_p : last_p);
     const unsigned so = pp * (unsigned)vbytes;
-    const int nrec = (int)(so + (unsigned)vbytes);
-    buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
-    if (JACOBI == 0) {
-      // planes that still hold all-zero initial messages are read through an empty descriptor
-      buf_load<R, VEC>(make_rsrc(bMd, (md_zero || (pair_second && ld_t > 0)) ? 0 : nrec), foff, so,
-                       r.md);
-      buf_load<R, VEC>(make_rsrc(bMi, mi_zero ? 0 : nrec), foff, so, r.mi);
-    } else if (JACOBI == 2) {
-      buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
-      buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
+    if constexpr (VEC) {
+      const int vo = (int)(lane_ok ? so + (unsigned)foff : kDeadWide);
+      buf_load<R, true>(rS, vo, 0u, r.s);
+      if (JACOBI == 0) {
+        buf_load<R, true>(first ? rMd0 : rMd, vo, 0u, r.md);
+        buf_load<R, true>(rMi, vo, 0u, r.mi);
+      } else if (JACOBI == 2) {
+        buf_load<R, true>(rMd0, vo, 0u, r.md);
+        buf_load<R, true>(rMi, vo, 0u, r.mi);
+      }
+    } else {
+      const int nrec = (int)(so + (unsigned)vbytes);
+      buf_load<R, VEC>(make_rsrc(bS, nrec), foff, so, r.s);
+      if (JACOBI == 0) {
+        // planes that still hold all-zero initial messages are read through an empty descriptor
+        buf_load<R, VEC>(make_rsrc(bMd, (md_zero || (pair_second && ld_t > 0)) ? 0 : nrec), foff, so,
+                         r.md);
+        buf_load<R, VEC>(make_rsrc(bMi, mi_zero ? 0 : nrec), foff, so, r.mi);
+      } else if (JACOBI == 2) {
+        buf_load<R, VEC>(make_rsrc(bMd, nrec), foff, so, r.md);
+        buf_load<R, VEC>(make_rsrc(bMi, nrec), foff, so, r.mi);
+      }
     }
     r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
     ld_p += ch.pstep;
@@ -415,7 +445,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // buffers alternate, so there the start pixel is written with the zeros it keeps in the reference.
   float prev[R], uf[R];
   {
-    const PixF<R> p0 = load_next();
+    const PixF<R> p0 = load_next(true);
     float conv[R];  // the start pixel's belief-plane value in the other representation
 #pragma unroll
     for (int j = 0; j < R; ++j) conv[j] = 0.f;
@@ -430,16 +460,22 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       }
       uf[j] = valid[j] ? un : inf;
     }
+    const unsigned so0 = (unsigned)ch.pix0 * (unsigned)vbytes;
+    const int vo0 = (int)(lane_ok ? so0 + (unsigned)foff : kDeadWide);
     if (!JACOBI && p.pair_q && !p.skip_s_store) {
-      const unsigned so = (unsigned)ch.pix0 * (unsigned)vbytes;
-      buf_store<R, VEC>(make_rsrc(bSo, (int)(so + (unsigned)vbytes)), foff, so, conv);
+      if constexpr (VEC)
+        buf_store<R, true>(rSo, vo0, 0u, conv);
+      else
+        buf_store<R, VEC>(make_rsrc(bSo, (int)(so0 + (unsigned)vbytes)), foff, so0, conv);
     }
     if (JACOBI || p.zero_start) {
       float z[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) z[j] = 0.f;
-      const unsigned so = (unsigned)ch.pix0 * (unsigned)vbytes;
-      buf_store<R, VEC>(make_rsrc(bMo, (int)(so + (unsigned)vbytes)), foff, so, z);
+      if constexpr (VEC)
+        buf_store<R, true>(rMo, vo0, 0u, z);
+      else
+        buf_store<R, VEC>(make_rsrc(bMo, (int)(so0 + (unsigned)vbytes)), foff, so0, z);
     }
   }
 
@@ -448,20 +484,16 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   constexpr int kOps = (JACOBI == 1 ? 1 : 3) * vec_ops(R, VEC) + 1 + (JACOBI ? 1 : 2) * vec_ops(R, VEC) +
                        (TRAIN ? byte_ops(R, VEC) + 1 : 0);
   constexpr int D = ring_depth(kOps);
-  PixF<R> ring[D];
+  // Two banks of D pixels in flight: while the steps consume one, the loads of D pixels ahead land
+  // in the other, so that after 2 D steps every value sits in the register it started in (with a
+  // single bank the loop ends in one register move per value in flight).
+  PixF<R> ring[D], ring2[D];
 #pragma unroll
   for (int u = 0; u < D; ++u) ring[u] = load_next();
 
   int st_p = ch.pix0 + ch.pstep;
-  for (int t0 = 1; t0 < n; t0 += D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      const int t = t0 + u;
+  auto step = [&](const PixF<R>& px, const int t) __attribute__((always_inline)) {
       const bool live = t < n;  // steps past the end compute on stale data and store nothing
-      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
-      wait_vmem<(D - 1) * kOps>();
-      const PixF<R> px = ring[u];
-      ring[u] = load_next();
       float tt[R], un[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) {
@@ -486,7 +518,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         float am = a[0];
 #pragma unroll
         for (int j = 1; j < R; ++j) am = fminf(am, a[j]);
-        const float amin = wave_min(am);
+        const float amin = wave_min_fast(am);
         int fstar = L - 1;
         if (TRAIN) {
           bool pr[R];
@@ -543,24 +575,33 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         float vm = inf;
 #pragma unroll
         for (int j = 0; j < R; ++j) vm = fminf(vm, valid[j] ? v[j] : inf);
-        nmin = (KT == -21) ? wave_min_f32(vm) : wave_min(vm);
+        nmin = wave_min_fast(vm);
       }
       float m[R], sn[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) {
         m[j] = v[j] - nmin;  // MsgNormNaive, commonCUDA.cuh:126-128
         sn[j] = pair_first ? tt[j] - px.mi[j] : tt[j] + m[j];
-        prev[j] = valid[j] ? m[j] : 0.f;
+        prev[j] = m[j];  // (a lane without a label keeps a = +inf through uf, whatever prev is)
         uf[j] = un[j];
       }
       const unsigned sp = (unsigned)uniform_i(st_p);
       const unsigned so = sp * (unsigned)vbytes;
-      const int nrec = live ? (int)(so + (unsigned)vbytes) : 0;  // nothing is stored past the end
-      buf_store<R, VEC>(make_rsrc(bMo, nrec), foff, so, m);
-      if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, p.skip_s_store ? 0 : nrec), foff, so, sn);
+      const unsigned sob = sp * (unsigned)L;
+      if constexpr (VEC) {
+        const bool on = lane_ok && live;  // nothing is stored past the end
+        const int vo = (int)(on ? so + (unsigned)foff : kDeadWide);
+        buf_store<R, true>(rMo, vo, 0u, m);
+        if (!JACOBI) buf_store<R, true>(rSo, vo, 0u, sn);
+        if (TRAIN) buf_store_u8<R, true>(rImin, (int)(on ? sob + (unsigned)lab0 : kDeadWide), 0u, fd_idx);
+      } else {
+        const int nrec = live ? (int)(so + (unsigned)vbytes) : 0;
+        buf_store<R, VEC>(make_rsrc(bMo, nrec), foff, so, m);
+        if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, p.skip_s_store ? 0 : nrec), foff, so, sn);
+        if (TRAIN)
+          buf_store_u8<R, VEC>(make_rsrc(bImin, live ? (int)(sob + (unsigned)L) : 0), lab0, sob, fd_idx);
+      }
       if (TRAIN) {
-        const unsigned sob = sp * (unsigned)L;
-        buf_store_u8<R, VEC>(make_rsrc(bImin, live ? (int)(sob + (unsigned)L) : 0), lab0, sob, fd_idx);
         bool pr[R];
 #pragma unroll
         for (int j = 0; j < R; ++j) pr[j] = valid[j] && (v[j] == nmin);
@@ -569,6 +610,23 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm, live ? (int)sp : kDeadOffset, 0, 0);
       }
       st_p += ch.pstep;
+  };
+  for (int t0 = 1; t0 < n; t0 += 2 * D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
+      const PixF<R> px = ring[u];
+      ring2[u] = load_next();
+      step(px, t0 + u);
+    }
+    if (t0 + D >= n) break;  // wave-uniform
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      wait_vmem<(D - 1) * kOps>();
+      const PixF<R> px = ring2[u];
+      ring[u] = load_next();
+      step(px, t0 + D + u);
     }
   }
 }
