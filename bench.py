@@ -60,8 +60,8 @@ def parse():
   ap.add_argument("--n-dir", type=int, default=None, choices=[2, 4, 8, 16],
                   help="run the configuration on another connectivity (not the headline workload)")
   ap.add_argument("--alg", default="both", choices=["both", "TRWP", "ISGMR", "SOFT"],
-                  help="SOFT: soft-weighted TRWP (at most 64 labels; stores n_disp^2 floats per "
-                       "pixel, direction and iteration)")
+                  help="SOFT: soft-weighted TRWP (stores n_disp^2 floats per pixel, direction and "
+                       "iteration)")
   ap.add_argument("--fwd-only", action="store_true", help="inference forward only (C2/C3 style)")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   ap.add_argument("--copy-probe", action="store_true",
@@ -71,6 +71,8 @@ def parse():
                   help="also time the library's copy probes on planes of the workload's size: one-pass "
                        "streaming kernels and scan-shaped kernels (one long-lived wavefront per row "
                        "or column) for several read:write mixes (\"measured_stream_rates\")")
+  ap.add_argument("--no-peak-probe", action="store_true",
+                  help="leave the copy probes out of the default large-configuration run (profiler runs)")
   ap.add_argument("--module-probe", action="store_true",
                   help="also time forward+backward through the nn.Module surface, which allocates "
                        "its buffers on every call as the reference's does (reported under "
@@ -463,7 +465,7 @@ def main():
     alt_ms = (time.perf_counter() - t0) / a.steps * 1e3
     out["msg_uninit" if not uninit else "caller_cleared_messages"] = {
         "ms_per_step": alt_ms, "steps": a.steps, "value": units_per_step / (alt_ms * 1e-3)}
-  if a.peak_probe or (cfg["name"] == "C5" and a.scale == 1.0):
+  if a.peak_probe or (cfg["name"] == "C5" and a.scale == 1.0 and not a.no_peak_probe):
     # what this GPU sustains for traffic of the kernels' shapes, next to the published 8 TB/s
     out["measured_stream_rates"] = peak_probe(H, W, L, dev, reps=5 if a.peak_probe else 2)
   if a.module_probe and training:
