@@ -411,6 +411,454 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// At most 32 labels: with one label per lane a third or less of the wavefront works, and the step
+// is L exponentials per lane deep.  Here the front labels of the chain's pixel are split over
+// G = 4 / 3 / 2 groups of lanes (L <= 16 / 21 / 32): lane g * L + cd carries label cd like its
+// G - 1 replicas in the other groups (they load the same values and keep the same recurrence
+// state) but only looks at the front labels g * F .. g * F + F - 1, F = ceil(L / G).  Each lane
+// forms the softmin statistics of its F duals around their own minimum; one exchange
+// (ds_bpermute: every lane fetches the G partial triples of its label and combines them in group
+// order, so the replicas stay bit-identical) rescales them to the minimum over all front labels.
+// The duals move between registers and memory directly, F dwords per lane at the lane's places of
+// the pixel's block; the lanes of group 0 store the label vectors.  FM: compile-time bound of F.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bperm_f(int addr, float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(int, x)));
+}
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+constexpr float kLog2e = 1.4426950408889634f;
+// exp(m - x) with m * kLog2e given: one multiply-add and the hardware's 2^x
+__device__ __forceinline__ float exp_below(float x, float m_log2e) {
+  return __builtin_amdgcn_exp2f(fmaf(x, -kLog2e, m_log2e));
+}
+
+// Reductions as chains of DPP-fused operations (a lane without a source lane keeps its value; a
+// DPP operand written by the instruction before needs two wait states, which the compiler cannot
+// see inside the statement).  NL = 16 / 32 / 64: over the first NL lanes only, the others are
+// ignored; the result is wave-uniform.
+#define MPL_RED_DPP(OP, CTRL) \
+  asm("s_nop 1\n\t" OP " %0, %0, %0 " CTRL " bank_mask:0xf" : "+v"(x))
+template <int NL>
+__device__ __forceinline__ float lanes_sum(float x) {
+  MPL_RED_DPP("v_add_f32_dpp", "row_shr:1 row_mask:0xf");
+  MPL_RED_DPP("v_add_f32_dpp", "row_shr:2 row_mask:0xf");
+  MPL_RED_DPP("v_add_f32_dpp", "row_shr:4 row_mask:0xf");
+  MPL_RED_DPP("v_add_f32_dpp", "row_shr:8 row_mask:0xf");
+  if (NL > 16) MPL_RED_DPP("v_add_f32_dpp", "row_bcast:15 row_mask:0xa");
+  if (NL > 32) MPL_RED_DPP("v_add_f32_dpp", "row_bcast:31 row_mask:0xc");
+  asm("s_nop 1" : "+v"(x));
+  return readlane_f(x, NL - 1);
+}
+template <int NL>
+__device__ __forceinline__ float lanes_min(float x) {
+  MPL_RED_DPP("v_min_f32_dpp", "row_shr:1 row_mask:0xf");
+  MPL_RED_DPP("v_min_f32_dpp", "row_shr:2 row_mask:0xf");
+  MPL_RED_DPP("v_min_f32_dpp", "row_shr:4 row_mask:0xf");
+  MPL_RED_DPP("v_min_f32_dpp", "row_shr:8 row_mask:0xf");
+  if (NL > 16) MPL_RED_DPP("v_min_f32_dpp", "row_bcast:15 row_mask:0xa");
+  if (NL > 32) MPL_RED_DPP("v_min_f32_dpp", "row_bcast:31 row_mask:0xc");
+  asm("s_nop 1" : "+v"(x));
+  return readlane_f(x, NL - 1);
+}
+#undef MPL_RED_DPP
+
+// (minimum, sum of weights, weighted sum of duals) of a label over all its front labels from the
+// per-lane partial triples, each taken around its own minimum.  `scale` returns the factor that
+// turns this lane's weights exp(mn_lane - dual) into exp(mn - dual).
+template <int G>
+__device__ __forceinline__ void group_softmin(const int (&addr)[G], float mn_l, float se_l,
+                                              float sd_l, float& mn, float& se, float& sd,
+                                              float& scale) {
+  float pm[G], ps[G], pd[G];
+#pragma unroll
+  for (int k = 0; k < G; ++k) {
+    pm[k] = bperm_f(addr[k], mn_l);
+    ps[k] = bperm_f(addr[k], se_l);
+    pd[k] = bperm_f(addr[k], sd_l);
+  }
+  mn = pm[0];
+#pragma unroll
+  for (int k = 1; k < G; ++k) mn = fminf(mn, pm[k]);
+  se = 0.f;
+  sd = 0.f;
+#pragma unroll
+  for (int k = 0; k < G; ++k) {
+    const float f = exp_below(pm[k], mn * kLog2e);  // (a group without front labels: 2^-inf = 0)
+    se = fmaf(f, ps[k], se);
+    sd = fmaf(f, pd[k], sd);
+  }
+  scale = exp_below(mn_l, mn * kLog2e);
+}
+
+template <int FM>
+struct PixSS {
+  float a, hd, hi, w, de;
+  int nidx;
+  float dual[FM];
+};
+
+// NT4: float4 stores per lane that cover the pixel's block of duals (256 * NT4 >= L * L)
+template <bool TRAIN, int G, int FM, int NT4>
+__global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams p) {
+  extern __shared__ float smem[];
+  const int L = p.L, LL = L * L;
+  float* tile = smem;              // 256 * NT4 floats (training): the pixel's block as it is stored
+  float* tab = smem + (TRAIN ? 256 * NT4 : 0);  // LL floats
+  const int lane = threadIdx.x;
+  const ChainCtx ch = locate_chain(p);
+  if (ch.n < 2) return;  // nothing to write
+  fill_table(p.ctx, L, p.ctx2d, lane, tab);
+  __syncthreads();
+
+  const int64_t HW = (int64_t)p.H * p.W;
+  const int64_t P = (int64_t)p.B * HW;
+  const int64_t N = P * L;
+  const int dir = ch.dir;
+  const int64_t img_p = (int64_t)ch.bv * HW;
+  const int64_t img_e = img_p * L;
+  const int vbytes = L * 4;
+  // one descriptor per plane over the batch item's image; a lane without work carries an offset
+  // that no descriptor covers
+  const int img_bytes = (int)(unsigned)(HW * L * 4);
+  const rsrc_t rS = make_rsrc(p.belief + img_e, img_bytes);
+  const rsrc_t rMd = make_rsrc(p.msg_in + (int64_t)dir * N + img_e, img_bytes);
+  const rsrc_t rMi = make_rsrc(p.msg_in + (int64_t)(dir ^ 1) * N + img_e, img_bytes);
+  const rsrc_t rMo = make_rsrc(p.msg_out + (int64_t)dir * N + img_e, img_bytes);
+  const rsrc_t rSo = make_rsrc(p.belief_out + img_e, img_bytes);
+  float* __restrict__ bBlk = TRAIN ? p.edge_label + ((int64_t)dir * P + img_p) * LL : nullptr;
+  const int img_bytes_p = (int)(HW * 4 > 0x7fffffff ? 0x7fffffff : HW * 4);
+  const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P + img_p, img_bytes_p);
+  const rsrc_t dInorm = make_rsrc(TRAIN ? p.idx_norm + (int64_t)dir * P + img_p : nullptr,
+                                  TRAIN ? (int)HW : 0);
+  const float rho = p.rho;
+  const float inf = INFINITY;
+  const int n = ch.n;
+  const int F = (L + G - 1) / G;
+  const bool valid = lane < G * L;
+  const int g = valid ? lane / L : 0;
+  const int cd = valid ? lane - g * L : 0;
+  const bool store_lane = lane < L;  // group 0
+  const unsigned foff = (unsigned)cd * 4u;
+  const bool even = (dir & 1) == 0;
+  int addr[G];
+#pragma unroll
+  for (int k = 0; k < G; ++k) addr[k] = (valid ? k * L + cd : lane) * 4;
+  // this lane's front labels fd0 + i; beyond the last label the entry repeats it with weight 0
+  const int fd0 = g * F;
+  float tcol[FM];
+  int src[FM], tidx[FM];
+  bool inr[FM];
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    inr[i] = valid && i < F && fd0 + i < L;
+    const int fd = inr[i] ? fd0 + i : L - 1;
+    tcol[i] = tab[fd * L + cd];  // ctx(cd, fd)
+    src[i] = fd * 4;             // a[fd] from group 0's replica
+    tidx[i] = even ? fd * L + cd : cd * L + fd;  // place of (cd, fd) inside the stored block
+  }
+  // the block leaves as NT4 16-byte stores per lane and, L * L being 0 or 1 modulo 4, one last dword
+  int qoff[NT4];
+#pragma unroll
+  for (int k = 0; k < NT4; ++k) {
+    const int q = lane + kWave * k;
+    qoff[k] = 4 * q + 3 < LL ? 16 * q : kDeadOffset;
+  }
+  const int tail_off = (lane == 0 && (LL & 3)) ? (LL - 1) * 4 : kDeadOffset;
+
+  const int last_p = ch.pix0 + (n - 1) * ch.pstep;
+  int ld_p = ch.pix0;
+  int ld_t = 0;
+  auto load_next = [&]() __attribute__((always_inline)) {
+    PixSF r;
+    const unsigned pp = (unsigned)uniform_i(ld_t < n ? ld_p : last_p);
+    const int vo = (int)(valid ? pp * (unsigned)vbytes + foff : kDeadWide);
+    float t1[1];
+    buf_load<1, true>(rS, vo, 0u, t1);
+    r.s = t1[0];
+    buf_load<1, true>(rMd, vo, 0u, t1);
+    r.md = t1[0];
+    buf_load<1, true>(rMi, vo, 0u, t1);
+    r.mi = t1[0];
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
+    ld_p += ch.pstep;
+    ld_t += 1;
+    return r;
+  };
+
+  float prev = 0.f, uf;
+  {
+    const PixSF p0 = load_next();
+    uf = fmaf(p0.s - p0.md, rho, -p0.mi);
+  }
+
+  constexpr int kOps = 4 + 2 + (TRAIN ? 2 + NT4 : 0);
+  constexpr int D = ring_depth(kOps);
+  PixSF ring[D];
+#pragma unroll
+  for (int u = 0; u < D; ++u) ring[u] = load_next();
+
+  int st_p = ch.pix0 + ch.pstep;
+  for (int t0 = 1; t0 < n; t0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int t = t0 + u;
+      const bool live = t < n;
+      wait_vmem<(D - 1) * kOps>();
+      const PixSF px = ring[u];
+      ring[u] = load_next();
+      const float tt = px.s - px.md;
+      const float un = fmaf(tt, rho, -px.mi);  // UpdateUnaryKernelSoft, TRWP_forward_soft.cu:161-181
+      const float w = uniform_f(px.w);
+      const float a = fmaf(rho, prev, uf);  // (every group holds the same a)
+      // this lane's duals and their softmin statistics around their own minimum (:81-97)
+      float dual[FM];
+      float mn_l = inf;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        dual[i] = fmaf(w, tcol[i], bperm_f(src[i], a));
+        mn_l = fminf(mn_l, inr[i] ? dual[i] : inf);
+      }
+      float se_l = 0.f, sd_l = 0.f;
+      const float ml2 = mn_l * kLog2e;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        const float e = inr[i] ? exp_below(dual[i], ml2) : 0.f;
+        se_l += e;
+        sd_l = fmaf(e, dual[i], sd_l);
+      }
+      if (TRAIN) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+          if (inr[i]) tile[tidx[i]] = dual[i];
+      }
+      float mn, se, sd, scale;
+      group_softmin<G>(addr, mn_l, se_l, sd_l, mn, se, sd, scale);
+      const float soft = sd * fast_rcp(se);
+      const float nmin = lanes_min<(G == 4 ? 16 : 32)>(store_lane ? soft : inf);
+      const float m = soft - nmin;
+      prev = m;
+      uf = un;
+      const unsigned sp = (unsigned)uniform_i(st_p);
+      const int vo = (int)((store_lane && live) ? sp * (unsigned)vbytes + foff : kDeadWide);
+      const float m1[1] = {m}, s1[1] = {tt + m};
+      buf_store<1, true>(rMo, vo, 0u, m1);
+      buf_store<1, true>(rSo, vo, 0u, s1);
+      if (TRAIN) {
+        const bool pr[1] = {store_lane && (soft == nmin)};
+        const int nidx = last_label<1>(pr, L - 1);
+        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm,
+                                             live ? (int)sp : kDeadOffset, 0, 0);
+        const rsrc_t dBlk = make_rsrc(bBlk + (int64_t)sp * LL, live ? LL * 4 : 0);
+#pragma unroll
+        for (int k = 0; k < NT4; ++k) {
+          const float4 v = reinterpret_cast<const float4*>(tile)[lane + kWave * k];
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), dBlk, qoff[k], 0,
+                                                 MPL_ST_AUX);
+        }
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, tile[LL - 1]), dBlk,
+                                              tail_off, 0, MPL_ST_AUX);
+      }
+      st_p += ch.pstep;
+    }
+  }
+}
+
+// NQ: float4 reads that cover a row of the gradient block (4 * NQ >= L).  The duals come straight
+// from memory into the registers of the lanes that use them (F gathers per lane: staging the block
+// through LDS with 16-byte loads, as the forward scan stores it, measured slower here).
+template <int G, int FM, int NQ>
+__global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams p) {
+  extern __shared__ float smem[];
+  const int L = p.L, LL = L * L;
+  constexpr int S = 4 * NQ;  // row stride of the gradient block
+  float* tab = smem;         // LL
+  const int LLp = (LL + 3) & ~3;  // (keeps the rows of the gradient block 16-byte aligned)
+  float* hist = tab + LLp;   // LL: per-pair dcontext accumulator [fd * L + cd]
+  float* grad = hist + LLp;  // L rows of S: ddual[fd * S + cd], 0 beyond cd = L - 1
+  const int lane = threadIdx.x;
+  const int64_t HW = (int64_t)p.H * p.W;
+  const int64_t P = (int64_t)p.B * HW;
+  const int64_t N = P * L;
+  const ChainCtx ch = locate_chain(p);
+  const int dir = ch.dir;
+  const int n = ch.n;
+
+  fill_table(p.ctx, L, p.ctx2d, lane, tab);
+  for (int i = lane; i < LL; i += kWave) hist[i] = 0.f;
+  for (int i = lane; i < L * S; i += kWave) grad[i] = 0.f;
+  __syncthreads();
+
+  const int64_t img_p = (int64_t)ch.bv * HW;
+  const int64_t img_e = img_p * L;
+  const int vbytes = L * 4;
+  const bool read_h = !p.first_touch;
+  const int img_bytes = (int)(unsigned)(HW * L * 4);
+  const rsrc_t rA = make_rsrc(p.a_in + img_e, img_bytes);
+  const rsrc_t rAo = make_rsrc(p.a_out + img_e, img_bytes);
+  float* const bHd = p.h + (int64_t)dir * N + img_e;
+  float* const bHi = p.h + (int64_t)(dir ^ 1) * N + img_e;
+  const rsrc_t rHdIn = make_rsrc(bHd, read_h ? img_bytes : 0);
+  const rsrc_t rHiIn = make_rsrc(bHi, read_h ? img_bytes : 0);
+  const rsrc_t rHd = make_rsrc(bHd, img_bytes);
+  const rsrc_t rHi = make_rsrc(bHi, img_bytes);
+  const float* __restrict__ bBlk = p.edge_label + ((int64_t)dir * P + img_p) * LL;
+  const int img_bytes_p = (int)(HW * 4 > 0x7fffffff ? 0x7fffffff : HW * 4);
+  const rsrc_t dInorm = make_rsrc(p.idx_norm + (int64_t)dir * P + img_p, (int)HW);
+  const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P + img_p, img_bytes_p);
+  const rsrc_t dDe = make_rsrc(p.dedge != nullptr ? p.dedge + (int64_t)dir * P + img_p : nullptr,
+                               p.dedge != nullptr ? img_bytes_p : 0);
+  const float rho = p.rho;
+  const float inf = INFINITY;
+  const int F = (L + G - 1) / G;
+  const bool valid = lane < G * L;
+  const int g = valid ? lane / L : 0;
+  const int cd = valid ? lane - g * L : 0;
+  const bool store_lane = lane < L;
+  const unsigned foff = (unsigned)cd * 4u;
+  const bool even = (dir & 1) == 0;
+  int addr[G];
+#pragma unroll
+  for (int k = 0; k < G; ++k) addr[k] = (valid ? k * L + cd : lane) * 4;
+  const int fd0 = g * F;
+  float tcol[FM], hreg[FM];
+  int boff[FM], gidx[FM];
+  bool inr[FM];
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    inr[i] = valid && i < F && fd0 + i < L;
+    const int fd = inr[i] ? fd0 + i : L - 1;
+    tcol[i] = tab[fd * L + cd];
+    hreg[i] = 0.f;
+    // place of (cd, fd) inside the pixel's stored block
+    boff[i] = inr[i] ? (even ? fd * L + cd : cd * L + fd) * 4 : kDeadOffset;
+    gidx[i] = fd * S + cd;
+  }
+  const float4* grow = reinterpret_cast<const float4*>(grad + cd * S);  // row of front label cd
+
+  int ld_t = n - 1;
+  int ld_p = ch.pix0 + (n - 1) * ch.pstep;
+  auto load_next = [&]() __attribute__((always_inline)) {
+    PixSS<FM> r;
+    const unsigned pp = (unsigned)uniform_i(ld_t >= 0 ? ld_p : ch.pix0);
+    const int vo = (int)(valid ? pp * (unsigned)vbytes + foff : kDeadWide);
+    float t1[1];
+    buf_load<1, true>(rA, vo, 0u, t1);
+    r.a = t1[0];
+    buf_load<1, true>(rHdIn, vo, 0u, t1);
+    r.hd = t1[0];
+    buf_load<1, true>(rHiIn, vo, 0u, t1);
+    r.hi = t1[0];
+    r.nidx = __builtin_amdgcn_raw_buffer_load_b8(dInorm, (int)pp, 0, 0);
+    r.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pp * 4u), 0, 0));
+    r.de = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(dDe, (int)(pp * 4u), 0, 0));
+    const rsrc_t dBlk = make_rsrc(bBlk + (int64_t)pp * LL, LL * 4);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+      r.dual[i] = __builtin_bit_cast(
+          float, __builtin_amdgcn_raw_buffer_load_b32(dBlk, boff[i], 0, MPL_LD_AUX));
+    ld_t -= 1;
+    ld_p -= ch.pstep;
+    return r;
+  };
+
+  constexpr int kOps = 3 + 3 + FM + 3 + 1;
+  constexpr int D = ring_depth(kOps);
+  PixSS<FM> ring[D];
+#pragma unroll
+  for (int u = 0; u < D; ++u) ring[u] = load_next();
+
+  float sc = 0.f;  // dU of the current pixel (every group holds the same value)
+  int st_p = ch.pix0 + (n - 1) * ch.pstep;
+  for (int s0 = 0; s0 < n; s0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int t = n - 1 - (s0 + u);
+      wait_vmem<(D - 1) * kOps>();
+      const PixSS<FM> px = ring[u];
+      ring[u] = load_next();
+      float scn = 0.f, det = 0.f;
+      if (t >= 1) {  // the chain start (t == 0) has no incoming edge
+        const float w = uniform_f(px.w);
+        const int nidx = __builtin_amdgcn_readfirstlane(px.nidx);
+        float gv = valid ? fmaf(rho, sc, px.a + px.hd) : 0.f;
+        // back norm, TRWP_backward_soft.cu:52-63
+        const float tot = lanes_sum<(G == 4 ? 16 : 32)>(store_lane ? gv : 0.f);
+        if (cd == nidx) gv -= tot;
+        // softmin statistics of this lane's label over all its front labels (:83-105)
+        float ex[FM];
+        float mn_l = inf;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) mn_l = fminf(mn_l, inr[i] ? px.dual[i] : inf);
+        float se_l = 0.f, sd_l = 0.f;
+        const float ml2 = mn_l * kLog2e;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          ex[i] = inr[i] ? exp_below(px.dual[i], ml2) : 0.f;
+          se_l += ex[i];
+          sd_l = fmaf(ex[i], px.dual[i], sd_l);
+        }
+        float mn, se, sd, scale;
+        group_softmin<G>(addr, mn_l, se_l, sd_l, mn, se, sd, scale);
+        const float inv = fast_rcp(se);
+        const float soft1 = fmaf(sd, inv, 1.f);
+        const float gs = gv * inv * scale;
+        float de = 0.f;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          // :110-113; nothing beyond the last label, and nothing on an idle lane (whose se is 0)
+          const float dd = inr[i] ? gs * ex[i] * (soft1 - px.dual[i]) : 0.f;
+          de = fmaf(tcol[i], dd, de);
+          hreg[i] = fmaf(w, dd, hreg[i]);
+          if (inr[i]) grad[gidx[i]] = dd;
+        }
+        // dU[q, fd] = sum_cd ddual[cd, fd]: every lane of label fd adds up the row in the same order
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) {
+          const float4 v = grow[q];
+          scn += (v.x + v.y) + (v.z + v.w);
+        }
+        det = lanes_sum<kWave>(de);
+      }
+      const unsigned sp = (unsigned)uniform_i(st_p);
+      const int vo = (int)((store_lane && t >= 0) ? sp * (unsigned)vbytes + foff : kDeadWide);
+      const float an = fmaf(rho, sc, px.a);  // g_k += rho*dU for every k, dunary too
+      const float a1[1] = {an}, h1[1] = {-an}, i1[1] = {px.hi - sc};
+      buf_store<1, true>(rAo, vo, 0u, a1);
+      buf_store<1, true>(rHd, vo, 0u, h1);
+      buf_store<1, true>(rHi, vo, 0u, i1);
+      __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
+                                            t >= 1 ? (int)(sp * 4u) : kDeadOffset, 0, 0);
+      sc = scn;
+      st_p -= ch.pstep;
+    }
+  }
+  if (p.dctx == nullptr) return;
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+    if (inr[i]) hist[(fd0 + i) * L + cd] = hreg[i];
+  __syncthreads();
+  // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D), the diagonal
+  // included (TRWP_backward_soft.cu:116-126)
+  if (!p.ctx2d) {
+    if (lane < L) {
+      float acc = 0.f;
+      for (int fd = 0; fd < L; ++fd) {
+        if (fd + lane < L) acc += hist[fd * L + fd + lane];
+        if (lane > 0 && fd - lane >= 0) acc += hist[fd * L + fd - lane];
+      }
+      if (acc != 0.f) atomicAdd(&p.dctx[lane], acc);
+    }
+  } else {
+    for (int i = lane; i < LL; i += kWave) {
+      const int fd = i / L, c2 = i - fd * L;
+      if (c2 > fd) continue;  // handled by the (fd, cd) entry
+      const float v = hist[i] + (c2 < fd ? hist[c2 * L + fd] : 0.f);
+      if (v != 0.f) atomicAdd(&p.dctx[c2 * L + fd], v);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // More than 64 labels (up to 256, the label count the reference's stereo build accepts for
 // ForwardSoft, TRWP_hard_soft/TRWP.cpp:336-340): R = ceil(L / 64) labels per lane, lane i owning
 // labels i, i + 64, ...  A pixel's block of duals (L * L floats, up to 256 KB) does not fit in LDS,
@@ -915,6 +1363,24 @@ void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st) {
   const int LL = p.L * p.L;
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (LL + (train ? (LL > kWave * T ? LL : kWave * T) : 0));
+  if (p.L <= 32 && p.L >= 2) {  // front labels split over the idle lanes
+#define MPL_SOFT_SPLIT_FWD(GG, FF, NN)                                                       \
+  do {                                                                                       \
+    const size_t slds = sizeof(float) * (LL + (train ? 256 * NN : 0));                       \
+    if (train)                                                                               \
+      soft_split_fwd_kernel<true, GG, FF, NN><<<blocks, kWave, slds, st>>>(p);               \
+    else                                                                                     \
+      soft_split_fwd_kernel<false, GG, FF, NN><<<blocks, kWave, slds, st>>>(p);              \
+  } while (0)
+    if (p.L <= 16)
+      MPL_SOFT_SPLIT_FWD(4, 4, 1);
+    else if (p.L <= 21)
+      MPL_SOFT_SPLIT_FWD(3, 7, 2);
+    else
+      MPL_SOFT_SPLIT_FWD(2, 16, 4);
+#undef MPL_SOFT_SPLIT_FWD
+    return;
+  }
   if (!train) {
     if (p.L == 21)
       soft_fwd_kernel<false, 0, 21><<<blocks, kWave, lds, st>>>(p);
@@ -951,6 +1417,17 @@ void launch_soft_bwd(const BackParams& p, hipStream_t st) {
   const int LL = p.L * p.L;
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (2 * LL + kWave * T + p.L * (p.L | 1));
+  if (p.L <= 32 && p.L >= 2) {  // front labels split over the idle lanes
+    const int NQ = p.L <= 16 ? 4 : (p.L <= 21 ? 6 : 8);
+    const size_t slds = sizeof(float) * (2 * ((LL + 3) & ~3) + p.L * 4 * NQ);
+    if (p.L <= 16)
+      soft_split_bwd_kernel<4, 4, 4><<<blocks, kWave, slds, st>>>(p);
+    else if (p.L <= 21)
+      soft_split_bwd_kernel<3, 7, 6><<<blocks, kWave, slds, st>>>(p);
+    else
+      soft_split_bwd_kernel<2, 16, 8><<<blocks, kWave, slds, st>>>(p);
+    return;
+  }
   if (p.L == 21) {
     soft_bwd_kernel<7, 21><<<blocks, kWave, lds, st>>>(p);
     return;

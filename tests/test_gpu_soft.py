@@ -21,6 +21,13 @@ CASES = [
     (4, 1, 1, 9, 8, "tl2", 2),
     (4, 1, 9, 1, 8, "tl2", 2),
     (2, 3, 3, 12, 3, "tl2", 3),
+    # up to 32 labels the front labels of a pixel are split over 4 / 3 / 2 groups of lanes
+    (4, 1, 4, 6, 2, "tl2", 2),          # one front label per group, two groups idle
+    (4, 1, 4, 5, 13, "dense2d", 2),     # 4 groups, the last one holds a single front label
+    (4, 1, 5, 4, 17, "dense2d", 1),     # smallest 3-group case: 6 + 6 + 5 front labels
+    (8, 1, 4, 5, 20, "tl3", 1),         # 7 + 7 + 6
+    (4, 1, 3, 4, 22, "dense1d", 1),     # smallest 2-group case
+    (4, 1, 3, 3, 32, "dense2d", 1),     # every lane used, 16 front labels each
     # more than 64 labels (the stereo build accepts up to 256, TRWP_hard_soft/TRWP.cpp:336-340):
     # several labels per lane, the duals move through LDS in chunks of 32 front labels
     (4, 1, 4, 5, 65, "tl3", 2),         # one label in the second register, one 1-label chunk
