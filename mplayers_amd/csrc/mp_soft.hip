@@ -36,12 +36,12 @@ __device__ __forceinline__ void fill_table(const float* ctx, int L, int ctx2d, i
   }
 }
 
-// LT > 0: the label count is known at compile time (the segmentation case, 21 labels): the loops
-// over front labels are unrolled and the lane's column of the context table lives in registers.
-template <bool TRAIN, int T, int LT>
+// One label per lane: 33 to 64 labels; fewer labels take the lane-split kernels below, more the
+// several-labels-per-lane ones.
+template <bool TRAIN, int T>
 __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
   extern __shared__ float smem[];
-  const int L = LT > 0 ? LT : p.L, LL = L * L;
+  const int L = p.L, LL = L * L;
   float* tab = smem;        // LL floats
   float* tile = smem + LL;  // max(LL, 64 * T) floats: the pixel's block of duals
   const int lane = threadIdx.x;
@@ -74,11 +74,6 @@ __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
   const bool valid = lane < L;
   const int col = valid ? lane : L - 1;  // keeps the table reads of idle lanes in range
   const bool even = (dir & 1) == 0;
-  float tcol[LT > 0 ? LT : 1];  // ctx(cd = lane, fd)
-  if (LT > 0) {
-#pragma unroll
-    for (int fd = 0; fd < LT; ++fd) tcol[fd] = tab[fd * L + col];
-  }
   const int wstep = even ? L : 1;             // address step of the front label inside the block
   const int wbase = even ? lane : lane * L;   // address of (cd = lane, fd = 0)
 
@@ -132,38 +127,19 @@ __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
       // pass 1: minimum of the duals of this lane's label; the block goes to LDS
       float mn = inf;
       float se = 0.f, sd = 0.f;
-      if constexpr (LT > 0) {
-        float dual[LT];
-#pragma unroll
-        for (int fd = 0; fd < LT; ++fd) {
-          dual[fd] = fmaf(w, tcol[fd], readlane_f(a, fd));
-          mn = fminf(mn, dual[fd]);
-        }
-        if (TRAIN && valid) {  // one predicated region for the whole column, not one per store
-#pragma unroll
-          for (int fd = 0; fd < LT; ++fd) tile[wbase + fd * wstep] = dual[fd];
-        }
-        // pass 2: softmin weights and the expected dual
-#pragma unroll
-        for (int fd = 0; fd < LT; ++fd) {
-          const float e = fast_exp(mn - dual[fd]);
-          se += e;
-          sd = fmaf(e, dual[fd], sd);
-        }
-      } else {
 #pragma unroll 4
-        for (int fd = 0; fd < L; ++fd) {
-          const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
-          mn = fminf(mn, dual);
-          if (TRAIN && valid) tile[wbase + fd * wstep] = dual;
-        }
+      for (int fd = 0; fd < L; ++fd) {
+        const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
+        mn = fminf(mn, dual);
+        if (TRAIN && valid) tile[wbase + fd * wstep] = dual;
+      }
+      // pass 2: softmin weights and the expected dual
 #pragma unroll 4
-        for (int fd = 0; fd < L; ++fd) {
-          const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
-          const float e = fast_exp(mn - dual);
-          se += e;
-          sd = fmaf(e, dual, sd);
-        }
+      for (int fd = 0; fd < L; ++fd) {
+        const float dual = fmaf(w, tab[fd * L + col], readlane_f(a, fd));
+        const float e = fast_exp(mn - dual);
+        se += e;
+        sd = fmaf(e, dual, sd);
       }
       const float soft = sd / se;
       const float nmin = wave_min(valid ? soft : inf);
@@ -204,10 +180,10 @@ struct PixSB {
   float blk[T];
 };
 
-template <int T, int LT>
+template <int T>
 __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
   extern __shared__ float smem[];
-  const int L = LT > 0 ? LT : p.L, LL = L * L;
+  const int L = p.L, LL = L * L;
   const int Lp = L | 1;  // odd row stride of the transposed gradient block: conflict-free reads
   constexpr int kTile = kWave * T;
   float* tab = smem;            // LL
@@ -248,14 +224,6 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
   const bool even = (dir & 1) == 0;
   const int dstep = even ? L : 1;             // address step of the front label inside the block
   const int dbase = even ? col : col * L;     // address of (cd = lane, fd = 0)
-  float tcol[LT > 0 ? LT : 1], hreg[LT > 0 ? LT : 1];  // ctx(lane, fd); dcontext partial sums
-  if (LT > 0) {
-#pragma unroll
-    for (int fd = 0; fd < LT; ++fd) {
-      tcol[fd] = tab[fd * L + col];
-      hreg[fd] = 0.f;
-    }
-  }
 
   int ld_t = n - 1;
   int ld_p = ch.pix0 + (n - 1) * ch.pstep;
@@ -311,55 +279,26 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
         // softmin statistics of this lane's label, :83-105
         float mn = INFINITY;
         float se = 0.f, sd = 0.f, de = 0.f;
-        if constexpr (LT > 0) {
-          float dual[LT], ex[LT];
-#pragma unroll
-          for (int fd = 0; fd < LT; ++fd) {
-            dual[fd] = tile[dbase + fd * dstep];
-            mn = fminf(mn, dual[fd]);
-          }
-#pragma unroll
-          for (int fd = 0; fd < LT; ++fd) {
-            ex[fd] = fast_exp(mn - dual[fd]);
-            se += ex[fd];
-            sd = fmaf(ex[fd], dual[fd], sd);
-          }
-          const float inv = 1.f / se;
-          const float soft1 = fmaf(sd, inv, 1.f);
-          const float gs = gv * inv;
-#pragma unroll
-          for (int fd = 0; fd < LT; ++fd) {
-            const float dd = gs * ex[fd] * (soft1 - dual[fd]);  // :110-113
-            de = fmaf(tcol[fd], dd, de);
-            hreg[fd] = fmaf(w, dd, hreg[fd]);
-            ex[fd] = dd;
-          }
-          if (valid) {  // one predicated region for the whole column, not one per store
-#pragma unroll
-            for (int fd = 0; fd < LT; ++fd) grad[fd * Lp + lane] = ex[fd];
-          }
-        } else {
 #pragma unroll 4
-          for (int fd = 0; fd < L; ++fd) mn = fminf(mn, tile[dbase + fd * dstep]);
+        for (int fd = 0; fd < L; ++fd) mn = fminf(mn, tile[dbase + fd * dstep]);
+#pragma unroll 4
+        for (int fd = 0; fd < L; ++fd) {
+          const float dual = tile[dbase + fd * dstep];
+          const float e = fast_exp(mn - dual);
+          se += e;
+          sd = fmaf(e, dual, sd);
+        }
+        const float inv = 1.f / se;
+        const float soft1 = fmaf(sd, inv, 1.f);
+        const float gs = gv * inv;
+        if (valid) {  // (lanes without a label carry gv = 0 and would add nothing)
 #pragma unroll 4
           for (int fd = 0; fd < L; ++fd) {
             const float dual = tile[dbase + fd * dstep];
-            const float e = fast_exp(mn - dual);
-            se += e;
-            sd = fmaf(e, dual, sd);
-          }
-          const float inv = 1.f / se;
-          const float soft1 = fmaf(sd, inv, 1.f);
-          const float gs = gv * inv;
-          if (valid) {  // (lanes without a label carry gv = 0 and would add nothing)
-#pragma unroll 4
-            for (int fd = 0; fd < L; ++fd) {
-              const float dual = tile[dbase + fd * dstep];
-              const float dd = gs * fast_exp(mn - dual) * (soft1 - dual);  // :110-113
-              de = fmaf(tab[fd * L + col], dd, de);
-              hist[fd * L + lane] = fmaf(w, dd, hist[fd * L + lane]);  // this lane's own entries
-              grad[fd * Lp + lane] = dd;
-            }
+            const float dd = gs * fast_exp(mn - dual) * (soft1 - dual);  // :110-113
+            de = fmaf(tab[fd * L + col], dd, de);
+            hist[fd * L + lane] = fmaf(w, dd, hist[fd * L + lane]);  // this lane's own entries
+            grad[fd * Lp + lane] = dd;
           }
         }
         // dU[q, fd] = sum_cd ddual[cd, fd]: lane fd adds up its row of the transposed block
@@ -384,10 +323,6 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
     }
   }
   if (p.dctx == nullptr) return;
-  if (LT > 0 && valid) {
-#pragma unroll
-    for (int fd = 0; fd < LT; ++fd) hist[fd * L + lane] = hreg[fd];
-  }
   __syncthreads();
   // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D), the diagonal
   // included (TRWP_backward_soft.cu:116-126)
@@ -1331,10 +1266,9 @@ __global__ void __launch_bounds__(kWave) swm_bwd_kernel(const float* __restrict_
   }
 }
 
-int tile_bucket(int L) {
-  const int need = (L * L + kWave - 1) / kWave;
-  return need <= 4 ? 4 : (need <= 7 ? 7 : (need <= 16 ? 16 : 64));
-}
+// dwords per lane that cover a pixel's block of duals in the one-label-per-lane kernels (33 to 64
+// labels: up to 64)
+int tile_bucket(int) { return kWave; }
 
 }  // namespace
 
@@ -1363,7 +1297,7 @@ void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st) {
   const int LL = p.L * p.L;
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (LL + (train ? (LL > kWave * T ? LL : kWave * T) : 0));
-  if (p.L <= 32 && p.L >= 2) {  // front labels split over the idle lanes
+  if (p.L <= 32) {  // front labels split over the idle lanes
 #define MPL_SOFT_SPLIT_FWD(GG, FF, NN)                                                       \
   do {                                                                                       \
     const size_t slds = sizeof(float) * (LL + (train ? 256 * NN : 0));                       \
@@ -1381,23 +1315,10 @@ void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st) {
 #undef MPL_SOFT_SPLIT_FWD
     return;
   }
-  if (!train) {
-    if (p.L == 21)
-      soft_fwd_kernel<false, 0, 21><<<blocks, kWave, lds, st>>>(p);
-    else
-      soft_fwd_kernel<false, 0, 0><<<blocks, kWave, lds, st>>>(p);
-    return;
-  }
-  if (p.L == 21) {
-    soft_fwd_kernel<true, 7, 21><<<blocks, kWave, lds, st>>>(p);
-    return;
-  }
-  switch (T) {
-    case 4: soft_fwd_kernel<true, 4, 0><<<blocks, kWave, lds, st>>>(p); break;
-    case 7: soft_fwd_kernel<true, 7, 0><<<blocks, kWave, lds, st>>>(p); break;
-    case 16: soft_fwd_kernel<true, 16, 0><<<blocks, kWave, lds, st>>>(p); break;
-    default: soft_fwd_kernel<true, 64, 0><<<blocks, kWave, lds, st>>>(p); break;
-  }
+  if (!train)
+    soft_fwd_kernel<false, 0><<<blocks, kWave, lds, st>>>(p);
+  else
+    soft_fwd_kernel<true, kWave><<<blocks, kWave, lds, st>>>(p);
 }
 
 void launch_soft_bwd(const BackParams& p, hipStream_t st) {
@@ -1417,7 +1338,7 @@ void launch_soft_bwd(const BackParams& p, hipStream_t st) {
   const int LL = p.L * p.L;
   const int T = tile_bucket(p.L);
   const size_t lds = sizeof(float) * (2 * LL + kWave * T + p.L * (p.L | 1));
-  if (p.L <= 32 && p.L >= 2) {  // front labels split over the idle lanes
+  if (p.L <= 32) {  // front labels split over the idle lanes
     const int NQ = p.L <= 16 ? 4 : (p.L <= 21 ? 6 : 8);
     const size_t slds = sizeof(float) * (2 * ((LL + 3) & ~3) + p.L * 4 * NQ);
     if (p.L <= 16)
@@ -1428,21 +1349,10 @@ void launch_soft_bwd(const BackParams& p, hipStream_t st) {
       soft_split_bwd_kernel<2, 16, 8><<<blocks, kWave, slds, st>>>(p);
     return;
   }
-  if (p.L == 21) {
-    soft_bwd_kernel<7, 21><<<blocks, kWave, lds, st>>>(p);
-    return;
-  }
-  switch (T) {
-    case 4: soft_bwd_kernel<4, 0><<<blocks, kWave, lds, st>>>(p); break;
-    case 7: soft_bwd_kernel<7, 0><<<blocks, kWave, lds, st>>>(p); break;
-    case 16: soft_bwd_kernel<16, 0><<<blocks, kWave, lds, st>>>(p); break;
-    default:
-      // up to 66 KB of LDS at 64 labels: above the default limit of a workgroup
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&soft_bwd_kernel<64, 0>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      soft_bwd_kernel<64, 0><<<blocks, kWave, lds, st>>>(p);
-      break;
-  }
+  // up to 66 KB of LDS at 64 labels: above the default limit of a workgroup
+  (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&soft_bwd_kernel<kWave>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  soft_bwd_kernel<kWave><<<blocks, kWave, lds, st>>>(p);
 }
 
 void launch_swm_fwd(const float* msg, int n_trees, int L, float* out, uint8_t* min_ind,

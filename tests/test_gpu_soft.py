@@ -22,6 +22,7 @@ CASES = [
     (4, 1, 9, 1, 8, "tl2", 2),
     (2, 3, 3, 12, 3, "tl2", 3),
     # up to 32 labels the front labels of a pixel are split over 4 / 3 / 2 groups of lanes
+    (4, 1, 3, 4, 1, "tl2", 2),          # a single label: every message is 0
     (4, 1, 4, 6, 2, "tl2", 2),          # one front label per group, two groups idle
     (4, 1, 4, 5, 13, "dense2d", 2),     # 4 groups, the last one holds a single front label
     (4, 1, 5, 4, 17, "dense2d", 1),     # smallest 3-group case: 6 + 6 + 5 front labels
