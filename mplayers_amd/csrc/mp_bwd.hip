@@ -177,12 +177,9 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
       buf_load_u8<R, VEC>(make_rsrc(bImin, (int)(pp * (unsigned)L + (unsigned)L)), lab0,
                           pp * (unsigned)L, r.fd);
     }
-    if (!JACOBI) {
-      if (inv_from_a) {
-#pragma unroll
-        for (int j = 0; j < R; ++j) r.hi[j] = -r.a[j];
-      }
-    } else {
+    // (no arithmetic on what was just loaded in here: it would have to wait for the loads, and the
+    // compiler places such work at the end of the loop body, where the wait drains the whole queue)
+    if (JACOBI) {
 #pragma unroll
       for (int j = 0; j < R; ++j) r.hd[j] = r.hi[j] = 0.f;
     }
@@ -205,7 +202,12 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   // register it started in (a single bank ends the loop in one register move per value in flight)
   PixB<R> ring[D], ring2[D];
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    MPL_ORDER_LOADS();
+  }
 
   float sc[R];  // dU of the current pixel: what the previous step scattered into it
   float hist_reg[R];        // dcontext[label] partial sums of this lane's own labels (1-D context)
@@ -399,7 +401,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
         for (int j = 0; j < R; ++j) {
           an[j] = fmaf(rho, sc[j], px.a[j]);  // g_k += rho*dU for every k, dunary too
           hdn[j] = -an[j];                    // g_dir = 0 after its sweep
-          hin[j] = px.hi[j] - sc[j];          // g_inv -= dU
+          // g_inv -= dU; after the opposite direction's sweep g_inv is -A and was not read
+          hin[j] = (inv_from_a ? -px.a[j] : px.hi[j]) - sc[j];
         }
         // h_dir = -A is only read by the next launch when that one sweeps the opposite
         // direction, which derives it from A instead: nothing is stored then (nor after the last

@@ -59,6 +59,13 @@ __device__ __forceinline__ void wait_vmem() {
   __builtin_amdgcn_s_waitcnt((n & 0xf) | ((n >> 4) << 14) | (0x7 << 4) | (0xf << 8));
 }
 
+// Scheduling fence between the groups of loads that fill the prefetch ring before a scan loop.
+#ifndef MPL_NO_ORDER_LOADS
+#define MPL_ORDER_LOADS() __builtin_amdgcn_sched_barrier(0)
+#else
+#define MPL_ORDER_LOADS() ((void)0)
+#endif
+
 // number of instructions one R-label access of floats / of bytes takes
 constexpr int vec_ops(int R, bool vec) { return vec ? 1 : R; }
 constexpr int byte_ops(int R, bool vec) { return (vec && (R == 4 || R == 2)) ? 1 : R; }

@@ -446,6 +446,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   float prev[R], uf[R];
   {
     const PixF<R> p0 = load_next(true);
+    MPL_ORDER_LOADS();  // (the chain start's loads stay ahead of the ring's)
     float conv[R];  // the start pixel's belief-plane value in the other representation
 #pragma unroll
     for (int j = 0; j < R; ++j) conv[j] = 0.f;
@@ -489,7 +490,12 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // single bank the loop ends in one register move per value in flight).
   PixF<R> ring[D], ring2[D];
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    MPL_ORDER_LOADS();
+  }
 
   int st_p = ch.pix0 + ch.pstep;
   auto step = [&](const PixF<R>& px, const int t) __attribute__((always_inline)) {

@@ -191,6 +191,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
   float prev = 0.f, uf;
   {
     const PixPF p0 = load_next();
+    MPL_ORDER_LOADS();  // (the chain start's loads stay ahead of the ring's)
     const float t0 = pair_second ? p0.s + p0.mi : p0.s - p0.md;
     const float un = JACOBI ? p0.s : fmaf(t0, rho, -p0.mi);
     uf = on ? un : inf;
@@ -205,7 +206,12 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
   constexpr int D = ring_depth(kOps);
   PixPF ring[D];
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    MPL_ORDER_LOADS();
+  }
 
   int st_pix = ch.pix0 + ch.pstep;
   for (int t0 = 1; t0 < ch.n_max; t0 += D) {
@@ -347,7 +353,12 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
   constexpr int D = ring_depth(kOps);
   PixPB ring[D];
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    MPL_ORDER_LOADS();
+  }
 
   float sc = 0.f;  // dU of the current pixel: what the previous step scattered into it
   int st_pix = ch.pix0 + (n - 1) * ch.pstep;

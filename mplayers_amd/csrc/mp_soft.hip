@@ -101,25 +101,25 @@ __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
   float prev = 0.f, uf;
   {
     const PixSF p0 = load_next();
+    __builtin_amdgcn_sched_barrier(0);  // (the chain start's loads stay ahead of the ring's)
     const float un = fmaf(p0.s - p0.md, rho, -p0.mi);
     uf = valid ? un : inf;
   }
 
   constexpr int kOps = 4 + 2 + (TRAIN ? 1 + T : 0);
   constexpr int D = ring_depth(kOps);
-  PixSF ring[D];
+  PixSF ring[D], ring2[D];  // two banks, filled and used in turn: no register is moved
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   int st_p = ch.pix0 + ch.pstep;
-  for (int t0 = 1; t0 < n; t0 += D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      const int t = t0 + u;
+  auto step = [&](const PixSF& px, const int t) __attribute__((always_inline)) {
       const bool live = t < n;
-      wait_vmem<(D - 1) * kOps>();
-      const PixSF px = ring[u];
-      ring[u] = load_next();
       const float tt = px.s - px.md;
       const float un = valid ? fmaf(tt, rho, -px.mi) : inf;  // UpdateUnaryKernelSoft, :161-181
       const float w = uniform_f(px.w);
@@ -168,6 +168,25 @@ __global__ void __launch_bounds__(kWave) soft_fwd_kernel(const SweepParams p) {
         }
       }
       st_p += ch.pstep;
+  };
+  for (int t0 = 1; t0 < n; t0 += 2 * D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring[u];
+      ring2[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);  // the next pixel's loads go out before this step's work
+      step(px, t0 + u);
+    }
+    if (t0 + D >= n) break;  // wave-uniform
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring2[u];
+      ring[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);
+      step(px, t0 + D + u);
     }
   }
 }
@@ -254,19 +273,18 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
 
   constexpr int kOps = 3 + 3 + T + 3 + 1;
   constexpr int D = ring_depth(kOps);
-  PixSB<T> ring[D];
+  PixSB<T> ring[D], ring2[D];  // two banks, filled and used in turn: no register is moved
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   float sc = 0.f;  // dU of the current pixel: what the previous step scattered into it
   int st_p = ch.pix0 + (n - 1) * ch.pstep;
-  for (int s0 = 0; s0 < n; s0 += D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      const int t = n - 1 - (s0 + u);
-      wait_vmem<(D - 1) * kOps>();
-      const PixSB<T> px = ring[u];
-      ring[u] = load_next();
+  auto step = [&](const PixSB<T>& px, const int t) __attribute__((always_inline)) {
       float scn = 0.f, det = 0.f;
       if (t >= 1) {  // the chain start (t == 0) has no incoming edge
         const float w = uniform_f(px.w);
@@ -320,6 +338,25 @@ __global__ void __launch_bounds__(kWave) soft_bwd_kernel(const BackParams p) {
                                             t >= 1 ? (int)(sp * 4u) : kDeadOffset, 0, 0);
       sc = scn;
       st_p -= ch.pstep;
+  };
+  for (int s0 = 0; s0 < n; s0 += 2 * D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring[u];
+      ring2[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);  // the next pixel's loads go out before this step's work
+      step(px, n - 1 - (s0 + u));
+    }
+    if (s0 + D >= n) break;  // wave-uniform
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring2[u];
+      ring[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);
+      step(px, n - 1 - (s0 + D + u));
     }
   }
   if (p.dctx == nullptr) return;
@@ -523,24 +560,24 @@ __global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams
   float prev = 0.f, uf;
   {
     const PixSF p0 = load_next();
+    __builtin_amdgcn_sched_barrier(0);  // (the chain start's loads stay ahead of the ring's)
     uf = fmaf(p0.s - p0.md, rho, -p0.mi);
   }
 
   constexpr int kOps = 4 + 2 + (TRAIN ? 2 + NT4 : 0);
   constexpr int D = ring_depth(kOps);
-  PixSF ring[D];
+  PixSF ring[D], ring2[D];  // two banks, filled and used in turn: no register is moved
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   int st_p = ch.pix0 + ch.pstep;
-  for (int t0 = 1; t0 < n; t0 += D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      const int t = t0 + u;
+  auto step = [&](const PixSF& px, const int t) __attribute__((always_inline)) {
       const bool live = t < n;
-      wait_vmem<(D - 1) * kOps>();
-      const PixSF px = ring[u];
-      ring[u] = load_next();
       const float tt = px.s - px.md;
       const float un = fmaf(tt, rho, -px.mi);  // UpdateUnaryKernelSoft, TRWP_forward_soft.cu:161-181
       const float w = uniform_f(px.w);
@@ -594,6 +631,25 @@ __global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams
                                               tail_off, 0, MPL_ST_AUX);
       }
       st_p += ch.pstep;
+  };
+  for (int t0 = 1; t0 < n; t0 += 2 * D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring[u];
+      ring2[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);  // the next pixel's loads go out before this step's work
+      step(px, t0 + u);
+    }
+    if (t0 + D >= n) break;  // wave-uniform
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring2[u];
+      ring[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);
+      step(px, t0 + D + u);
     }
   }
 }
@@ -698,19 +754,18 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
 
   constexpr int kOps = 3 + 3 + FM + 3 + 1;
   constexpr int D = ring_depth(kOps);
-  PixSS<FM> ring[D];
+  PixSS<FM> ring[D], ring2[D];  // two banks, filled and used in turn: no register is moved
 #pragma unroll
-  for (int u = 0; u < D; ++u) ring[u] = load_next();
+  for (int u = 0; u < D; ++u) {
+    ring[u] = load_next();
+    // keeps the pixels' loads in this order: the compiler's own waits in the loop are sized for
+    // the order it sees here, and a later pixel's loads placed first would make them drain the queue
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   float sc = 0.f;  // dU of the current pixel (every group holds the same value)
   int st_p = ch.pix0 + (n - 1) * ch.pstep;
-  for (int s0 = 0; s0 < n; s0 += D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      const int t = n - 1 - (s0 + u);
-      wait_vmem<(D - 1) * kOps>();
-      const PixSS<FM> px = ring[u];
-      ring[u] = load_next();
+  auto step = [&](const PixSS<FM>& px, const int t) __attribute__((always_inline)) {
       float scn = 0.f, det = 0.f;
       if (t >= 1) {  // the chain start (t == 0) has no incoming edge
         const float w = uniform_f(px.w);
@@ -765,6 +820,25 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
                                             t >= 1 ? (int)(sp * 4u) : kDeadOffset, 0, 0);
       sc = scn;
       st_p -= ch.pstep;
+  };
+  for (int s0 = 0; s0 < n; s0 += 2 * D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring[u];
+      ring2[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);  // the next pixel's loads go out before this step's work
+      step(px, n - 1 - (s0 + u));
+    }
+    if (s0 + D >= n) break;  // wave-uniform
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      wait_vmem<(D - 1) * kOps>();
+      const auto px = ring2[u];
+      ring[u] = load_next();
+      __builtin_amdgcn_sched_barrier(0);
+      step(px, n - 1 - (s0 + D + u));
     }
   }
   if (p.dctx == nullptr) return;
