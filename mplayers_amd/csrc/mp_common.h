@@ -60,11 +60,7 @@ __device__ __forceinline__ void wait_vmem() {
 }
 
 // Scheduling fence between the groups of loads that fill the prefetch ring before a scan loop.
-#ifndef MPL_NO_ORDER_LOADS
 #define MPL_ORDER_LOADS() __builtin_amdgcn_sched_barrier(0)
-#else
-#define MPL_ORDER_LOADS() ((void)0)
-#endif
 
 // number of instructions one R-label access of floats / of bytes takes
 constexpr int vec_ops(int R, bool vec) { return vec ? 1 : R; }
