@@ -331,7 +331,8 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
     r.a = ldf(dA, eo);
     if (!JACOBI) {
       r.hd = ldf(dHdIn, eo);
-      r.hi = ldf(dHiIn, eo);  // (not read after the opposite direction's sweep: -A, see the step)
+      r.hi = ldf(dHiIn, eo);
+      if (inv_from_a) r.hi = -r.a;
     } else {
       r.hd = r.hi = 0.f;
     }
@@ -350,7 +351,7 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
 
   constexpr int kOps = (JACOBI ? 1 : 3) + 3 + (DE ? 1 : 0) + (JACOBI ? 1 : 3) + (DE ? 1 : 0);
   constexpr int D = ring_depth(kOps);
-  PixPB ring[D], ring2[D];  // two banks, filled and used in turn: no register is moved
+  PixPB ring[D];
 #pragma unroll
   for (int u = 0; u < D; ++u) {
     ring[u] = load_next();
@@ -361,9 +362,14 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
 
   float sc = 0.f;  // dU of the current pixel: what the previous step scattered into it
   int st_pix = ch.pix0 + (n - 1) * ch.pstep;
-  auto step = [&](const PixPB& px, const int s) __attribute__((always_inline)) {
-      const int t = n - 1 - s;         // per lane
+  for (int s0 = 0; s0 < ch.n_max; s0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int t = n - 1 - (s0 + u);  // per lane
       const bool here = on && t >= 0;  // this lane's chain has a pixel at this step
+      wait_vmem<(D - 1) * kOps>();
+      const PixPB px = ring[u];
+      ring[u] = load_next();
       // gradient w.r.t. the normalised message of this pixel (none at the chain start, t == 0)
       const bool edge = on && t >= 1;
       float g = edge ? fmaf(rho, sc, JACOBI ? px.a : px.a + px.hd) : 0.f;
@@ -400,32 +406,13 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
         const float an = fmaf(rho, sc, px.a);  // g_k += rho * dU for every k, dunary too
         stf(dAo, eo, an);
         stf(dHdOut, eo, -an);          // g_dir = 0 after its sweep
-        stf(dHiOut, eo, (inv_from_a ? -px.a : px.hi) - sc);   // g_inv -= dU
+        stf(dHiOut, eo, px.hi - sc);   // g_inv -= dU
       }
       if (DE)
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, px.de + det), dDe,
                                               (edge && l == 0) ? st_pix * 4 : kDeadOffset, 0, 0);
       sc = here ? scn : 0.f;
       st_pix -= ch.pstep;
-  };
-  for (int s0 = 0; s0 < ch.n_max; s0 += 2 * D) {
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
-      wait_vmem<(D - 1) * kOps>();
-      const PixPB px = ring[u];
-      ring2[u] = load_next();
-      MPL_ORDER_LOADS();  // the next pixel's loads go out before this step's work
-      step(px, s0 + u);
-    }
-    if (s0 + D >= ch.n_max) break;  // wave-uniform
-#pragma unroll
-    for (int u = 0; u < D; ++u) {
-      wait_vmem<(D - 1) * kOps>();
-      const PixPB px = ring2[u];
-      ring[u] = load_next();
-      MPL_ORDER_LOADS();
-      step(px, s0 + D + u);
     }
   }
   if (!DC) return;
