@@ -257,21 +257,14 @@ def test_large_config_properties_at_full_size(gpu, mode):
   assert float(dedge[0, 0, 0, :, 1:].abs().max()) > 0.0
 
 
-@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
-def test_full_size_rows_match_oracle(gpu, oracle, mode):
-  """With only the two horizontal directions the rows of an image do not interact, so the oracle
-  can check a few rows of a full-size (1500 x 2000 x 192) run exactly as it checks small images:
-  first rows, a middle row and the last rows, whose byte offsets lie beyond 2^31."""
+def _check_rows(gpu, oracle, mode, unary, ctx, ew, dcost, n_iter, rho, what):
+  """Runs forward and backward with the two horizontal directions on device tensors and checks the
+  first rows, a middle row and the last rows against the oracle."""
   import torch
-  from mplayers_amd import lib_stereo, synthetic
-  cfg = synthetic.make_config("C5", seed=0, mode=mode)
-  B, H, W, L = cfg["B"], cfg["H"], cfg["W"], cfg["L"]
-  n_dir, n_iter, rho = 2, 2, cfg["rho"]
-  dev = "cuda:0"
-  unary = cfg["unary"].to(dev)
-  ctx = cfg["context"].to(dev)
-  ew = cfg["edge_weights"][:n_dir].contiguous().to(dev)
-  dcost = synthetic.upstream_grad(cfg).to(dev)
+  from mplayers_amd import lib_stereo
+  B, _, H, W, L = unary.shape
+  n_dir = 2
+  dev = unary.device
   msg = torch.zeros(n_dir, B, 1, H, W, L, device=dev)
   cost = torch.zeros(B, 1, H, W, L, device=dev)
   scratch = torch.zeros(B, 1, H, W, L, device=dev)
@@ -282,7 +275,7 @@ def test_full_size_rows_match_oracle(gpu, oracle, mode):
   dedge = torch.zeros(n_dir, B, 1, H, W, device=dev)
   dctx = torch.zeros(L, device=dev)
   dmsg = torch.empty_like(msg)
-  print("full-size rows", mode, flush=True)
+  print(what, mode, flush=True)
   if mode == "TRWP":
     lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch, empty)
     lib_stereo.TRWP.backward(rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, dmsg, scratch)
@@ -292,6 +285,7 @@ def test_full_size_rows_match_oracle(gpu, oracle, mode):
                              msg_tmp, empty)
     lib_stereo.ISGMR.backward(0, rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, scratch,
                               scratch, dmsg)
+    del msg_tmp
   torch.cuda.synchronize()
   rows = [0, 1, H // 2, H - 2, H - 1]
   sub = lambda t, ax: t.index_select(ax, torch.tensor(rows, device=t.device)).cpu().numpy()
@@ -310,6 +304,36 @@ def test_full_size_rows_match_oracle(gpu, oracle, mode):
                               dn.astype(np.float64), sub(imin, 4), sub(inorm, 4), rho)
   assert np.abs(sub(dunary, 2) - du).max() <= 1e-4 * max(1.0, np.abs(du).max())
   assert np.abs(sub(dedge, 3) - de).max() <= 1e-4 * max(1.0, np.abs(de).max())
+
+
+@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
+def test_full_size_rows_match_oracle(gpu, oracle, mode):
+  """With only the two horizontal directions the rows of an image do not interact, so the oracle
+  can check a few rows of a full-size (1500 x 2000 x 192) run exactly as it checks small images:
+  first rows, a middle row and the last rows, whose byte offsets lie beyond 2^31."""
+  from mplayers_amd import synthetic
+  cfg = synthetic.make_config("C5", seed=0, mode=mode)
+  dev = "cuda:0"
+  _check_rows(gpu, oracle, mode, cfg["unary"].to(dev), cfg["context"].to(dev),
+              cfg["edge_weights"][:2].contiguous().to(dev), synthetic.upstream_grad(cfg).to(dev),
+              2, cfg["rho"], "full-size rows")
+
+
+@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
+def test_rows_of_the_largest_image_match_oracle(gpu, oracle, mode):
+  """2684 x 2000 pixels of 200 labels: 4 294 400 000 bytes per plane, 567 232 below the largest
+  image the library accepts, so the vector offsets of the last rows use all 32 bits."""
+  import torch
+  H, W, L = 2684, 2000, 200
+  dev = "cuda:0"
+  g = torch.Generator(device=dev)
+  g.manual_seed(11)
+  unary = torch.rand(1, 1, H, W, L, device=dev, generator=g)
+  ew = 0.2 + torch.rand(2, 1, 1, H, W, device=dev, generator=g)
+  dcost = torch.randn(1, 1, H, W, L, device=dev, generator=g)
+  ctx = (0.25 * torch.clamp(torch.arange(L, dtype=torch.float32), max=3.0)).to(dev)
+  rho = 0.5 if mode == "TRWP" else 1.0
+  _check_rows(gpu, oracle, mode, unary, ctx, ew, dcost, 1, rho, "largest image rows")
 
 
 @pytest.mark.parametrize("mode,pair", [("TRWP", 2), ("ISGMR", 2), ("TRWP", 4), ("ISGMR", 6)])
