@@ -336,6 +336,24 @@ def test_rows_of_the_largest_image_match_oracle(gpu, oracle, mode):
   _check_rows(gpu, oracle, mode, unary, ctx, ew, dcost, 1, rho, "largest image rows")
 
 
+@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
+def test_rows_of_a_batch_beyond_2_31_elements(gpu, oracle, mode):
+  """Four 1500 x 2000 images of 192 labels: 2.304 G elements per plane, more than a 32-bit element
+  index holds (the scans address per batch item, the element-wise kernels over the whole plane)."""
+  import torch
+  B, H, W, L = 4, 1500, 2000, 192
+  dev = "cuda:0"
+  g = torch.Generator(device=dev)
+  g.manual_seed(12)
+  unary = torch.rand(B, 1, H, W, L, device=dev, generator=g)
+  ew = 0.2 + torch.rand(2, B, 1, H, W, device=dev, generator=g)
+  dcost = torch.randn(B, 1, H, W, L, device=dev, generator=g)
+  ctx = (0.25 * torch.clamp(torch.arange(L, dtype=torch.float32), max=4.0)).to(dev)
+  rho = 0.5 if mode == "TRWP" else 1.0
+  _check_rows(gpu, oracle, mode, unary, ctx, ew, dcost, 1, rho, "batch of four rows")
+  torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("mode,pair", [("TRWP", 2), ("ISGMR", 2), ("TRWP", 4), ("ISGMR", 6)])
 def test_full_size_chains_match_oracle(gpu, oracle, mode, pair):
   """Zero edge weights make a direction's messages vanish, so with every direction but one
