@@ -86,6 +86,9 @@ def parse():
                        "(default: the reference's operator contract, the step zero-fills `msg` "
                        "inside the timed region and the operators read it as initial messages; the "
                        "other contract is timed over the same number of steps and reported beside it)")
+  ap.add_argument("--no-fused-pairs", action="store_true",
+                  help="TRWP: one launch per direction even for launches of at most 1024 chains "
+                       "(MPL_F_FUSED_PAIRS_OFF)")
   ap.add_argument("--dunary-only", action="store_true",
                   help="backward without dcontext and dedge_weights (a fixed pairwise table and "
                        "edge weights that are not learned); not the headline workload")
@@ -332,6 +335,7 @@ def main():
     imin = inorm = empty
 
   uninit = bool(a.msg_uninit)
+  trwp_flags = _lib.F_FUSED_PAIRS_OFF if a.no_fused_pairs else 0
   if training and a.dunary_only:
     dedge = dctx = torch.empty(0, **f32)
 
@@ -353,10 +357,10 @@ def main():
                                                   dunary, dctx, dedge, dmsg, dscratch)
       elif alg == "TRWP":
         lib_stereo.TRWP.forward(rho, n_iter, 0, unary, context, edge, msg, cost, imin, inorm,
-                                belief, empty, msg_uninit=uninit)
+                                belief, empty, msg_uninit=uninit, flags=trwp_flags)
         if training:
           lib_stereo.TRWP.backward(rho, context, edge, dcost, imin, inorm, dunary, dctx, dedge,
-                                   dmsg, dscratch)
+                                   dmsg, dscratch, flags=trwp_flags)
       else:
         lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, context, edge, msg, cost, imin, inorm,
                                  belief, msg_tmp, empty, msg_uninit=uninit)

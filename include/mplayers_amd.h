@@ -64,7 +64,10 @@ typedef struct mpl_shape {
  * (entry 0 of a 1-D table, the diagonal of a 2-D one), as the hard operator of the reference's
  * TRWP_hard_soft build does (MPLayers/TRWP_hard_soft/TRWP_backward.cu:104-111, 188-195, 258-265);
  * the TRWP and ISGMR builds skip them (MPLayers/TRWP/TRWP_backward.cu:111-112). */
-#define MPL_F_ALL 0x1fu
+#define MPL_F_FUSED_PAIRS_OFF 0x20u
+/* TRWP calls: one launch per direction even where a launch has so few chains (at most 1024) that
+ * the library would run both sweeps of a pair of opposite directions in one. */
+#define MPL_F_ALL 0x3fu
 
 /* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.
  * msg: initial messages in, final normalised messages out.  msg_min_index/msg_norm_index NULL =>

@@ -28,6 +28,7 @@ F_PACKED_OFF = 0x02
 F_PACKED_ALWAYS = 0x04
 F_FUSED_U_OFF = 0x08
 F_DCONTEXT_SAME_LABEL = 0x10
+F_FUSED_PAIRS_OFF = 0x20
 
 
 class KernelStat(ctypes.Structure):

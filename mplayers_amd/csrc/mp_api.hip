@@ -442,6 +442,7 @@ thread_local char g_err[512] = "";
 // was called): lets a benchmark read each kernel's average duration without an external profiler.
 struct ProfRec {
   int kind;
+  int sweeps;  // direction sweeps the launch stands for (2 for a fused pair)
   hipEvent_t start, stop;
 };
 struct Profiler {
@@ -465,11 +466,12 @@ std::mutex g_prof_mu;
 struct Timed {
   hipStream_t st;
   hipEvent_t stop = nullptr;
-  Timed(int kind, hipStream_t s) : st(s) {
+  Timed(int kind, hipStream_t s, int sweeps = 1) : st(s) {
     if (!g_prof.on) return;
     std::lock_guard<std::mutex> lk(g_prof_mu);
     ProfRec r;
     r.kind = kind;
+    r.sweeps = sweeps;
     r.start = g_prof.get_event();
     r.stop = g_prof.get_event();
     if (r.start == nullptr || r.stop == nullptr) return;
@@ -564,6 +566,7 @@ std::atomic<int> g_fused_u{1};       // MPL_OPT_FUSED_U
 struct CallOpts {
   int packed;   // 0 off, 1 by chain count, 2 always
   bool fused_u;
+  bool fused_pairs;
 };
 
 int read_flags(unsigned flags, const char* what, CallOpts* o) {
@@ -573,12 +576,17 @@ int read_flags(unsigned flags, const char* what, CallOpts* o) {
   o->packed = (flags & MPL_F_PACKED_OFF) ? 0
               : (flags & MPL_F_PACKED_ALWAYS) ? 2 : g_packed_scans.load(std::memory_order_relaxed);
   o->fused_u = (flags & MPL_F_FUSED_U_OFF) ? false : g_fused_u.load(std::memory_order_relaxed) != 0;
+  o->fused_pairs = (flags & MPL_F_FUSED_PAIRS_OFF) == 0;
   return MPL_OK;
 }
 
+// TRWP launches with at most this many chains (one wavefront each: at most one per SIMD) run both
+// sweeps of a pair of opposite directions in one launch
+constexpr int kFusedPairMaxChains = 1024;
+
 void launch_fwd(const SweepParams& p, bool train, bool jacobi, const CallOpts& o, hipStream_t st) {
-  Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st);
-  if (o.packed && launch_packed_fwd(p, train, jacobi, o.packed == 2, st)) return;
+  Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st, p.fused_pair ? 2 : 1);
+  if (!p.fused_pair && o.packed && launch_packed_fwd(p, train, jacobi, o.packed == 2, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_fwd<1>(p, train, jacobi, st); break;
     case 2: launch_sweep_fwd<2>(p, train, jacobi, st); break;
@@ -588,8 +596,8 @@ void launch_fwd(const SweepParams& p, bool train, bool jacobi, const CallOpts& o
 }
 
 void launch_bwd(const BackParams& p, bool jacobi, const CallOpts& o, hipStream_t st) {
-  Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st);
-  if (o.packed && launch_packed_bwd(p, jacobi, o.packed == 2, st)) return;
+  Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st, p.fused_pair ? 2 : 1);
+  if (!p.fused_pair && o.packed && launch_packed_bwd(p, jacobi, o.packed == 2, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_bwd<1>(p, jacobi, st); break;
     case 2: launch_sweep_bwd<2>(p, jacobi, st); break;
@@ -700,7 +708,7 @@ int mpl_profile_end(mpl_kernel_stat* stats, int n_stats) {
     if (e != hipSuccess) {
       rc = fail(MPL_ELAUNCH, "profile_end: %s", hipGetErrorString(e));
     } else if (r.kind >= 0 && r.kind < n_stats) {
-      stats[r.kind].launches += 1;
+      stats[r.kind].launches += r.sweeps;
       stats[r.kind].total_ms += ms;
     }
     g_prof.pool.push_back(r.start);
@@ -772,13 +780,21 @@ int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
       p.pair_q = 1;
       p.belief = (uninit && it == 0 && d <= 1) ? unary : unary_update;
       p.zero_start = (uninit && it == 0) ? 1 : 0;
-      p.skip_s_store = ((it == n_iter - 1) && (d == s->n_dir - 1)) ||  // cost_final is re-summed
-                       (uninit && it == 0 && d == 0);
+      auto skip_s = [&](int dd) {
+        return (((it == n_iter - 1) && (dd == s->n_dir - 1)) ||  // cost_final is re-summed
+                (uninit && it == 0 && dd == 0)) ? 1 : 0;
+      };
+      p.skip_s_store = skip_s(d);
+      // few chains: the wavefront of a chain sweeps d and then d + 1 (the same pixels in reverse)
+      p.fused_pair = (opts.fused_pairs && opts.packed != 2 && !(d & 1) &&
+                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+      p.skip_s_store2 = skip_s(d + 1);
       if (train) {
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
         p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       }
       launch_fwd(p, train, false, opts, st);
+      if (p.fused_pair) ++d;
     }
     if (label_all) {
       Timed timed(MPL_KERNEL_LABEL, st);
@@ -926,8 +942,13 @@ int mpl_trwp_backward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
       p.skip_hi_store = (!(d & 1) && it == 0) ? 1 : 0;
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
+      // few chains: the wavefront of a chain walks d (odd) and then d - 1 (same pixels, reversed)
+      p.fused_pair = (opts.fused_pairs && opts.packed != 2 && (d & 1) &&
+                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+      p.skip_h2 = (it == 0) ? 1 : 0;
       launch_bwd(p, false, opts, st);
       first = false;
+      if (p.fused_pair) --d;
     }
   }
   return launch_ok("trwp_backward");

@@ -76,9 +76,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const int lane = threadIdx.x;
   const int64_t P = (int64_t)p.B * p.H * p.W;
   const int64_t N = P * L;
-  const ChainCtx ch = locate_chain(p);
-  const int dir = ch.dir;
-  const int n = ch.n;
+  const ChainCtx ch0 = locate_chain(p);
+  const int n = ch0.n;
 
   const bool same = DC && p.same_label != 0;
   for (int i = lane; i < n_ctx; i += kWave) {
@@ -104,15 +103,49 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     near_max = kb - 1 < 1 ? 1 : (kb - 1 > kNear ? kNear : kb - 1);
   }
 
+  const int lab0 = R * lane;
+  bool valid[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) valid[j] = MASK ? (lab0 + j < L) : true;
+  float hist_reg[R];        // dcontext[label] partial sums of this lane's own labels (1-D context)
+  float near_acc[kNear + 1];  // dcontext[k] partial sums for k <= kNear (1-D context)
+#pragma unroll
+  for (int j = 0; j < R; ++j) hist_reg[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k <= kNear; ++k) near_acc[k] = 0.f;
+
+  // Gauss-Seidel, chain-starved launches (p.fused_pair): the wavefront walks its chain for the odd
+  // direction and then, over the same pixels in reverse, for the even one, which the next launch
+  // would otherwise do; what the first walk stored is read back by the same wavefront in program
+  // order, and dcontext is collected over both walks and flushed once.
+  const int halves = (!JACOBI && p.fused_pair) ? 2 : 1;
+#pragma clang loop unroll(disable)
+  for (int half = 0; half < halves; ++half) {
+  ChainCtx ch = ch0;
+  bool first_touch = p.first_touch != 0, inv_a = p.inv_from_a != 0;
+  bool skip_hd_store = p.skip_hd_store != 0, skip_hi_store = p.skip_hi_store != 0;
+  const float* a_in = p.a_in;
+  if (half) {
+    ch.dir = ch0.dir ^ 1;
+    ch.pix0 = ch0.pix0 + (n - 1) * ch0.pstep;
+    ch.pstep = -ch0.pstep;
+    first_touch = false;
+    inv_a = true;  // the walk before this one swept the opposite direction
+    skip_hd_store = skip_hi_store = p.skip_h2 != 0;
+    a_in = p.a_out;
+    wait_vmem<0>();
+    __syncthreads();
+  }
+  const int dir = ch.dir;
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t img_p = (int64_t)ch.bv * HW;  // first pixel of this batch item
   const int64_t img_e = img_p * L;
   const int vbytes = L * 4;
-  const bool read_h = !JACOBI && !p.first_touch;
-  const bool inv_from_a = !JACOBI && p.inv_from_a;
+  const bool read_h = !JACOBI && !first_touch;
+  const bool inv_from_a = !JACOBI && inv_a;
   // plane bases of this batch item and direction; label-vector descriptors are formed per access
   const float* __restrict__ bA =
-      (JACOBI ? p.gu_in + (int64_t)(p.gu_pair_share ? (dir & ~1) : dir) * p.gu_stride : p.a_in) +
+      (JACOBI ? p.gu_in + (int64_t)(p.gu_pair_share ? (dir & ~1) : dir) * p.gu_stride : a_in) +
       img_e;
   float* __restrict__ bAo = (JACOBI ? p.du_out + (int64_t)dir * N : p.a_out) + img_e;
   float* hbase = JACOBI ? p.du_out : p.h;  // Jacobi never touches these two planes
@@ -124,12 +157,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const rsrc_t dW = make_rsrc(p.edge + (int64_t)dir * P + img_p, img_bytes_p);
   const rsrc_t dDe = make_rsrc(DE ? p.dedge + (int64_t)dir * P + img_p : nullptr, DE ? img_bytes_p : 0);
   const float rho = p.rho;
-  const int lab0 = R * lane;
   const int foff = lab0 * 4;
-
-  bool valid[R];
-#pragma unroll
-  for (int j = 0; j < R; ++j) valid[j] = MASK ? (lab0 + j < L) : true;
 
   // VEC: one descriptor per plane for the whole kernel, covering the batch item's image; a lane
   // reaches its labels of a pixel through its vector offset, a lane without labels (or a step that
@@ -142,8 +170,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   const rsrc_t rAo = make_rsrc(bAo, img_bytes);
   const rsrc_t rHdIn = make_rsrc(bHd, (!JACOBI && read_h) ? img_bytes : 0);
   const rsrc_t rHiIn = make_rsrc(bHi, (!JACOBI && read_h && !inv_from_a) ? img_bytes : 0);
-  const rsrc_t rHdOut = make_rsrc(bHd, (JACOBI || p.skip_hd_store) ? 0 : img_bytes);
-  const rsrc_t rHiOut = make_rsrc(bHi, (JACOBI || p.skip_hi_store) ? 0 : img_bytes);
+  const rsrc_t rHdOut = make_rsrc(bHd, (JACOBI || skip_hd_store) ? 0 : img_bytes);
+  const rsrc_t rHiOut = make_rsrc(bHi, (JACOBI || skip_hi_store) ? 0 : img_bytes);
   const rsrc_t rImin = make_rsrc(bImin, (int)(HW * L));
   // loads run from the last pixel of the chain down to the first; past it the first is refetched
   // (VEC: the prefetch simply runs on; what lies there is another pixel or reads as 0)
@@ -210,12 +238,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   }
 
   float sc[R];  // dU of the current pixel: what the previous step scattered into it
-  float hist_reg[R];        // dcontext[label] partial sums of this lane's own labels (1-D context)
-  float near_acc[kNear + 1];  // dcontext[k] partial sums for k <= kNear (1-D context)
 #pragma unroll
-  for (int j = 0; j < R; ++j) sc[j] = hist_reg[j] = 0.f;
-#pragma unroll
-  for (int k = 0; k <= kNear; ++k) near_acc[k] = 0.f;
+  for (int j = 0; j < R; ++j) sc[j] = 0.f;
   const int last_lane = (L - 1) / R, last_reg = (L - 1) % R;
 
   int st_p = ch.pix0 + (n - 1) * ch.pstep;
@@ -413,8 +437,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           buf_store<R, true>(rHiOut, vo, 0u, hin);
         } else {
           buf_store<R, VEC>(make_rsrc(bAo, nrec), foff, so, an);
-          buf_store<R, VEC>(make_rsrc(bHd, p.skip_hd_store ? 0 : nrec), foff, so, hdn);
-          buf_store<R, VEC>(make_rsrc(bHi, p.skip_hi_store ? 0 : nrec), foff, so, hin);
+          buf_store<R, VEC>(make_rsrc(bHd, skip_hd_store ? 0 : nrec), foff, so, hdn);
+          buf_store<R, VEC>(make_rsrc(bHi, skip_hi_store ? 0 : nrec), foff, so, hin);
         }
       }
       // each pixel receives over exactly one edge per direction: plain read-modify-write
@@ -443,6 +467,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
       step(px, n - 1 - (s0 + D + u));
     }
   }
+  }  // both walks of a fused pair
   if (!DC) return;
   __syncthreads();
   if (small_l) {

@@ -458,6 +458,8 @@ struct SweepParams {
   int pack;                        // packed scans (mp_pack.hip): chains per wavefront
   int pair_q;                      // Gauss-Seidel: belief plane holds Q between the sweeps of a pair
   int skip_s_store;                // Gauss-Seidel: last sweep of the call, nobody reads S after it
+  int fused_pair;                  // Gauss-Seidel: every wavefront sweeps dirs[0], then dirs[0] ^ 1
+  int skip_s_store2;               // skip_s_store of that second sweep
   int first_iter;                  // Gauss-Seidel: first iteration (planes not yet swept hold the
                                    // caller's initial messages, which need not be read when zero)
   int u_pair_share;                // Jacobi: directions d and d^1 read the U plane of the even one
@@ -485,6 +487,8 @@ struct BackParams {
   int inv_from_a;           // h_inv == -A (the previous launch swept the opposite direction)
   int skip_hd_store;        // h_dir is not read again before it is overwritten (or ever)
   int skip_hi_store;        // h_inv is never read again (last sweeps of the backward pass)
+  int fused_pair;           // Gauss-Seidel: every wavefront walks dirs[0] (odd), then dirs[0] ^ 1
+  int skip_h2;              // that second walk stores neither h plane (last iteration walked)
   // ISGMR: gu_in planes (plane stride gu_stride; 0 on the first iteration where gu_k = dcost_final),
   // du_out (n_dir_total, N) receives dU_d in place of gu_d
   const float* gu_in;

@@ -320,7 +320,8 @@ __device__ __forceinline__ void linear_step(const float (&a)[R], float w, float 
 // VEC: L % R == 0 (vector accesses).  MASK: some lanes own labels >= L.
 template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI, int KT>
 __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
-                                              const ChainCtx& ch, float* a_s, const float* ctx_s) {
+                                              const ChainCtx& ch, float* a_s, const float* ctx_s,
+                                              const bool skip_s_store) {
   const int L = p.L;
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t P = (int64_t)p.B * HW;
@@ -400,7 +401,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   const rsrc_t rMd = make_rsrc(bMd, (md_zero || pair_second) ? 0 : img_bytes);
   const rsrc_t rMi = make_rsrc(bMi, mi_zero ? 0 : img_bytes);
   const rsrc_t rMo = make_rsrc(bMo, img_bytes);
-  const rsrc_t rSo = make_rsrc(bSo, (JACOBI || p.skip_s_store) ? 0 : img_bytes);
+  const rsrc_t rSo = make_rsrc(bSo, (JACOBI || skip_s_store) ? 0 : img_bytes);
   const rsrc_t rImin = make_rsrc(bImin, TRAIN ? (int)(HW * L) : 0);
   // loads of the next pixel; past the end of the chain the last pixel is fetched again
   const int last_p = ch.pix0 + (n - 1) * ch.pstep;
@@ -463,7 +464,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     }
     const unsigned so0 = (unsigned)ch.pix0 * (unsigned)vbytes;
     const int vo0 = (int)(lane_ok ? so0 + (unsigned)foff : kDeadWide);
-    if (!JACOBI && p.pair_q && !p.skip_s_store) {
+    if (!JACOBI && p.pair_q && !skip_s_store) {
       if constexpr (VEC)
         buf_store<R, true>(rSo, vo0, 0u, conv);
       else
@@ -603,7 +604,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       } else {
         const int nrec = live ? (int)(so + (unsigned)vbytes) : 0;
         buf_store<R, VEC>(make_rsrc(bMo, nrec), foff, so, m);
-        if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, p.skip_s_store ? 0 : nrec), foff, so, sn);
+        if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, skip_s_store ? 0 : nrec), foff, so, sn);
         if (TRAIN)
           buf_store_u8<R, VEC>(make_rsrc(bImin, live ? (int)(sob + (unsigned)L) : 0), lab0, sob, fd_idx);
       }
@@ -672,38 +673,56 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
   }
   __syncthreads();
 
-  // wide truncated-linear contexts: two label scans instead of 2K-1 taps or the dense scan
-  if (desc.linear && !p.ctx2d && (desc.band_k == 0 || desc.band_k > 4)) {
-    run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -2>(p, desc, ch, a_s, ctx_s);
-    return;
-  }
-  switch (desc.band_k) {
-    case 0:
-      if (R == 1 && L == 21)
-        run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, (R == 1 ? -21 : -1)>(p, desc, ch, a_s, ctx_s);
-      else
-        run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -1>(p, desc, ch, a_s, ctx_s);
-      break;
-    case 2: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 2>(p, desc, ch, a_s, ctx_s); break;
-    case 3: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 3>(p, desc, ch, a_s, ctx_s); break;
-    case 4: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 4>(p, desc, ch, a_s, ctx_s); break;
-    default:
-      // wider bands with the taps in registers: the table is constant from band_k on, so the
-      // taps between band_k and the compiled width are the dense scan's own candidates
-      // (only with several labels per lane: the short chains of small label counts gain nothing
-      // and pay for the larger kernel)
-      if constexpr (R >= 2) {
-        if (desc.band_k <= 8) {
-          run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 8>(p, desc, ch, a_s, ctx_s);
-          break;
+  // Gauss-Seidel, chain-starved launches: the sweep of the opposite direction visits the same
+  // pixels in reverse and depends on nothing but this chain's own first sweep, so the wavefront
+  // runs it right away (p.fused_pair) instead of a second launch doing so.  What the first sweep
+  // stored is read back by the same wavefront, in program order.
+  const int halves = (!JACOBI && p.fused_pair) ? 2 : 1;
+#pragma clang loop unroll(disable)
+  for (int half = 0; half < halves; ++half) {
+    ChainCtx c = ch;
+    bool skip_s = p.skip_s_store != 0;
+    if (half) {
+      c.dir = ch.dir ^ 1;
+      c.pix0 = ch.pix0 + (ch.n - 1) * ch.pstep;
+      c.pstep = -ch.pstep;
+      skip_s = p.skip_s_store2 != 0;
+      wait_vmem<0>();
+      __syncthreads();
+    }
+    // wide truncated-linear contexts: two label scans instead of 2K-1 taps or the dense scan
+    if (desc.linear && !p.ctx2d && (desc.band_k == 0 || desc.band_k > 4)) {
+      run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -2>(p, desc, c, a_s, ctx_s, skip_s);
+      continue;
+    }
+    switch (desc.band_k) {
+      case 0:
+        if (R == 1 && L == 21)
+          run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, (R == 1 ? -21 : -1)>(p, desc, c, a_s, ctx_s, skip_s);
+        else
+          run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -1>(p, desc, c, a_s, ctx_s, skip_s);
+        break;
+      case 2: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 2>(p, desc, c, a_s, ctx_s, skip_s); break;
+      case 3: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 3>(p, desc, c, a_s, ctx_s, skip_s); break;
+      case 4: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 4>(p, desc, c, a_s, ctx_s, skip_s); break;
+      default:
+        // wider bands with the taps in registers: the table is constant from band_k on, so the
+        // taps between band_k and the compiled width are the dense scan's own candidates
+        // (only with several labels per lane: the short chains of small label counts gain nothing
+        // and pay for the larger kernel)
+        if constexpr (R >= 2) {
+          if (desc.band_k <= 8) {
+            run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 8>(p, desc, c, a_s, ctx_s, skip_s);
+            break;
+          }
+          if (desc.band_k <= 16) {
+            run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 16>(p, desc, c, a_s, ctx_s, skip_s);
+            break;
+          }
         }
-        if (desc.band_k <= 16) {
-          run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 16>(p, desc, ch, a_s, ctx_s);
-          break;
-        }
-      }
-      run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0>(p, desc, ch, a_s, ctx_s);
-      break;
+        run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0>(p, desc, c, a_s, ctx_s, skip_s);
+        break;
+    }
   }
 }
 
