@@ -1052,8 +1052,12 @@ int mpl_trwp_soft_forward(const mpl_shape* s, unsigned flags, float rho, int n_i
         p.edge_label = msg_edge_label + (int64_t)it * s->n_dir * N * s->n_disp;
         p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       }
-      Timed timed(MPL_KERNEL_FWD_SWEEP, st);
+      // few chains of at most 32 labels: the wavefront of a chain sweeps d and then d + 1
+      p.fused_pair = (opts.fused_pairs && s->n_disp <= 32 &&
+                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+      Timed timed(MPL_KERNEL_FWD_SWEEP, st, p.fused_pair ? 2 : 1);
       launch_soft_fwd(p, train, st);
+      if (p.fused_pair) ++d;
     }
     if (label_all) {
       Timed timed(MPL_KERNEL_LABEL, st);
@@ -1107,9 +1111,13 @@ int mpl_trwp_soft_backward(const mpl_shape* s, unsigned flags, float rho, int n_
       p.first_touch = (it == n_iter - 1) && (d & 1);
       p.edge_label = msg_edge_label + (int64_t)it * s->n_dir * N * s->n_disp;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
-      Timed timed(MPL_KERNEL_BWD_SWEEP, st);
+      // few chains of at most 32 labels: the wavefront of a chain walks d (odd) and then d - 1
+      p.fused_pair = (opts.fused_pairs && s->n_disp <= 32 &&
+                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+      Timed timed(MPL_KERNEL_BWD_SWEEP, st, p.fused_pair ? 2 : 1);
       launch_soft_bwd(p, st);
       first = false;
+      if (p.fused_pair) --d;
     }
   }
   return launch_ok("trwp_soft_backward");

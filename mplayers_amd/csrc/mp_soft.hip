@@ -477,11 +477,24 @@ __global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams
   float* tile = smem;              // 256 * NT4 floats (training): the pixel's block as it is stored
   float* tab = smem + (TRAIN ? 256 * NT4 : 0);  // LL floats
   const int lane = threadIdx.x;
-  const ChainCtx ch = locate_chain(p);
-  if (ch.n < 2) return;  // nothing to write
+  const ChainCtx ch0 = locate_chain(p);
+  if (ch0.n < 2) return;  // nothing to write
   fill_table(p.ctx, L, p.ctx2d, lane, tab);
   __syncthreads();
 
+  // chain-starved launches (p.fused_pair): the wavefront sweeps its chain for dirs[0] and then, over
+  // the same pixels in reverse, for the opposite direction, reading back what it stored
+  const int halves = p.fused_pair ? 2 : 1;
+#pragma clang loop unroll(disable)
+  for (int half = 0; half < halves; ++half) {
+  ChainCtx ch = ch0;
+  if (half) {
+    ch.dir = ch0.dir ^ 1;
+    ch.pix0 = ch0.pix0 + (ch0.n - 1) * ch0.pstep;
+    ch.pstep = -ch0.pstep;
+    wait_vmem<0>();
+    __syncthreads();
+  }
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t P = (int64_t)p.B * HW;
   const int64_t N = P * L;
@@ -652,6 +665,7 @@ __global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams
       step(px, t0 + D + u);
     }
   }
+  }  // both sweeps of a fused pair
 }
 
 // NQ: float4 reads that cover a row of the gradient block (4 * NQ >= L).  The duals come straight
@@ -670,21 +684,41 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t P = (int64_t)p.B * HW;
   const int64_t N = P * L;
-  const ChainCtx ch = locate_chain(p);
-  const int dir = ch.dir;
-  const int n = ch.n;
+  const ChainCtx ch0 = locate_chain(p);
+  const int n = ch0.n;
 
   fill_table(p.ctx, L, p.ctx2d, lane, tab);
   for (int i = lane; i < LL; i += kWave) hist[i] = 0.f;
   for (int i = lane; i < L * S; i += kWave) grad[i] = 0.f;
   __syncthreads();
 
+  float hreg[FM];  // dcontext partial sums of this lane's (cd, fd) pairs, over both walks of a pair
+#pragma unroll
+  for (int i = 0; i < FM; ++i) hreg[i] = 0.f;
+  // chain-starved launches (p.fused_pair): the odd direction's walk, then the even one's over the
+  // same pixels in reverse
+  const int halves = p.fused_pair ? 2 : 1;
+#pragma clang loop unroll(disable)
+  for (int half = 0; half < halves; ++half) {
+  ChainCtx ch = ch0;
+  bool first_touch = p.first_touch != 0;
+  const float* a_in = p.a_in;
+  if (half) {
+    ch.dir = ch0.dir ^ 1;
+    ch.pix0 = ch0.pix0 + (n - 1) * ch0.pstep;
+    ch.pstep = -ch0.pstep;
+    first_touch = false;
+    a_in = p.a_out;
+    wait_vmem<0>();
+    __syncthreads();
+  }
+  const int dir = ch.dir;
   const int64_t img_p = (int64_t)ch.bv * HW;
   const int64_t img_e = img_p * L;
   const int vbytes = L * 4;
-  const bool read_h = !p.first_touch;
+  const bool read_h = !first_touch;
   const int img_bytes = (int)(unsigned)(HW * L * 4);
-  const rsrc_t rA = make_rsrc(p.a_in + img_e, img_bytes);
+  const rsrc_t rA = make_rsrc(a_in + img_e, img_bytes);
   const rsrc_t rAo = make_rsrc(p.a_out + img_e, img_bytes);
   float* const bHd = p.h + (int64_t)dir * N + img_e;
   float* const bHi = p.h + (int64_t)(dir ^ 1) * N + img_e;
@@ -711,7 +745,7 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
 #pragma unroll
   for (int k = 0; k < G; ++k) addr[k] = (valid ? k * L + cd : lane) * 4;
   const int fd0 = g * F;
-  float tcol[FM], hreg[FM];
+  float tcol[FM];
   int boff[FM], gidx[FM];
   bool inr[FM];
 #pragma unroll
@@ -719,7 +753,6 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
     inr[i] = valid && i < F && fd0 + i < L;
     const int fd = inr[i] ? fd0 + i : L - 1;
     tcol[i] = tab[fd * L + cd];
-    hreg[i] = 0.f;
     // place of (cd, fd) inside the pixel's stored block
     boff[i] = inr[i] ? (even ? fd * L + cd : cd * L + fd) * 4 : kDeadOffset;
     gidx[i] = fd * S + cd;
@@ -841,10 +874,17 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
       step(px, n - 1 - (s0 + D + u));
     }
   }
+  }  // both walks of a fused pair
   if (p.dctx == nullptr) return;
+  {
+    const int F = (L + G - 1) / G;
+    const bool valid = lane < G * L;
+    const int g = valid ? lane / L : 0;
+    const int cd = valid ? lane - g * L : 0;
 #pragma unroll
-  for (int i = 0; i < FM; ++i)
-    if (inr[i]) hist[(fd0 + i) * L + cd] = hreg[i];
+    for (int i = 0; i < FM; ++i)
+      if (valid && i < F && g * F + i < L) hist[(g * F + i) * L + cd] = hreg[i];
+  }
   __syncthreads();
   // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D), the diagonal
   // included (TRWP_backward_soft.cu:116-126)

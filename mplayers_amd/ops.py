@@ -212,7 +212,7 @@ class TRWP_hard_soft(object):
 
   @staticmethod
   def forward_soft(rho, n_iter, unary, context, edge_weights, msg, msg_edge_label, msg_norm_index,
-                   cost_final, unary_update, label_all):
+                   cost_final, unary_update, label_all, flags=0):
     lib = _lib.load()
     shape, P, L, ctx2d = _Op._shape_from_msg(msg)
     N = P * L
@@ -229,7 +229,7 @@ class TRWP_hard_soft(object):
     if label_all.numel() > 0:
       _check("label_all", label_all, u8, n_iter * P)
     with torch.cuda.device(unary.device):
-      rc = lib.mpl_trwp_soft_forward(shape, 0, float(rho), int(n_iter), _ptr(unary), _ptr(context),
+      rc = lib.mpl_trwp_soft_forward(shape, int(flags), float(rho), int(n_iter), _ptr(unary), _ptr(context),
                                      _ptr(edge_weights), _ptr(msg), _ptr(msg_edge_label),
                                      _ptr(msg_norm_index), _ptr(cost_final), _ptr(unary_update),
                                      _ptr(label_all), _Op._stream(unary))
@@ -237,7 +237,7 @@ class TRWP_hard_soft(object):
 
   @staticmethod
   def backward_soft(rho, dcost_final, context, edge_weights, msg_edge_label, msg_norm_index,
-                    dunary, dcontext, dedge_weights, dmsg, dunary_update):
+                    dunary, dcontext, dedge_weights, dmsg, dunary_update, flags=0):
     lib = _lib.load()
     if msg_norm_index.dim() != 6:
       raise RuntimeError("msg_norm_index must be (n_iter, n_dir, batch, cv, h, w)")
@@ -260,7 +260,7 @@ class TRWP_hard_soft(object):
       _check("dedge_weights", dedge_weights, f32, n_dir * P)
     _check("dmsg", dmsg, f32, n_dir * N)
     with torch.cuda.device(dcost_final.device):
-      rc = lib.mpl_trwp_soft_backward(shape, 0, float(rho), int(n_iter), _ptr(dcost_final),
+      rc = lib.mpl_trwp_soft_backward(shape, int(flags), float(rho), int(n_iter), _ptr(dcost_final),
                                       _ptr(context), _ptr(edge_weights), _ptr(msg_edge_label),
                                       _ptr(msg_norm_index), _ptr(dunary), _ptr(dcontext),
                                       _ptr(dedge_weights), _ptr(dmsg), _ptr(dunary_update),

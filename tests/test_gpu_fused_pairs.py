@@ -93,3 +93,60 @@ def test_fused_pairs_are_bit_identical(gpu, L, n_dir, B, H, W, n_iter, rho, trai
     assert np.array_equal(a, b), (name, np.abs(a.astype(np.float64) - b).max())
   if dc_f is not None:  # float atomics across chains: equal up to their order
     assert np.abs(dc_f - dc_p).max() <= 1e-4 * max(1.0, np.abs(dc_p).max())
+
+
+SOFT_CASES = [
+    # L, n_dir, B, H, W, n_iter
+    (21, 4, 2, 17, 15, 2),    # three lane groups, 2-D context
+    (16, 8, 1, 9, 11, 2),     # four groups
+    (30, 4, 1, 6, 7, 1),      # two groups
+    (5, 16, 1, 7, 8, 2),
+    (3, 4, 1, 1, 9, 2),       # one row
+]
+
+
+@pytest.mark.parametrize("L,n_dir,B,H,W,n_iter", SOFT_CASES)
+@pytest.mark.parametrize("train", [True, False])
+def test_fused_pairs_soft_are_bit_identical(gpu, L, n_dir, B, H, W, n_iter, train):
+  """The soft-weighted scans of at most 32 labels fuse pairs the same way."""
+  import torch
+  from mplayers_amd import _lib, lib_stereo
+  g = torch.Generator().manual_seed(31 * L + n_dir)
+  dev = "cuda"
+  unary = torch.rand(B, 1, H, W, L, generator=g).to(dev)
+  context = (torch.rand(L, L, generator=g).triu() if L == 21 else torch.rand(L, generator=g)).to(dev)
+  edge = (0.2 + torch.rand(n_dir, B, 1, H, W, generator=g)).to(dev)
+  dcost = torch.randn(B, 1, H, W, L, generator=g).to(dev)
+  u8 = dict(dtype=torch.uint8, device=dev)
+  print("soft case", L, n_dir, B, H, W, n_iter, train, flush=True)
+
+  def run(flags):
+    msg = torch.zeros(n_dir, B, 1, H, W, L, device=dev)
+    cost = torch.zeros(B, 1, H, W, L, device=dev)
+    scratch = torch.zeros(B, 1, H, W, L, device=dev)
+    mel = torch.zeros(n_iter, n_dir, B, 1, H, W, L, L, device=dev) if train else torch.empty(0)
+    inorm = torch.zeros(n_iter, n_dir, B, 1, H, W, **u8) if train else torch.empty(0, dtype=torch.uint8)
+    label = torch.zeros(n_iter, B, 1, H, W, **u8)
+    lib_stereo.TRWP_hard_soft.forward_soft(rho, n_iter, unary, context, edge, msg, mel, inorm, cost,
+                                           scratch, label, flags=flags)
+    out = [msg, cost, label]
+    dctx = None
+    if train:
+      dunary = torch.zeros(B, 1, H, W, L, device=dev)
+      dctx = torch.zeros_like(context)
+      dedge = torch.zeros(n_dir, B, 1, H, W, device=dev)
+      dmsg = torch.full((n_dir, B, 1, H, W, L), float("nan"), device=dev)
+      lib_stereo.TRWP_hard_soft.backward_soft(rho, dcost, context, edge, mel, inorm, dunary, dctx,
+                                              dedge, dmsg, torch.empty(0, device=dev), flags=flags)
+      out += [mel, inorm, dunary, dedge]
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in out], (dctx.cpu().numpy() if dctx is not None else None)
+
+  rho = 0.5
+  fused, dc_f = run(0)
+  plain, dc_p = run(_lib.F_FUSED_PAIRS_OFF)
+  for i, (a, b) in enumerate(zip(fused, plain)):
+    assert not np.isnan(a.astype(np.float64)).any(), i
+    assert np.array_equal(a, b), (i, np.abs(a.astype(np.float64) - b).max())
+  if dc_f is not None:
+    assert np.abs(dc_f - dc_p).max() <= 1e-4 * max(1.0, np.abs(dc_p).max())
