@@ -274,8 +274,8 @@ const char* mpl_last_error(void);
  * one-chain-per-wavefront kernels, 2 packs whenever the label count allows it (the results agree
  * to the parity tolerance; 0 and 2 are meant for tests and comparisons). */
 #define MPL_OPT_PACKED_SCANS 0
-/* MPL_OPT_FUSED_U (default 1): ISGMR forward with 4 directions, rho == 1 and more than 32 labels
- * forms U inside the scans (unary + the old messages of the other pair of directions) instead of
+/* MPL_OPT_FUSED_U (default 1): ISGMR forward with 4 directions, rho == 1 and one chain per
+ * wavefront (more than 32 labels, or a launch the packed scans do not take) forms U inside the scans (unary + the old messages of the other pair of directions) instead of
  * storing it in a pass of its own; 0 always runs that pass (results agree to the parity tolerance,
  * bit for bit on inputs whose sums do not round). */
 #define MPL_OPT_FUSED_U 1

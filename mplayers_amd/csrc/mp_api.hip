@@ -843,9 +843,13 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
   // Four directions at rho = 1: U of a pair of opposite directions is the unary plus the two
   // messages of the other pair, so the scans can form it on the fly (3 planes read per direction
   // instead of 1) and the pass that stores U (5 planes in, 2 out per iteration) is dropped; with
-  // more directions the scans would read more than that pass moves.  (Not for the packed scans
-  // of small label counts.)
-  const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && s->n_disp > 32;
+  // more directions the scans would read more than that pass moves.  (Not where the packed scans
+  // of small label counts run: they are bound by the instructions of a step, and two more loads
+  // per step cost them more than the pass.)
+  const bool packed_runs =
+      opts.packed && packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp,
+                                            p.block_prefix[p.n_dirs], opts.packed == 2) >= 2;
+  const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && !packed_runs;
   if (msg_uninit && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {

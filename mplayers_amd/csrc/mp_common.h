@@ -522,6 +522,8 @@ void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 constexpr int kPackedMaxL = 32;
 constexpr int kPackedMinChains = 2048;  // two wavefronts per SIMD of the 256 CUs when unpacked
 // always: pack whatever the number of chains (tests and comparisons)
+// chains per wavefront the packed scans would use for such a launch (below 2: they do not apply)
+int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool always);
 bool launch_packed_fwd(const SweepParams& p, bool train, bool jacobi, bool always, hipStream_t st);
 bool launch_packed_bwd(const BackParams& p, bool jacobi, bool always, hipStream_t st);
 

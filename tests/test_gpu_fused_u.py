@@ -1,4 +1,5 @@
-"""ISGMR with four directions and more than 32 labels forms U inside the scans (no U pass).  The
+"""ISGMR with four directions at rho = 1 forms U inside the scans (no U pass) wherever one chain
+runs per wavefront (more than 32 labels, or fewer chains than the packed scans take).  The
 message buffers then alternate differently from the pass-based schedule, so every combination of
 iteration-count parity, cleared / declared-zero / non-zero initial messages and training /
 inference is checked against the oracle, and against the pass-based schedule of the library itself
@@ -26,9 +27,11 @@ def _case(L, n_iter, seed, H=7, W=9, B=2, n_dir=4):
 
 @pytest.mark.parametrize("train", [True, False])
 @pytest.mark.parametrize("n_iter", [1, 2, 3, 4])
-@pytest.mark.parametrize("L", [33, 96, 256])
+@pytest.mark.parametrize("L", [5, 16, 21, 33, 96, 256])
 def test_fused_u_matches_oracle(gpu, oracle, L, n_iter, train):
   unary, ctx, ew = _case(L, n_iter, seed=L + n_iter)
+  if L == 21:  # the operators take a 2-D table at 21 labels
+    ctx = np.triu(np.random.default_rng(L + n_iter).random((L, L))).astype(np.float32)
   ref = oracle.forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, saving_label=True, want_gaps=True)
   got = gpu.gpu_forward("ISGMR", unary, ctx, ew, 4, n_iter, 1.0, training=train, saving_label=True)
   belief = ref["cost_final"]
@@ -105,3 +108,4 @@ def test_fused_u_agrees_with_the_u_pass(gpu, n_iter):
   gpu.assert_values_close(got["msg"], want["msg"], what="msg", belief=want["cost_final"])
   gpu.assert_values_close(got["cost_final"], want["cost_final"], what="cost")
   assert (got["label_all"] != want["label_all"]).mean() < 0.01
+
