@@ -520,7 +520,7 @@ void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 // packed scans for small label counts (mp_pack.hip): several chains per wavefront.
 // The launchers return false, without launching, when the problem does not qualify.
 constexpr int kPackedMaxL = 32;
-constexpr int kPackedMinChains = 2048;  // two wavefronts per SIMD of the 256 CUs when unpacked
+constexpr int kPackedMinChains = 1025;  // more chains than the 256 CUs have SIMDs
 // always: pack whatever the number of chains (tests and comparisons)
 // chains per wavefront the packed scans would use for such a launch (below 2: they do not apply)
 int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool always);

@@ -20,54 +20,95 @@
 namespace mpl {
 namespace {
 
-__device__ __forceinline__ float bperm_f(int addr, float x) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(int, x)));
-}
-__device__ __forceinline__ int bperm_i(int addr, int x) { return __builtin_amdgcn_ds_bpermute(addr, x); }
-
-// A lane's place in its segment and the bpermute addresses of the shift-down tree.
+// Values shared inside a chain's segment of lanes go through LDS: every lane writes its value into
+// the slot of its label, and reads the whole segment back with 16-byte loads (all lanes of a segment
+// read the same addresses: broadcasts).  One write, one wait and a handful of wide reads replace the
+// lane-to-lane exchanges of a reduction tree (six dependent ds_bpermute round trips per reduction at
+// 21 labels) or of a loop over the segment's labels (one ds_bpermute per label).  A segment's slots
+// start on a 16-byte boundary (Lp = L rounded up to 4 floats); the slots past the last label keep
+// the identity of their buffer's operation; lanes without a chain write behind all segments.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+constexpr int kRedFloats = 192;  // floats per exchange buffer: G * Lp <= 112, 64 for idle lanes, pad
 struct Seg {
-  int l;         // label
-  int first;     // byte address (lane * 4) of the segment's first lane
-  int down[5];   // byte address of lane + 16, 8, 4, 2, 1 when that lane belongs to the segment, else own
-  bool has[5];
+  int l;      // label
+  int widx;   // where this lane writes
+  int rbase;  // first slot of this lane's segment
+  int nq;     // 16-byte reads per segment
 };
 
 __device__ __forceinline__ Seg make_seg(int lane, int L, int G) {
   Seg s;
   const int g = lane / L;
+  const int Lp = (L + 3) & ~3;
   s.l = lane - g * L;
   const bool in = g < G;
-  s.first = (in ? g * L : lane) * 4;
-#pragma unroll
-  for (int k = 0; k < 5; ++k) {
-    const int off = 16 >> k;
-    s.has[k] = in && (s.l + off < L);
-    s.down[k] = (s.has[k] ? lane + off : lane) * 4;
-  }
+  s.widx = in ? g * Lp + s.l : G * Lp + (lane - G * L);
+  s.rbase = in ? g * Lp : 0;
+  s.nq = Lp / 4;
   return s;
 }
 
-__device__ __forceinline__ float seg_min(const Seg& s, float x) {
-#pragma unroll
-  for (int k = 0; k < 5; ++k) x = fminf(x, bperm_f(s.down[k], x));
-  return bperm_f(s.first, x);
+// fills the slots past the last label of every segment with the buffer's identity
+__device__ __forceinline__ void seg_init(float* buf, float ident, int lane) {
+  for (int i = lane; i < kRedFloats; i += kWave) buf[i] = ident;
 }
-__device__ __forceinline__ int seg_max(const Seg& s, int x) {
+
+// NQ: compile-time bound of the reads per segment (exactly s.nq when the label count is a
+// template constant, 8 otherwise)
+template <int NQ, bool EXACT>
+__device__ __forceinline__ float seg_min(float* buf, const Seg& s, float x) {
+  buf[s.widx] = x;
+  const f32x4* q = reinterpret_cast<const f32x4*>(buf + s.rbase);
+  float m = INFINITY;
 #pragma unroll
-  for (int k = 0; k < 5; ++k) {
-    const int y = bperm_i(s.down[k], x);
-    x = y > x ? y : x;
+  for (int k = 0; k < NQ; ++k) {
+    if (!EXACT && k >= s.nq) break;
+    const f32x4 v = q[k];
+    m = fminf(m, fminf(fminf(v.x, v.y), fminf(v.z, v.w)));
   }
-  return bperm_i(s.first, x);
+  return m;
 }
-__device__ __forceinline__ float seg_sum(const Seg& s, float x) {
+template <int NQ, bool EXACT>
+__device__ __forceinline__ int seg_max(float* buf, const Seg& s, int x) {
+  buf[s.widx] = __builtin_bit_cast(float, x);
+  const i32x4* q = reinterpret_cast<const i32x4*>(buf + s.rbase);
+  int m = -1;
 #pragma unroll
-  for (int k = 0; k < 5; ++k) {
-    const float y = bperm_f(s.down[k], x);
-    x += s.has[k] ? y : 0.f;
+  for (int k = 0; k < NQ; ++k) {
+    if (!EXACT && k >= s.nq) break;
+    const i32x4 v = q[k];
+    const int a = v.x > v.y ? v.x : v.y, b = v.z > v.w ? v.z : v.w;
+    const int c = a > b ? a : b;
+    m = c > m ? c : m;
   }
-  return bperm_f(s.first, x);
+  return m;
+}
+template <int NQ, bool EXACT>
+__device__ __forceinline__ float seg_sum(float* buf, const Seg& s, float x) {
+  buf[s.widx] = x;
+  const f32x4* q = reinterpret_cast<const f32x4*>(buf + s.rbase);
+  float m = 0.f;
+#pragma unroll
+  for (int k = 0; k < NQ; ++k) {
+    if (!EXACT && k >= s.nq) break;
+    const f32x4 v = q[k];
+    m += (v.x + v.y) + (v.z + v.w);
+  }
+  return m;
+}
+// the values of all labels of the segment: out[c] = value of label c (c < 4 * NQ)
+template <int NQ>
+__device__ __forceinline__ void seg_all(float* buf, const Seg& s, float x, float (&out)[4 * NQ]) {
+  buf[s.widx] = x;
+  const f32x4* q = reinterpret_cast<const f32x4*>(buf + s.rbase);
+#pragma unroll
+  for (int k = 0; k < NQ; ++k) {
+    const f32x4 v = q[k];
+    out[4 * k] = v.x;
+    out[4 * k + 1] = v.y;
+    out[4 * k + 2] = v.z;
+    out[4 * k + 3] = v.w;
+  }
 }
 
 // full symmetric context table tab[fd * L + cd] = ctx(cd, fd), TRWP_forward.cu:101-113
@@ -128,12 +169,20 @@ struct PixPF {
 template <bool TRAIN, bool JACOBI, int LT>
 __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) {
   extern __shared__ float smem[];
-  float* tab = smem;  // L * L
+  float* xa = smem;                  // exchange buffers (see Seg): beliefs a,
+  float* xm = xa + kRedFloats;       // normalisation minimum,
+  float* xi = xm + kRedFloats;       // its label
+  float* tab = xi + kRedFloats;      // L * L
   const int L = LT > 0 ? LT : p.L;
   const int G = p.pack;
   const int lane = threadIdx.x;
   const PackedChains ch = locate_packed(p, lane, L, G);
   const Seg sg = make_seg(lane, L, G);
+  constexpr int NQ = LT > 0 ? (LT + 3) / 4 : 8;
+  constexpr bool EXACT = LT > 0;
+  seg_init(xa, 0.f, lane);
+  seg_init(xm, INFINITY, lane);
+  seg_init(xi, __builtin_bit_cast(float, -1), lane);
   fill_table(p.ctx, L, p.ctx2d, lane, tab);
   __syncthreads();
   if (!JACOBI && !p.pair_q && ch.n_max < 2) return;
@@ -231,9 +280,11 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
       float best = inf;
       int arg = L - 1;
       if constexpr (LT > 0) {
+        float av[4 * NQ];  // a of every label of this lane's chain
+        seg_all<NQ>(xa, sg, a, av);
 #pragma unroll
         for (int fd = LT - 1; fd >= 0; --fd) {
-          const float val = fmaf(w, tcol[fd], bperm_f(sg.first + fd * 4, a));
+          const float val = fmaf(w, tcol[fd], av[fd]);
           if (TRAIN) {
             const bool take = (fd == LT - 1) || (val < best);
             best = take ? val : best;
@@ -243,9 +294,10 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
           }
         }
       } else {
+        xa[sg.widx] = a;
 #pragma unroll 4
         for (int fd = L - 1; fd >= 0; --fd) {
-          const float val = fmaf(w, tab[fd * L + l], bperm_f(sg.first + fd * 4, a));
+          const float val = fmaf(w, tab[fd * L + l], xa[sg.rbase + fd]);
           if (TRAIN) {
             const bool take = (fd == L - 1) || (val < best);
             best = take ? val : best;
@@ -255,7 +307,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
           }
         }
       }
-      const float nmin = seg_min(sg, on ? best : inf);  // MsgNormNaive, commonCUDA.cuh:92-129
+      const float nmin = seg_min<NQ, EXACT>(xm, sg, on ? best : inf);  // MsgNormNaive, commonCUDA.cuh:92-129
       const float m = best - nmin;
       prev = on ? m : 0.f;
       uf = un;
@@ -265,7 +317,7 @@ __global__ void __launch_bounds__(kWave) packed_fwd_kernel(const SweepParams p) 
       if (TRAIN) {
         __builtin_amdgcn_raw_buffer_store_b8((unsigned char)arg, dImin,
                                              live ? st_pix * L + l : kDeadOffset, 0, MPL_ST_AUX);
-        const int nidx = seg_max(sg, (on && best == nmin) ? l : -1);  // largest label on ties
+        const int nidx = seg_max<NQ, EXACT>(xi, sg, (on && best == nmin) ? l : -1);  // largest label on ties
         __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm,
                                              (live && l == 0) ? st_pix : kDeadOffset, 0, 0);
       }
@@ -287,11 +339,21 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
   extern __shared__ float smem[];
   const int L = LT > 0 ? LT : p.L;
   const int G = p.pack;
-  float* tab = smem;           // L * L
-  float* pairs = smem + L * L; // G tables of L * L: dcontext per (cd, fd) pair and chain slot
+  float* xg = smem;                  // exchange buffers (see Seg): gradients g,
+  float* xf = xg + kRedFloats;       // argmin labels,
+  float* xs = xf + kRedFloats;       // the two sums
+  float* xd = xs + kRedFloats;
+  float* tab = xd + kRedFloats;      // L * L
+  float* pairs = tab + L * L;        // G tables of L * L: dcontext per (cd, fd) pair and chain slot
   const int lane = threadIdx.x;
   const PackedChains ch = locate_packed(p, lane, L, G);
   const Seg sg = make_seg(lane, L, G);
+  constexpr int NQ = LT > 0 ? (LT + 3) / 4 : 8;
+  constexpr bool EXACT = LT > 0;
+  seg_init(xg, 0.f, lane);
+  seg_init(xf, __builtin_bit_cast(float, -1), lane);
+  seg_init(xs, 0.f, lane);
+  seg_init(xd, 0.f, lane);
   if (DE) fill_table(p.ctx, L, p.ctx2d, lane, tab);
   if (DC)
     for (int i = lane; i < G * L * L; i += kWave) pairs[i] = 0.f;
@@ -373,23 +435,24 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
       // gradient w.r.t. the normalised message of this pixel (none at the chain start, t == 0)
       const bool edge = on && t >= 1;
       float g = edge ? fmaf(rho, sc, JACOBI ? px.a : px.a + px.hd) : 0.f;
-      const float tot = seg_sum(sg, g);  // MsgNormNaiveBack, commonCUDA.cuh:131-145
+      const float tot = seg_sum<NQ, EXACT>(xs, sg, g);  // MsgNormNaiveBack, commonCUDA.cuh:131-145
       if (edge && l == px.nidx) g -= tot;
       const int fd = px.fd;
       // dU[q, f] = sum of g[c] over the labels c of this chain whose argmin is f
       float scn = 0.f;
       if constexpr (LT > 0) {
+        float gv[4 * NQ], fv[4 * NQ];  // gradient and argmin label of every label of the chain
+        seg_all<NQ>(xg, sg, g, gv);
+        seg_all<NQ>(xf, sg, __builtin_bit_cast(float, fd), fv);
 #pragma unroll
-        for (int c = 0; c < LT; ++c) {
-          const float gc = bperm_f(sg.first + c * 4, g);
-          const int fc = bperm_i(sg.first + c * 4, fd);
-          scn += (fc == l) ? gc : 0.f;
-        }
+        for (int c = 0; c < LT; ++c) scn += (__builtin_bit_cast(int, fv[c]) == l) ? gv[c] : 0.f;
       } else {
+        xg[sg.widx] = g;
+        xf[sg.widx] = __builtin_bit_cast(float, fd);
 #pragma unroll 4
         for (int c = 0; c < L; ++c) {
-          const float gc = bperm_f(sg.first + c * 4, g);
-          const int fc = bperm_i(sg.first + c * 4, fd);
+          const float gc = xg[sg.rbase + c];
+          const int fc = __builtin_bit_cast(int, xf[sg.rbase + c]);
           scn += (fc == l) ? gc : 0.f;
         }
       }
@@ -397,7 +460,7 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
       // (TRWP_backward.cu:109-112)
       const int fdc = edge ? fd : 0;
       float det = 0.f;
-      if (DE) det = seg_sum(sg, tab[fdc * L + l] * g);
+      if (DE) det = seg_sum<NQ, EXACT>(xd, sg, tab[fdc * L + l] * g);
       if (DC && edge && (same || fdc != l)) my_pairs[fdc] = fmaf(px.w, g, my_pairs[fdc]);
       const unsigned eo = here ? (unsigned)(st_pix * L + l) * 4u : (unsigned)kDeadOffset;
       if (JACOBI) {
@@ -466,10 +529,10 @@ Params with_wave_prefix(const Params& p, int G) {
 int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool always) {
   if (L > kPackedMaxL) return 0;
   if ((int64_t)B * H * W * L * 4 >= (int64_t)kDeadOffset) return 0;  // 32-bit plane offsets
-  // A packed step issues fewer instructions per chain but has the longer dependent chain (its
-  // reductions go through ds_bpermute): it pays once every SIMD of the 256 CUs would otherwise
-  // hold two or more wavefronts (measured: 516 chains of 129 pixels and 21 labels per launch are
-  // 25 % faster unpacked, 2064 chains 15-40 % faster packed).
+  // A packed step serves up to 64 / L chains but is longer than the step of a wavefront with one
+  // chain (every value shared inside a chain crosses LDS): it pays once the launch has more chains
+  // than the chip has SIMDs (measured with 21 labels: 832 and 1024 chains per launch 9 % faster
+  // unpacked, 1032 and 1232 chains 7-13 % faster packed, 8256 chains twice as fast packed).
   if (chains < (always ? 1 : kPackedMinChains)) return 0;
   int G = kWave / L;
   return G > 16 ? 16 : G;
@@ -481,7 +544,7 @@ bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, bool alwa
   if (G < 2) return false;
   const SweepParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
-  const size_t lds = sizeof(float) * p.L * p.L;
+  const size_t lds = sizeof(float) * (3 * kRedFloats + p.L * p.L);
 #define MPL_PACKED_FWD(LT)                                                                 \
   do {                                                                                     \
     if (train) {                                                                           \
@@ -509,7 +572,7 @@ bool launch_packed_bwd(const BackParams& p0, bool jacobi, bool always, hipStream
   if (G < 2) return false;
   const BackParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
-  const size_t lds = sizeof(float) * p.L * p.L * (1 + G);
+  const size_t lds = sizeof(float) * (4 * kRedFloats + p.L * p.L * (1 + G));
 #define MPL_PACKED_BWD(GRAD)                                                  \
   do {                                                                        \
     if (p.L == 21) {                                                          \
