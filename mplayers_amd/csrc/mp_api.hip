@@ -580,13 +580,24 @@ int read_flags(unsigned flags, const char* what, CallOpts* o) {
   return MPL_OK;
 }
 
-// TRWP launches with at most this many chains (one wavefront each: at most one per SIMD) run both
-// sweeps of a pair of opposite directions in one launch
+// TRWP launches of at most this many wavefronts (at most one per SIMD) run both sweeps of a pair of
+// opposite directions in one launch
 constexpr int kFusedPairMaxChains = 1024;
+
+// wavefronts of a one-direction launch: one per chain, or one per group of chains where the packed
+// scans take the launch
+template <typename Params>
+int launch_waves(const mpl_shape* s, const Params& p, const CallOpts& o) {
+  const int chains = p.block_prefix[p.n_dirs];
+  const int G = o.packed ? packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp, chains,
+                                                  o.packed == 2)
+                         : 0;
+  return G >= 2 ? (chains + G - 1) / G : chains;
+}
 
 void launch_fwd(const SweepParams& p, bool train, bool jacobi, const CallOpts& o, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st, p.fused_pair ? 2 : 1);
-  if (!p.fused_pair && o.packed && launch_packed_fwd(p, train, jacobi, o.packed == 2, st)) return;
+  if (o.packed && launch_packed_fwd(p, train, jacobi, o.packed == 2, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_fwd<1>(p, train, jacobi, st); break;
     case 2: launch_sweep_fwd<2>(p, train, jacobi, st); break;
@@ -597,7 +608,7 @@ void launch_fwd(const SweepParams& p, bool train, bool jacobi, const CallOpts& o
 
 void launch_bwd(const BackParams& p, bool jacobi, const CallOpts& o, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st, p.fused_pair ? 2 : 1);
-  if (!p.fused_pair && o.packed && launch_packed_bwd(p, jacobi, o.packed == 2, st)) return;
+  if (o.packed && launch_packed_bwd(p, jacobi, o.packed == 2, st)) return;
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_bwd<1>(p, jacobi, st); break;
     case 2: launch_sweep_bwd<2>(p, jacobi, st); break;
@@ -786,8 +797,8 @@ int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
       };
       p.skip_s_store = skip_s(d);
       // few chains: the wavefront of a chain sweeps d and then d + 1 (the same pixels in reverse)
-      p.fused_pair = (opts.fused_pairs && opts.packed != 2 && !(d & 1) &&
-                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+      p.fused_pair = (opts.fused_pairs && !(d & 1) &&
+                      launch_waves(s, p, opts) <= kFusedPairMaxChains) ? 1 : 0;
       p.skip_s_store2 = skip_s(d + 1);
       if (train) {
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
@@ -947,8 +958,8 @@ int mpl_trwp_backward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       // few chains: the wavefront of a chain walks d (odd) and then d - 1 (same pixels, reversed)
-      p.fused_pair = (opts.fused_pairs && opts.packed != 2 && (d & 1) &&
-                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+      p.fused_pair = (opts.fused_pairs && (d & 1) &&
+                      launch_waves(s, p, opts) <= kFusedPairMaxChains) ? 1 : 0;
       p.skip_h2 = (it == 0) ? 1 : 0;
       launch_bwd(p, false, opts, st);
       first = false;

@@ -39,9 +39,27 @@ def make_context(kind, L, g):
   return torch.rand(L, generator=g)
 
 
+PACKED_CASES = [
+    # several chains per wavefront (forced for these sizes): the packed scans fuse pairs, too
+    (21, 4, 3, 14, 15, 2, 0.5, True, "dense2d"),
+    (12, 8, 5, 9, 11, 2, 0.5, True, "tl3"),
+    (32, 4, 2, 8, 9, 2, 0.5, False, "dense1d"),
+    (5, 16, 2, 7, 9, 1, 0.5, True, "dense1d"),
+]
+
+
+@pytest.mark.parametrize("L,n_dir,B,H,W,n_iter,rho,train,kind", PACKED_CASES)
+@pytest.mark.parametrize("start", ["cleared", "uninit", "given"])
+def test_fused_pairs_packed_are_bit_identical(gpu, L, n_dir, B, H, W, n_iter, rho, train, kind, start):
+  from mplayers_amd import _lib
+  test_fused_pairs_are_bit_identical(gpu, L, n_dir, B, H, W, n_iter, rho, train, kind, start,
+                                     base_flags=_lib.F_PACKED_ALWAYS)
+
+
 @pytest.mark.parametrize("L,n_dir,B,H,W,n_iter,rho,train,kind", CASES)
 @pytest.mark.parametrize("start", ["cleared", "uninit", "given"])
-def test_fused_pairs_are_bit_identical(gpu, L, n_dir, B, H, W, n_iter, rho, train, kind, start):
+def test_fused_pairs_are_bit_identical(gpu, L, n_dir, B, H, W, n_iter, rho, train, kind, start,
+                                       base_flags=0):
   import torch
   from mplayers_amd import _lib, lib_stereo
   g = torch.Generator().manual_seed(77 * L + n_dir)
@@ -85,8 +103,8 @@ def test_fused_pairs_are_bit_identical(gpu, L, n_dir, B, H, W, n_iter, rho, trai
     torch.cuda.synchronize()
     return [o.cpu().numpy() for o in out], None
 
-  fused, dc_f = run(0)
-  plain, dc_p = run(_lib.F_FUSED_PAIRS_OFF)
+  fused, dc_f = run(base_flags)
+  plain, dc_p = run(base_flags | _lib.F_FUSED_PAIRS_OFF)
   names = ["msg", "cost_final", "msg_min_index", "msg_norm_index", "label_all", "dunary", "dedge"]
   for name, a, b in zip(names, fused, plain):
     assert not np.isnan(a.astype(np.float64)).any(), name
