@@ -137,6 +137,72 @@ __device__ __forceinline__ void dense_step_r1(float a, int L, float w, int lane,
   fd_idx = arg;
 }
 
+// For the 21 candidates of a lane's label and their minimum `best`: the largest fd with
+// val[fd] == best, and in `red` (on entry: best in the lanes of the 21 labels, +inf elsewhere) the
+// minimum over lanes 0..31 in lane 31.
+// A comparison leaves its lane mask in scalar registers, and a select may read such a mask only two
+// issue slots after it was written; a lane shift may read a vector register only two slots after
+// it was written.  The compiler keeps every mask in vcc and pads each of these pairs with idle
+// slots (some 50 per pixel, and a wavefront that has its SIMD to itself pays for every slot), so
+// the three chains are interleaved by hand: masks rotate over three registers, every select comes
+// at least two instructions after its comparison, every shift at least two after the one before,
+// and the first shift three after the start (the compiler wrote `red` just before).
+__device__ __forceinline__ void argmin_and_lane_min_21(const float (&val)[21], float best, float& red,
+                                                       int& arg) {
+  unsigned long long m1, m2;
+  asm(
+      "v_cmp_eq_f32_e64 vcc, %5, %4\n\t"
+      "v_cmp_eq_f32_e64 %2, %6, %4\n\t"
+      "v_cmp_eq_f32_e64 %3, %7, %4\n\t"
+      "v_min_f32_dpp %1, %1, %1 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cndmask_b32_e64 %0, 20, 0, vcc\n\t"
+      "v_cmp_eq_f32_e64 vcc, %8, %4\n\t"
+      "v_min_f32_dpp %1, %1, %1 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cndmask_b32_e64 %0, %0, 1, %2\n\t"
+      "v_cmp_eq_f32_e64 %2, %9, %4\n\t"
+      "v_min_f32_dpp %1, %1, %1 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cndmask_b32_e64 %0, %0, 2, %3\n\t"
+      "v_cmp_eq_f32_e64 %3, %10, %4\n\t"
+      "v_min_f32_dpp %1, %1, %1 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_cndmask_b32_e64 %0, %0, 3, vcc\n\t"
+      "v_cmp_eq_f32_e64 vcc, %11, %4\n\t"
+      "v_min_f32_dpp %1, %1, %1 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_cndmask_b32_e64 %0, %0, 4, %2\n\t"
+      "v_cmp_eq_f32_e64 %2, %12, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 5, %3\n\t"
+      "v_cmp_eq_f32_e64 %3, %13, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 6, vcc\n\t"
+      "v_cmp_eq_f32_e64 vcc, %14, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 7, %2\n\t"
+      "v_cmp_eq_f32_e64 %2, %15, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 8, %3\n\t"
+      "v_cmp_eq_f32_e64 %3, %16, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 9, vcc\n\t"
+      "v_cmp_eq_f32_e64 vcc, %17, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 10, %2\n\t"
+      "v_cmp_eq_f32_e64 %2, %18, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 11, %3\n\t"
+      "v_cmp_eq_f32_e64 %3, %19, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 12, vcc\n\t"
+      "v_cmp_eq_f32_e64 vcc, %20, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 13, %2\n\t"
+      "v_cmp_eq_f32_e64 %2, %21, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 14, %3\n\t"
+      "v_cmp_eq_f32_e64 %3, %22, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 15, vcc\n\t"
+      "v_cmp_eq_f32_e64 vcc, %23, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 16, %2\n\t"
+      "v_cmp_eq_f32_e64 %2, %24, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 17, %3\n\t"
+      "v_cmp_eq_f32_e64 %3, %25, %4\n\t"
+      "v_cndmask_b32_e64 %0, %0, 18, vcc\n\t"
+      "v_cndmask_b32_e64 %0, %0, 19, %2\n\t"
+      "v_cndmask_b32_e64 %0, %0, 20, %3\n\t"
+      : "=&v"(arg), "+v"(red), "=&s"(m1), "=&s"(m2)
+      : "v"(best), "v"(val[0]), "v"(val[1]), "v"(val[2]), "v"(val[3]), "v"(val[4]), "v"(val[5]), "v"(val[6]), "v"(val[7]), "v"(val[8]), "v"(val[9]), "v"(val[10]), "v"(val[11]), "v"(val[12]), "v"(val[13]), "v"(val[14]), "v"(val[15]), "v"(val[16]), "v"(val[17]), "v"(val[18]), "v"(val[19]), "v"(val[20])
+      : "vcc");
+}
+
 // Band O(L*K) step for 1-D contexts with a constant tail (c[k] == cmax for k >= K, c[k] <= cmax
 // below), exact for w >= 0:
 //   v[cd] = min( min_{|k|<K} a[cd+k] + w*c[|k|],  min_fd a[fd] + w*cmax )
@@ -547,22 +613,32 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         }
       } else if (R == 1 && KT < 0 && desc.band_k == 0) {  // (the full table is in LDS then)
         if constexpr (LT > 0) {
-          // 21 labels: the scan over front labels fully unrolled, context column in registers
-          float best = inf;
-          int arg = LT - 1;
+          // 21 labels: the scan over front labels fully unrolled, context column in registers.
+          // The edge weight stays in a vector register (every lane loaded the same one): a[fd]
+          // arrives in a scalar register, and a multiply-add takes one scalar operand only.
+          float af[LT], val[LT];
 #pragma unroll
-          for (int fd = LT - 1; fd >= 0; --fd) {
-            const float val = fmaf(w, tcol[fd], readlane_f(a[0], fd));
-            if (TRAIN) {
-              const bool take = (fd == LT - 1) || (val < best);
-              best = take ? val : best;
-              arg = take ? fd : arg;
-            } else {
-              best = fminf(best, val);
-            }
-          }
+          for (int fd = 0; fd < LT; ++fd) af[fd] = readlane_f(a[0], fd);
+          // (a multiply-add may read a[fd] only two issue slots after it reached its scalar
+          // register: all of them first, then the multiply-adds)
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int fd = 0; fd < LT; ++fd) val[fd] = fmaf(px.w, tcol[fd], af[fd]);
+          float best = val[LT - 1];
+#pragma unroll
+          for (int fd = LT - 2; fd >= 1; fd -= 2) best = fminf(fminf(val[fd], val[fd - 1]), best);
+          if ((LT & 1) == 0) best = fminf(best, val[0]);
           v[0] = best;
-          fd_idx[0] = arg;
+          if (TRAIN) {
+            // the scan in descending order with a strict comparison keeps the largest front label
+            // that attains the minimum
+            float red = valid[0] ? best : inf;
+            argmin_and_lane_min_21(val, best, red, fd_idx[0]);
+            nmin = readlane_f(red, 31);
+            need_nmin = false;
+          } else {
+            fd_idx[0] = LT - 1;
+          }
         } else {
           dense_step_r1<TRAIN>(a[0], L, w, lane, ctx_s, v[0], fd_idx[0]);
         }
