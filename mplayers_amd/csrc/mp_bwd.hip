@@ -261,7 +261,8 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           gv[j] = valid[j] ? fmaf(rho, sc[j], base) : 0.f;
           part += gv[j];
         }
-        const float tot = wave_sum(part);  // MsgNormNaiveBack, commonCUDA.cuh:131-145
+        // MsgNormNaiveBack, commonCUDA.cuh:131-145
+        const float tot = R == 1 ? wave_sum_fast(part) : wave_sum(part);
         if constexpr (R == 1 && SMALL) {
           const int cd = lane, fd = px.fd[0];
           float g = gv[0];
@@ -278,7 +279,31 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
             scn[0] = gather_by_target<8>(g, fd, lane);
           else
             scn[0] = gather_by_target<16>(g, fd, lane);
-          if (DE) det = wave_sum(de);
+          if (DE) det = wave_sum_fast(de);
+        } else if (R == 1 && ctx2d) {
+          // 2-D table (21 labels): the argmin labels of a learned table are spread over all labels,
+          // so neither of the shortcuts below catches many of them: everything goes through the
+          // LDS accumulators at once
+          const int cd = lane, fd = px.fd[0];
+          const int ci = !valid[0] ? 0 : min(cd, fd) * L + max(cd, fd);
+          const float cv = DE ? ctx_s[ci] : 0.f;
+          float g = gv[0];
+          if (cd == nidx) g -= tot;
+          float dev = valid[0] ? cv * g : 0.f;
+          asm volatile("" : "+v"(dev));  // (formed here, not behind the atomics)
+          // The table entry is there before the atomics are issued, so the sum of dedge below runs
+          // while they are under way.  The LDS executes the instructions of a wavefront in their
+          // order: the exchange finds the sums complete without a wait in between, and the
+          // histogram's atomic, which nothing waits for, queues up behind it.
+          __builtin_amdgcn_wave_barrier();
+          if (valid[0]) {
+            atomicAdd(&sc_s[fd], g);
+            __builtin_amdgcn_wave_barrier();
+            scn[0] = atomicExch(&sc_s[lane], 0.f);  // read and clear
+            __builtin_amdgcn_wave_barrier();
+            if (DC && (same || cd != fd)) atomicAdd(&hist_s[ci], w * g);
+          }
+          if (DE) det = wave_sum_fast(dev);
         } else {
         // the two popular targets: where the first and the last label point
         const int f0 = __builtin_amdgcn_readlane(px.fd[0], 0);

@@ -131,18 +131,15 @@ __device__ __forceinline__ float wave_min_f32(float x) {
 // not emit by itself: v_min_f32 with a DPP source, in place, so that a lane without a source keeps
 // its own value.  No conversions to integer keys and back: 6 instructions and the read-out.  (A
 // DPP operand written by the instruction before needs two wait states, which the compiler cannot
-// see inside the statement: each one carries its own.)
+// see inside the statement: each instruction carries its own, in one statement, since the
+// compiler pads the gap between two statements itself.)
 __device__ __forceinline__ float wave_min_fast(float x) {
-#define MPL_MIN_DPP(CTRL) \
-  asm("s_nop 1\n\tv_min_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf" : "+v"(x))
-  MPL_MIN_DPP("row_shr:1 row_mask:0xf");
-  MPL_MIN_DPP("row_shr:2 row_mask:0xf");
-  MPL_MIN_DPP("row_shr:4 row_mask:0xf");
-  MPL_MIN_DPP("row_shr:8 row_mask:0xf");
-  MPL_MIN_DPP("row_bcast:15 row_mask:0xa");
-  MPL_MIN_DPP("row_bcast:31 row_mask:0xc");
+#define MPL_MIN_DPP(CTRL) "s_nop 1\n\tv_min_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf\n\t"
+  asm(MPL_MIN_DPP("row_shr:1 row_mask:0xf") MPL_MIN_DPP("row_shr:2 row_mask:0xf")
+      MPL_MIN_DPP("row_shr:4 row_mask:0xf") MPL_MIN_DPP("row_shr:8 row_mask:0xf")
+      MPL_MIN_DPP("row_bcast:15 row_mask:0xa") MPL_MIN_DPP("row_bcast:31 row_mask:0xc") "s_nop 0"
+      : "+v"(x));
 #undef MPL_MIN_DPP
-  asm("s_nop 1" : "+v"(x));
   return readlane_f(x, 63);
 }
 
@@ -154,6 +151,21 @@ __device__ __forceinline__ float wave_sum(float x) {
   x += dpp_f<0x118>(0.f, x);
   x += dpp_f<0x142, 0xa>(0.f, x);
   x += dpp_f<0x143, 0xc>(0.f, x);
+  return readlane_f(x, 63);
+}
+
+// The same with each lane shift folded into the add, like wave_min_fast (a lane without a source
+// keeps its value, which is what adding zero gives): 6 instructions instead of 10, but one block
+// that the compiler cannot spread other work into.  For steps of a wavefront that has its SIMD to
+// itself, where every issue slot counts; where several wavefronts share a SIMD the version above,
+// whose gaps the compiler fills, is the faster one.  Both give the same bits.
+__device__ __forceinline__ float wave_sum_fast(float x) {
+#define MPL_ADD_DPP(CTRL) "s_nop 1\n\tv_add_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf\n\t"
+  asm(MPL_ADD_DPP("row_shr:1 row_mask:0xf") MPL_ADD_DPP("row_shr:2 row_mask:0xf")
+      MPL_ADD_DPP("row_shr:4 row_mask:0xf") MPL_ADD_DPP("row_shr:8 row_mask:0xf")
+      MPL_ADD_DPP("row_bcast:15 row_mask:0xa") MPL_ADD_DPP("row_bcast:31 row_mask:0xc") "s_nop 0"
+      : "+v"(x));
+#undef MPL_ADD_DPP
   return readlane_f(x, 63);
 }
 
