@@ -269,8 +269,8 @@ const char* mpl_last_error(void);
 /* Process-wide defaults of what the per-call flags MPL_F_PACKED_* and MPL_F_FUSED_U_OFF select
  * (no counterpart in the reference).  A call that passes one of those flags is not affected by
  * these; the values are read atomically once per call.
- * MPL_OPT_PACKED_SCANS (default 1): launches of more than 1024 chains with at most 32 labels, whose
- * planes stay below 2 GiB, are scanned with several chains per wavefront; 0 forces the
+ * MPL_OPT_PACKED_SCANS (default 1): launches of more than 1024 chains (2048 with 21 labels) with
+ * at most 32 labels, whose planes stay below 2 GiB, are scanned with several chains per wavefront; 0 forces the
  * one-chain-per-wavefront kernels, 2 packs whenever the label count allows it (the results agree
  * to the parity tolerance; 0 and 2 are meant for tests and comparisons). */
 #define MPL_OPT_PACKED_SCANS 0

@@ -533,6 +533,9 @@ void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 // The launchers return false, without launching, when the problem does not qualify.
 constexpr int kPackedMaxL = 32;
 constexpr int kPackedMinChains = 1025;  // more chains than the 256 CUs have SIMDs
+// 21 labels with their 2-D table: the one-chain-per-wavefront scans have a short step of their own,
+// and two of their wavefronts fit a SIMD
+constexpr int kPackedMinChains21 = 2049;
 // always: pack whatever the number of chains (tests and comparisons)
 // chains per wavefront the packed scans would use for such a launch (below 2: they do not apply)
 int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool always);

@@ -598,9 +598,14 @@ int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool alwa
   if ((int64_t)B * H * W * L * 4 >= (int64_t)kDeadOffset) return 0;  // 32-bit plane offsets
   // A packed step serves up to 64 / L chains but is longer than the step of a wavefront with one
   // chain (every value shared inside a chain crosses LDS): it pays once the launch has more chains
-  // than the chip has SIMDs (measured with 21 labels: 832 and 1024 chains per launch 9 % faster
-  // unpacked, 1032 and 1232 chains 7-13 % faster packed, 8256 chains twice as fast packed).
-  if (chains < (always ? 1 : kPackedMinChains)) return 0;
+  // than the chip has SIMDs.  With 21 labels the unpacked step is short enough to win while all
+  // wavefronts of the launch are resident at once, two to a SIMD (measured, TRWP fwd+bwd on
+  // 4 x H x H: 1032 chains per launch 5.4 ms unpacked against 6.2 packed, 1548 chains 8.5 against
+  // 9.3, 1804 chains 10.2 against 10.8, but 2064 chains 15.0 against 12.6; ISGMR with 1536 chains
+  // per launch 0.85 against 0.88, with 2064 chains 1.28 against 1.12, with 8256 chains 11.4
+  // against 6.9).
+  const int min_chains = L == 21 ? kPackedMinChains21 : kPackedMinChains;
+  if (chains < (always ? 1 : min_chains)) return 0;
   int G = kWave / L;
   return G > 16 ? 16 : G;
 }

@@ -406,32 +406,34 @@ __device__ __forceinline__ float exp_below(float x, float m_log2e) {
 
 // Reductions as chains of DPP-fused operations (a lane without a source lane keeps its value; a
 // DPP operand written by the instruction before needs two wait states, which the compiler cannot
-// see inside the statement).  NL = 16 / 32 / 64: over the first NL lanes only, the others are
-// ignored; the result is wave-uniform.
-#define MPL_RED_DPP(OP, CTRL) \
-  asm("s_nop 1\n\t" OP " %0, %0, %0 " CTRL " bank_mask:0xf" : "+v"(x))
+// see inside a statement: each instruction carries its own, and a chain is one statement, since
+// the compiler pads the gap between two statements itself).  NL = 16 / 32 / 64: over the first NL
+// lanes only, the others are ignored; the result is wave-uniform.
+#define MPL_RED_DPP(OP, CTRL) "s_nop 1\n\t" OP " %0, %0, %0 " CTRL " bank_mask:0xf\n\t"
+#define MPL_RED_ROW(OP)                                                            \
+  MPL_RED_DPP(OP, "row_shr:1 row_mask:0xf") MPL_RED_DPP(OP, "row_shr:2 row_mask:0xf") \
+      MPL_RED_DPP(OP, "row_shr:4 row_mask:0xf") MPL_RED_DPP(OP, "row_shr:8 row_mask:0xf")
+#define MPL_RED_LANES(OP)                                                                      \
+  if constexpr (NL <= 16)                                                                      \
+    asm(MPL_RED_ROW(OP) "s_nop 0" : "+v"(x));                                                  \
+  else if constexpr (NL <= 32)                                                                 \
+    asm(MPL_RED_ROW(OP) MPL_RED_DPP(OP, "row_bcast:15 row_mask:0xa") "s_nop 0" : "+v"(x));     \
+  else                                                                                         \
+    asm(MPL_RED_ROW(OP) MPL_RED_DPP(OP, "row_bcast:15 row_mask:0xa")                           \
+            MPL_RED_DPP(OP, "row_bcast:31 row_mask:0xc") "s_nop 0"                             \
+        : "+v"(x))
 template <int NL>
 __device__ __forceinline__ float lanes_sum(float x) {
-  MPL_RED_DPP("v_add_f32_dpp", "row_shr:1 row_mask:0xf");
-  MPL_RED_DPP("v_add_f32_dpp", "row_shr:2 row_mask:0xf");
-  MPL_RED_DPP("v_add_f32_dpp", "row_shr:4 row_mask:0xf");
-  MPL_RED_DPP("v_add_f32_dpp", "row_shr:8 row_mask:0xf");
-  if (NL > 16) MPL_RED_DPP("v_add_f32_dpp", "row_bcast:15 row_mask:0xa");
-  if (NL > 32) MPL_RED_DPP("v_add_f32_dpp", "row_bcast:31 row_mask:0xc");
-  asm("s_nop 1" : "+v"(x));
+  MPL_RED_LANES("v_add_f32_dpp");
   return readlane_f(x, NL - 1);
 }
 template <int NL>
 __device__ __forceinline__ float lanes_min(float x) {
-  MPL_RED_DPP("v_min_f32_dpp", "row_shr:1 row_mask:0xf");
-  MPL_RED_DPP("v_min_f32_dpp", "row_shr:2 row_mask:0xf");
-  MPL_RED_DPP("v_min_f32_dpp", "row_shr:4 row_mask:0xf");
-  MPL_RED_DPP("v_min_f32_dpp", "row_shr:8 row_mask:0xf");
-  if (NL > 16) MPL_RED_DPP("v_min_f32_dpp", "row_bcast:15 row_mask:0xa");
-  if (NL > 32) MPL_RED_DPP("v_min_f32_dpp", "row_bcast:31 row_mask:0xc");
-  asm("s_nop 1" : "+v"(x));
+  MPL_RED_LANES("v_min_f32_dpp");
   return readlane_f(x, NL - 1);
 }
+#undef MPL_RED_LANES
+#undef MPL_RED_ROW
 #undef MPL_RED_DPP
 
 // (minimum, sum of weights, weighted sum of duals) of a label over all its front labels from the
@@ -475,7 +477,7 @@ __global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams
   extern __shared__ float smem[];
   const int L = p.L, LL = L * L;
   float* tile = smem;              // 256 * NT4 floats (training): the pixel's block as it is stored
-  float* tab = smem + (TRAIN ? 256 * NT4 : 0);  // LL floats
+  float* tab = smem + (TRAIN ? 256 * NT4 : 0);  // LL floats (training: and a spare word per lane)
   const int lane = threadIdx.x;
   const ChainCtx ch0 = locate_chain(p);
   if (ch0.n < 2) return;  // nothing to write
@@ -539,7 +541,10 @@ __global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams
     const int fd = inr[i] ? fd0 + i : L - 1;
     tcol[i] = tab[fd * L + cd];  // ctx(cd, fd)
     src[i] = fd * 4;             // a[fd] from group 0's replica
-    tidx[i] = even ? fd * L + cd : cd * L + fd;  // place of (cd, fd) inside the stored block
+    // place of (cd, fd) inside the stored block; an entry that does not exist goes to a spare word
+    // of this lane behind the table (a store to somewhere costs one instruction, a skipped one a
+    // save, a branch and a restore of the execution mask)
+    tidx[i] = inr[i] ? (even ? fd * L + cd : cd * L + fd) : 256 * NT4 + LL + lane;
   }
   // the block leaves as NT4 16-byte stores per lane and, L * L being 0 or 1 modulo 4, one last dword
   int qoff[NT4];
@@ -614,7 +619,7 @@ __global__ void __launch_bounds__(kWave) soft_split_fwd_kernel(const SweepParams
       if (TRAIN) {
 #pragma unroll
         for (int i = 0; i < FM; ++i)
-          if (inr[i]) tile[tidx[i]] = dual[i];
+          tile[tidx[i]] = dual[i];
       }
       float mn, se, sd, scale;
       group_softmin<G>(addr, mn_l, se_l, sd_l, mn, se, sd, scale);
@@ -679,7 +684,7 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
   float* tab = smem;         // LL
   const int LLp = (LL + 3) & ~3;  // (keeps the rows of the gradient block 16-byte aligned)
   float* hist = tab + LLp;   // LL: per-pair dcontext accumulator [fd * L + cd]
-  float* grad = hist + LLp;  // L rows of S: ddual[fd * S + cd], 0 beyond cd = L - 1
+  float* grad = hist + LLp;  // L rows of S: ddual[fd * S + cd], 0 beyond cd = L - 1; a spare word per lane
   const int lane = threadIdx.x;
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t P = (int64_t)p.B * HW;
@@ -755,7 +760,7 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
     tcol[i] = tab[fd * L + cd];
     // place of (cd, fd) inside the pixel's stored block
     boff[i] = inr[i] ? (even ? fd * L + cd : cd * L + fd) * 4 : kDeadOffset;
-    gidx[i] = fd * S + cd;
+    gidx[i] = inr[i] ? fd * S + cd : L * S + lane;  // (a spare word per lane behind the block)
   }
   const float4* grow = reinterpret_cast<const float4*>(grad + cd * S);  // row of front label cd
 
@@ -832,7 +837,7 @@ __global__ void __launch_bounds__(kWave) soft_split_bwd_kernel(const BackParams 
           const float dd = inr[i] ? gs * ex[i] * (soft1 - px.dual[i]) : 0.f;
           de = fmaf(tcol[i], dd, de);
           hreg[i] = fmaf(w, dd, hreg[i]);
-          if (inr[i]) grad[gidx[i]] = dd;
+          grad[gidx[i]] = dd;
         }
         // dU[q, fd] = sum_cd ddual[cd, fd]: every lane of label fd adds up the row in the same order
 #pragma unroll
@@ -1414,7 +1419,7 @@ void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st) {
   if (p.L <= 32) {  // front labels split over the idle lanes
 #define MPL_SOFT_SPLIT_FWD(GG, FF, NN)                                                       \
   do {                                                                                       \
-    const size_t slds = sizeof(float) * (LL + (train ? 256 * NN : 0));                       \
+    const size_t slds = sizeof(float) * (LL + (train ? 256 * NN + kWave : 0));               \
     if (train)                                                                               \
       soft_split_fwd_kernel<true, GG, FF, NN><<<blocks, kWave, slds, st>>>(p);               \
     else                                                                                     \
@@ -1454,7 +1459,7 @@ void launch_soft_bwd(const BackParams& p, hipStream_t st) {
   const size_t lds = sizeof(float) * (2 * LL + kWave * T + p.L * (p.L | 1));
   if (p.L <= 32) {  // front labels split over the idle lanes
     const int NQ = p.L <= 16 ? 4 : (p.L <= 21 ? 6 : 8);
-    const size_t slds = sizeof(float) * (2 * ((LL + 3) & ~3) + p.L * 4 * NQ);
+    const size_t slds = sizeof(float) * (2 * ((LL + 3) & ~3) + p.L * 4 * NQ + kWave);
     if (p.L <= 16)
       soft_split_bwd_kernel<4, 4, 4><<<blocks, kWave, slds, st>>>(p);
     else if (p.L <= 21)

@@ -1,5 +1,5 @@
 """Scans with several chains per wavefront (at most 32 labels).  By default only launches of more
-than 1024 chains take them, so the small cases are run with the policy forced (option value 2)
+than 1024 chains (2048 with 21 labels) take them, so the small cases are run with the policy forced (option value 2)
 and one case is large enough to take them on its own; every result is checked against the oracle
 exactly like the one-chain-per-wavefront kernels."""
 import numpy as np
@@ -81,7 +81,7 @@ def test_small_cases_forced_packed(gpu, oracle, always_packed, seed):
 
 @pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
 def test_segmentation_batch_takes_packed_scans(gpu, oracle, mode):
-  """8 x 65 x 64 pixels, 21 labels: more than 1024 chains per launch, so the default policy packs;
+  """8 x 65 x 64 pixels, 21 labels: more than 2048 chains per launch, so the default policy packs;
   the same call with packing switched off must agree with it to the tolerance."""
   from mplayers_amd import _lib
   rng = np.random.default_rng(11)
