@@ -587,7 +587,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       for (int j = 0; j < R; ++j) a[j] = fmaf(rho, prev[j], uf[j]);
       float nmin;
       bool need_nmin = true;
-      if ((KT >= 0 || KT == -2) && w >= 0.f) {
+      if ((KT >= 0 || KT == -2) && __builtin_expect(w >= 0.f, 1)) {  // (the usual case falls through)
         float am = a[0];
 #pragma unroll
         for (int j = 1; j < R; ++j) am = fminf(am, a[j]);
