@@ -19,28 +19,19 @@
 namespace mpl {
 namespace {
 
-// LDS float atomics cost ~190 clocks per wave instruction on this hardware and serialise per CU,
-// so the common cases of the scatter and of the dcontext histogram are done without them:
+// Several labels per lane, and 33 to 64 labels in launches that fill the chip: an LDS float atomic
+// and the exchange that reads its sums back take some 250 clocks and occupy the LDS of the CU, so
+// the common cases of the scatter and of the dcontext histogram are done without them:
 //   * argmin indices that point at the two most popular targets of the pixel (taken from the first
 //     and the last label; with a truncated pairwise term nearly every label points at argmin(a))
 //     are summed with a wave reduction,
 //   * indices within kNear labels of their own label are moved with DPP label shifts,
 //   * only what is left goes through LDS atomics.
+// One label per lane otherwise (DIRECT): the step is bound by its own latency, and one atomic for
+// the scatter, one exchange and one atomic for the histogram are the shortest way through it.
 constexpr int kNear = 3;
-constexpr int kSmallL = 16;  // beyond that the register/LDS scatter below is faster (measured at 21)
-
-// sum over the first LS lanes c of g[c] where target[c] == lane
-template <int LS>
-__device__ __forceinline__ float gather_by_target(float g, int target, int lane) {
-  float acc = 0.f;
-#pragma unroll
-  for (int c = 0; c < LS; ++c) {
-    const float gc = readlane_f(g, c);
-    const int fc = __builtin_amdgcn_readlane(target, c);
-    acc += (lane == fc) ? gc : 0.f;
-  }
-  return acc;
-}
+// launches of at most this many chains (two wavefronts per SIMD) are taken to be latency-bound
+constexpr int kDirectMaxChains = 2048;
 
 template <int R>
 struct PixB {
@@ -50,11 +41,11 @@ struct PixB {
   float w, de;
 };
 
-// SMALL: one label per lane and at most kSmallL labels (see small_l below)
+// DIRECT: one label per lane, everything through the LDS accumulators (see above and the launcher)
 // GRAD: bit 0 = dedge_weights is wanted, bit 1 = dcontext is wanted (a caller with a fixed pairwise
 // table or edge weights that are not learned passes null for them; that part of the step is then
 // not compiled in: no dedge read-modify-write, no context products, no histogram gathers)
-template <int R, bool VEC, bool MASK, bool JACOBI, bool SMALL, int GRAD>
+template <int R, bool VEC, bool MASK, bool JACOBI, bool DIRECT, int GRAD>
 __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   constexpr bool DE = (GRAD & 1) != 0, DC = (GRAD & 2) != 0;
   extern __shared__ float smem[];
@@ -69,10 +60,6 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   float* g1_s = g0_s + 3 * L;      // same for class 1
   float* ctx_s = g1_s + 3 * L;     // context table
   float* hist_s = ctx_s + n_ctx;   // dcontext accumulator of the slow path (and of 2-D contexts)
-  // one label per lane and at most kSmallL labels: the scatter is a loop over source labels and
-  // dcontext is accumulated per (cd, fd) pair, each lane owning the row of its label
-  constexpr bool small_l = SMALL;
-  float* pair_s = hist_s + n_ctx;  // L * L floats when small_l
   const int lane = threadIdx.x;
   const int64_t P = (int64_t)p.B * p.H * p.W;
   const int64_t N = P * L;
@@ -85,8 +72,6 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
     hist_s[i] = 0.f;
   }
   for (int i = lane; i < kMaxL + 6 * L; i += kWave) sc_s[i] = 0.f;  // sc_s, g0_s, g1_s
-  if (small_l)
-    for (int i = lane; i < L * L; i += kWave) pair_s[i] = 0.f;
   __syncthreads();
 
   // Offsets |fd - cd| come from the band of the context (entries below its constant tail) or from
@@ -96,7 +81,7 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   // (With one label per lane the step is short and the scans are bound by its latency, which
   // the wave-uniform branches would lengthen: the narrowing is for several labels per lane.)
   int near_max = kNear;
-  if (R > 1 && !ctx2d && !small_l) {
+  if (R > 1 && !ctx2d) {
     int kb = 0;
     for (int i = lane; i < L; i += kWave) kb = (ctx_s[i] != ctx_s[L - 1]) ? i + 1 : kb;
     kb = (int)-wave_min(-(float)kb);  // wave maximum: entries at and beyond kb equal the last one
@@ -263,29 +248,12 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
         }
         // MsgNormNaiveBack, commonCUDA.cuh:131-145
         const float tot = R == 1 ? wave_sum_fast(part) : wave_sum(part);
-        if constexpr (R == 1 && SMALL) {
+        if constexpr (R == 1 && DIRECT) {
+          // one atomic that scatters the gradients to their argmin labels, one exchange that
+          // reads the sums back and clears them, one atomic for the dcontext histogram
           const int cd = lane, fd = px.fd[0];
-          float g = gv[0];
-          if (cd == nidx) g -= tot;
-          if (!valid[0]) g = 0.f;
-          // this lane's own pair: dedge and dcontext (TRWP_backward.cu:109-112)
           const int ao = fd > cd ? fd - cd : cd - fd;
-          const int ci = !valid[0] ? 0 : (ctx2d ? (cd < fd ? cd * L + fd : fd * L + cd) : ao);
-          const float de = DE ? ctx_s[ci] * g : 0.f;
-          if (DC && valid[0] && (same || cd != fd)) pair_s[cd * L + fd] = fmaf(w, g, pair_s[cd * L + fd]);
-          // dU[q, f] = sum of g[c] over the labels c that point at f: one source label per trip
-          // (fully unrolled for the next size bucket: lanes past L carry g = 0)
-          if (L <= 8)
-            scn[0] = gather_by_target<8>(g, fd, lane);
-          else
-            scn[0] = gather_by_target<16>(g, fd, lane);
-          if (DE) det = wave_sum_fast(de);
-        } else if (R == 1 && ctx2d) {
-          // 2-D table (21 labels): the argmin labels of a learned table are spread over all labels,
-          // so neither of the shortcuts below catches many of them: everything goes through the
-          // LDS accumulators at once
-          const int cd = lane, fd = px.fd[0];
-          const int ci = !valid[0] ? 0 : min(cd, fd) * L + max(cd, fd);
+          const int ci = !valid[0] ? 0 : (ctx2d ? (int)__umul24(min(cd, fd), L) + max(cd, fd) : ao);
           const float cv = DE ? ctx_s[ci] : 0.f;
           float g = gv[0];
           if (cd == nidx) g -= tot;
@@ -495,27 +463,6 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
   }  // both walks of a fused pair
   if (!DC) return;
   __syncthreads();
-  if (small_l) {
-    // fold the pair table into dcontext's bins: |cd - fd| (1-D) or [min, max] (2-D); the pairs
-    // with cd == fd (bin 0 / the diagonal) were only collected when the caller asked for them
-    if (!ctx2d) {
-      if (lane < L) {
-        float acc = 0.f;
-        for (int c = 0; c < L; ++c) {
-          if (c + lane < L) acc += pair_s[c * L + c + lane];
-          if (lane >= 1 && c - lane >= 0) acc += pair_s[c * L + c - lane];
-        }
-        if (acc != 0.f) atomicAdd(&p.dctx[lane], acc);
-      }
-    } else {
-      for (int i = lane; i < L * L; i += kWave) {
-        const int c = i / L, f = i - c * L;
-        if (c > f) continue;  // the (f, c) entry is added here
-        const float v = pair_s[i] + (c < f ? pair_s[f * L + c] : 0.f);
-        if (v != 0.f) atomicAdd(&p.dctx[i], v);
-      }
-    }
-  }
   for (int i = lane; i < n_ctx; i += kWave) {
     float v = hist_s[i];
     if (v != 0.f) atomicAdd(&p.dctx[i], v);
@@ -541,10 +488,14 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
 template <int R, bool VEC, bool MASK, int GRAD>
 void launch_vmg(const BackParams& p, bool jacobi, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
-  const size_t lds = sizeof(float) * (kMaxL + 6 * p.L + 2 * (p.ctx2d ? p.L * p.L : p.L) +
-                                      ((R == 1 && p.L <= kSmallL) ? p.L * p.L : 0));
+  const size_t lds = sizeof(float) * (kMaxL + 6 * p.L + 2 * (p.ctx2d ? p.L * p.L : p.L));
   if constexpr (R == 1) {
-    if (p.L <= kSmallL) {
+    // Up to 32 labels every launch that fills the chip goes to the packed scans, and a 2-D table
+    // spreads its argmin labels over all labels; with 33 to 64 labels and a 1-D table the
+    // accumulators win while the launch is latency-bound (measured on 4 directions with
+    // min(k, 3) tables, fwd+bwd: 40 labels, 1200 chains per launch 4.7 -> 3.4 ms through the
+    // accumulators, but 64 labels, 3200 chains 7.5 -> 9.0 ms).
+    if (p.L <= kPackedMaxL || p.ctx2d || blocks <= kDirectMaxChains) {
       if (jacobi)
         sweep_bwd_kernel<R, VEC, MASK, true, true, GRAD><<<blocks, kWave, lds, st>>>(p);
       else
