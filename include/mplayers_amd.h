@@ -269,10 +269,14 @@ const char* mpl_last_error(void);
 /* Process-wide defaults of what the per-call flags MPL_F_PACKED_* and MPL_F_FUSED_U_OFF select
  * (no counterpart in the reference).  A call that passes one of those flags is not affected by
  * these; the values are read atomically once per call.
- * MPL_OPT_PACKED_SCANS (default 1): launches of more than 1024 chains (2048 with 21 labels) with
- * at most 32 labels, whose planes stay below 2 GiB, are scanned with several chains per wavefront; 0 forces the
- * one-chain-per-wavefront kernels, 2 packs whenever the label count allows it (the results agree
- * to the parity tolerance; 0 and 2 are meant for tests and comparisons). */
+ * MPL_OPT_PACKED_SCANS (default 1): launches with a 2-D table of at most 32 labels and more than
+ * 1024 chains (2048 with 21 labels), and launches with a 1-D table of at most 8 labels and more than
+ * 4096 chains, whose planes stay below 2 GiB, are scanned with several chains per wavefront; 0
+ * forces the one-chain-per-wavefront kernels, 2 packs whenever the label count (at most 32) allows
+ * it.  The packed step scans every front label whatever the table, so it is not the default for
+ * 1-D tables, which are nearly always bands; a caller whose 1-D tables of up to 32 labels are dense
+ * and whose launches have thousands of chains gains from 2 (or MPL_F_PACKED_ALWAYS per call).  The
+ * results agree to the parity tolerance in every case. */
 #define MPL_OPT_PACKED_SCANS 0
 /* MPL_OPT_FUSED_U (default 1): ISGMR forward with 4 directions, rho == 1 and one chain per
  * wavefront (more than 32 labels, or a launch the packed scans do not take) forms U inside the scans (unary + the old messages of the other pair of directions) instead of

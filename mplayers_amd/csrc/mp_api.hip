@@ -589,8 +589,8 @@ constexpr int kFusedPairMaxChains = 1024;
 template <typename Params>
 int launch_waves(const mpl_shape* s, const Params& p, const CallOpts& o) {
   const int chains = p.block_prefix[p.n_dirs];
-  const int G = o.packed ? packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp, chains,
-                                                  o.packed == 2)
+  const int G = o.packed ? packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp,
+                                                  s->ctx2d != 0, chains, o.packed == 2)
                          : 0;
   return G >= 2 ? (chains + G - 1) / G : chains;
 }
@@ -858,7 +858,7 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
   // of small label counts run: they are bound by the instructions of a step, and two more loads
   // per step cost them more than the pass.)
   const bool packed_runs =
-      opts.packed && packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp,
+      opts.packed && packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp, s->ctx2d != 0,
                                             p.block_prefix[p.n_dirs], opts.packed == 2) >= 2;
   const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && !packed_runs;
   if (msg_uninit && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);

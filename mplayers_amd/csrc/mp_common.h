@@ -532,13 +532,22 @@ void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 // packed scans for small label counts (mp_pack.hip): several chains per wavefront.
 // The launchers return false, without launching, when the problem does not qualify.
 constexpr int kPackedMaxL = 32;
-constexpr int kPackedMinChains = 1025;  // more chains than the 256 CUs have SIMDs
-// 21 labels with their 2-D table: the one-chain-per-wavefront scans have a short step of their own,
-// and two of their wavefronts fit a SIMD
+// A launch is packed by default when
+//  * its table is 2-D (a learned table, dense) and it has more chains than the 256 CUs have SIMDs;
+//    with 21 labels, whose one-chain-per-wavefront scans have a short step of their own, more
+//    chains than two wavefronts per SIMD,
+//  * its table is 1-D, it has at most 8 labels and more than 4096 chains.  The packed step is the
+//    dense one, L candidates per label, whatever the table; nearly every 1-D table is a band
+//    (Potts, truncated linear or quadratic), whose step in the one-chain scans takes a few taps,
+//    and only the device knows which it is.  A caller with dense 1-D tables of up to 32 labels
+//    and thousands of chains per launch passes MPL_F_PACKED_ALWAYS.
+constexpr int kPackedMinChains = 1025;
 constexpr int kPackedMinChains21 = 2049;
-// always: pack whatever the number of chains (tests and comparisons)
+constexpr int kPackedMinChains1d = 4097;
+constexpr int kPackedMaxL1d = 8;
+// always: pack whatever the table and the number of chains (tests, comparisons, such callers)
 // chains per wavefront the packed scans would use for such a launch (below 2: they do not apply)
-int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool always);
+int packed_chains_per_wave(int B, int H, int W, int L, bool ctx2d, int64_t chains, bool always);
 bool launch_packed_fwd(const SweepParams& p, bool train, bool jacobi, bool always, hipStream_t st);
 bool launch_packed_bwd(const BackParams& p, bool jacobi, bool always, hipStream_t st);
 

@@ -593,26 +593,35 @@ Params with_wave_prefix(const Params& p, int G) {
 
 }  // namespace
 
-int packed_chains_per_wave(int B, int H, int W, int L, int64_t chains, bool always) {
+int packed_chains_per_wave(int B, int H, int W, int L, bool ctx2d, int64_t chains, bool always) {
   if (L > kPackedMaxL) return 0;
   if ((int64_t)B * H * W * L * 4 >= (int64_t)kDeadOffset) return 0;  // 32-bit plane offsets
   // A packed step serves up to 64 / L chains but is longer than the step of a wavefront with one
-  // chain (every value shared inside a chain crosses LDS): it pays once the launch has more chains
-  // than the chip has SIMDs.  With 21 labels the unpacked step is short enough to win while all
-  // wavefronts of the launch are resident at once, two to a SIMD (measured, TRWP fwd+bwd on
-  // 4 x H x H: 1032 chains per launch 5.4 ms unpacked against 6.2 packed, 1548 chains 8.5 against
-  // 9.3, 1804 chains 10.2 against 10.8, but 2064 chains 15.0 against 12.6; ISGMR with 1536 chains
-  // per launch 0.85 against 0.88, with 2064 chains 1.28 against 1.12, with 8256 chains 11.4
-  // against 6.9).
-  const int min_chains = L == 21 ? kPackedMinChains21 : kPackedMinChains;
-  if (chains < (always ? 1 : min_chains)) return 0;
+  // chain (every value shared inside a chain crosses LDS, and it scans all L front labels per
+  // label whatever the table), so it pays once the launch has more chains than the chip has SIMDs,
+  // for a dense table.  Measured, fwd+bwd, packed against one chain per wavefront:
+  //  * 21 labels, 2-D table, 4 x H x H: TRWP with 1032 chains per launch 6.2 against 5.4 ms, 1548
+  //    chains 9.3 against 8.5, 1804 chains 10.8 against 10.2, but 2064 chains (a third wavefront on
+  //    some SIMDs) 12.6 against 15.0; ISGMR with 1536 chains 0.88 against 0.85, 2064 chains 1.12
+  //    against 1.28, 8256 chains 6.9 against 11.4;
+  //  * 1-D tables, ISGMR, 3 iterations: min(k, 3) with 16 / 32 labels and 1280 chains 2.0 / 3.7
+  //    against 0.73 / 0.88 ms; dense with 16 / 32 labels, 1280 chains 2.0 / 3.7 against 1.3 / 2.3
+  //    and 10240 chains 5.2 / 15.0 against 9.7 / 18.2; 8 labels, 5120 chains, dense 1.42 against
+  //    1.62 and min(k, 3) 1.42 against 1.36; 4 labels, 5120 chains, dense 0.98 against 1.34.
+  if (!always) {
+    if (ctx2d) {
+      if (chains < (L == 21 ? kPackedMinChains21 : kPackedMinChains)) return 0;
+    } else {
+      if (L > kPackedMaxL1d || chains < kPackedMinChains1d) return 0;
+    }
+  }
   int G = kWave / L;
   return G > 16 ? 16 : G;
 }
 
 bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, bool always, hipStream_t st) {
   if (p0.u_fused) return false;  // (set for more than 32 labels only)
-  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0), always);
+  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, p0.ctx2d != 0, chains_in_launch(p0), always);
   if (G < 2) return false;
   const SweepParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
@@ -640,7 +649,7 @@ bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, bool alwa
 }
 
 bool launch_packed_bwd(const BackParams& p0, bool jacobi, bool always, hipStream_t st) {
-  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, chains_in_launch(p0), always);
+  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, p0.ctx2d != 0, chains_in_launch(p0), always);
   if (G < 2) return false;
   const BackParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
