@@ -490,11 +490,12 @@ void launch_vmg(const BackParams& p, bool jacobi, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = sizeof(float) * (kMaxL + 6 * p.L + 2 * (p.ctx2d ? p.L * p.L : p.L));
   if constexpr (R == 1) {
-    // Up to 32 labels every launch that fills the chip goes to the packed scans, and a 2-D table
-    // spreads its argmin labels over all labels; with 33 to 64 labels and a 1-D table the
-    // accumulators win while the launch is latency-bound (measured on 4 directions with
-    // min(k, 3) tables, fwd+bwd: 40 labels, 1200 chains per launch 4.7 -> 3.4 ms through the
-    // accumulators, but 64 labels, 3200 chains 7.5 -> 9.0 ms).
+    // Through the accumulators: up to 32 labels (with few lanes of a wavefront in use the atomics
+    // are short even where several wavefronts share a SIMD: 8 x 400 x 400, min(k, 3) table, TRWP
+    // fwd+bwd with 16 / 24 / 32 labels 5.7 / 8.2 / 7.7 ms against 9.2 / 10.6 / 9.5 with the
+    // shortcuts), 2-D tables (their argmin labels are spread over all labels), and 33 to 64 labels
+    // while the launch is latency-bound (40 labels, 1200 chains per launch 3.4 against 4.7 ms, but
+    // 64 labels, 3200 chains 9.0 against 7.5).
     if (p.L <= kPackedMaxL || p.ctx2d || blocks <= kDirectMaxChains) {
       if (jacobi)
         sweep_bwd_kernel<R, VEC, MASK, true, true, GRAD><<<blocks, kWave, lds, st>>>(p);
