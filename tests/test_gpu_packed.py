@@ -105,6 +105,28 @@ def test_segmentation_batch_takes_packed_scans(gpu, oracle, mode):
   assert (got["msg_min_index"] != plain["msg_min_index"]).mean() < 1e-3
 
 
+def test_band_table_of_many_chains_stays_unpacked(gpu, oracle):
+  """A 1-D table is nearly always a band, whose step the one-chain-per-wavefront scans do in a few
+  taps while the packed step scans every front label: 16 labels and 1344 chains per launch are not
+  packed by default.  The two kinds of reverse scan sum dedge_weights in different orders, which
+  shows which one ran."""
+  from mplayers_amd import _lib
+  rng = np.random.default_rng(5)
+  B, H, W, L, n_dir, n_iter = 2, 160, 176, 16, 4, 1
+  ctx = (0.3 * np.minimum(np.arange(L), 3)).astype(np.float32)
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  dcost = rng.standard_normal((B, 1, H, W, L)).astype(np.float32)
+  fwd = gpu.gpu_forward("ISGMR", unary, ctx, ew, n_dir, n_iter, 1.0)
+  run = lambda flags: gpu.gpu_backward("ISGMR", ctx, ew, dcost, fwd["msg_min_index"],
+                                       fwd["msg_norm_index"], 1.0, flags=flags)
+  default, off, always = run(0), run(_lib.F_PACKED_OFF), run(_lib.F_PACKED_ALWAYS)
+  assert np.array_equal(default[2], off[2])
+  assert not np.array_equal(default[2], always[2])
+  assert np.abs(default[2] - always[2]).max() <= 1e-4 * np.abs(default[2]).max()
+  assert np.array_equal(default[0], off[0])
+
+
 def test_set_option_rejects_unknown(gpu):
   from mplayers_amd import _lib
   with pytest.raises(RuntimeError):
