@@ -168,6 +168,32 @@ def test_backward_matches_oracle(gpu, oracle, mode, n_dir, B, H, W, L, kind, n_i
     assert got[1][0] == 0
 
 
+@pytest.mark.parametrize("mode,L,kind", [("TRWP", 40, "tl3"), ("ISGMR", 64, "tl3"), ("TRWP", 33, "rand1d")])
+def test_backward_of_many_short_chains(gpu, oracle, mode, L, kind):
+  """33 to 64 labels with a 1-D table: launches of more than 2048 chains take the reverse scan that
+  sums popular argmin targets with wave reductions, smaller ones the LDS accumulators.  9 x 240 x 6
+  pixels give TRWP 2160 rows of 6 pixels (the first kind) and 54 columns of 240 (the second);
+  ISGMR puts all of them into one launch."""
+  rng = np.random.default_rng(L)
+  n_dir, n_iter, B, H, W = 4, 2, 9, 240, 6
+  rho = 0.5 if mode == "TRWP" else 1.0
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32) * 3
+  k = np.arange(L, dtype=np.float32)
+  ctx = (0.3 * np.minimum(k, 3)).astype(np.float32) if kind == "tl3" else rng.random(L).astype(np.float32)
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  dcost = rng.standard_normal(unary.shape).astype(np.float32)
+  print("case", mode, L, kind, flush=True)
+  fwd = oracle.forward(mode, unary, ctx, ew, n_dir, n_iter, rho)
+  ref = oracle.backward(mode, ctx.astype(np.float64), ew.astype(np.float64),
+                        dcost.astype(np.float64), fwd["msg_min_index"], fwd["msg_norm_index"], rho)
+  got = gpu.gpu_backward(mode, ctx, ew, dcost, fwd["msg_min_index"], fwd["msg_norm_index"], rho,
+                         garbage_scratch=True)
+  for g, r, name in zip(got, ref, ("dunary", "dcontext", "dedge_weights")):
+    scale = max(1.0, float(np.abs(r).max()))
+    assert np.abs(g - r).max() <= 1e-4 * scale, (name, float(np.abs(g - r).max()), scale)
+  assert got[1][0] == 0
+
+
 def test_sgm_flag(gpu, oracle):
   rng = np.random.default_rng(5)
   B, H, W, L, n_dir = 1, 6, 7, 24, 8
