@@ -127,6 +127,25 @@ def test_band_table_of_many_chains_stays_unpacked(gpu, oracle):
   assert np.array_equal(default[0], off[0])
 
 
+def test_few_labels_and_many_chains_pack_by_default(gpu, oracle):
+  """8 labels, 4928 chains in the launch: with at most 8 labels a 1-D table costs the packed step
+  little more than a band would, and 8 chains share a wavefront."""
+  from mplayers_amd import _lib
+  rng = np.random.default_rng(9)
+  B, H, W, L, n_dir, n_iter = 16, 150, 4, 8, 4, 2
+  ctx = (0.4 * np.minimum(np.arange(L), 2)).astype(np.float32)
+  unary = rng.random((B, 1, H, W, L)).astype(np.float32)
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  dcost = rng.standard_normal((B, 1, H, W, L)).astype(np.float32)
+  check_against_oracle(gpu, oracle, "ISGMR", n_dir, n_iter, unary, ctx, ew, dcost)
+  fwd = gpu.gpu_forward("ISGMR", unary, ctx, ew, n_dir, n_iter, 1.0)
+  run = lambda flags: gpu.gpu_backward("ISGMR", ctx, ew, dcost, fwd["msg_min_index"],
+                                       fwd["msg_norm_index"], 1.0, flags=flags)
+  default, always = run(0), run(_lib.F_PACKED_ALWAYS)
+  assert np.array_equal(default[2], always[2])  # (8-term sums: both kinds of scan give these bits)
+  assert np.array_equal(default[0], always[0])
+
+
 def test_set_option_rejects_unknown(gpu):
   from mplayers_amd import _lib
   with pytest.raises(RuntimeError):
