@@ -607,12 +607,15 @@ int packed_chains_per_wave(int B, int H, int W, int L, bool ctx2d, int64_t chain
   //  * 1-D tables, ISGMR, 3 iterations: min(k, 3) with 16 / 32 labels and 1280 chains 2.0 / 3.7
   //    against 0.73 / 0.88 ms; dense with 16 / 32 labels, 1280 chains 2.0 / 3.7 against 1.3 / 2.3
   //    and 10240 chains 5.2 / 15.0 against 9.7 / 18.2; 8 labels, 5120 chains, dense 1.42 against
-  //    1.62 and min(k, 3) 1.42 against 1.36; 4 labels, 5120 chains, dense 0.98 against 1.34.
+  //    1.62 and min(k, 3) 1.42 against 1.36; 4 labels, 5120 chains, dense 0.98 against 1.34;
+  //    min(k, 3) with 16 labels: 5120 chains 4.6 against 3.3, 10240 chains 5.2 against 6.4, 40960
+  //    chains 17.0 against 25.3 (TRWP, 10240 chains per launch: 21.1 against 25.2); with 12 labels
+  //    and 10240 chains 4.3 against 6.4; with 32 labels and 10240 chains 15.1 against 10.4.
   if (!always) {
     if (ctx2d) {
       if (chains < (L == 21 ? kPackedMinChains21 : kPackedMinChains)) return 0;
     } else {
-      if (L > kPackedMaxL1d || chains < kPackedMinChains1d) return 0;
+      if (L > 16 || chains < (L <= 8 ? kPackedMinChains1d8 : kPackedMinChains1d16)) return 0;
     }
   }
   int G = kWave / L;

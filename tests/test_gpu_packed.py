@@ -1,6 +1,6 @@
 """Scans with several chains per wavefront (at most 32 labels).  By default only launches with a
-2-D table and more than 1024 chains (2048 with 21 labels), or with at most 8 labels and more than
-4096 chains, take them, so the small cases are run with the policy forced (option value 2)
+2-D table and more than 1024 chains (2048 with 21 labels), or with a 1-D table of at most 8 / 16
+labels and more than 4096 / 8192 chains, take them, so the small cases are run with the policy forced (option value 2)
 and one case is large enough to take them on its own; every result is checked against the oracle
 exactly like the one-chain-per-wavefront kernels."""
 import numpy as np
