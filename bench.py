@@ -73,6 +73,10 @@ def parse():
                        "or column) for several read:write mixes (\"measured_stream_rates\")")
   ap.add_argument("--no-peak-probe", action="store_true",
                   help="leave the copy probes out of the default large-configuration run (profiler runs)")
+  ap.add_argument("--issue-probe", action="store_true",
+                  help="also report what instruction patterns cost a lone wavefront, in clocks per "
+                       "issue slot (under \"issue_costs\"): the bound of launches with fewer chains "
+                       "than the chip has SIMDs")
   ap.add_argument("--module-probe", action="store_true",
                   help="also time forward+backward through the nn.Module surface, which allocates "
                        "its buffers on every call as the reference's does (reported under "
@@ -207,6 +211,27 @@ def peak_probe(H, W, L, dev, reps=5):
       torch.cuda.synchronize()
       ms = start.elapsed_time(stop) / reps
       res["%s_%din_%dout_GBs" % (sname, n_in, n_out)] = round((n_in + n_out) * 4 * n / ms / 1e6, 1)
+  return res
+
+
+def issue_probe(dev):
+  """Clocks per issue slot of instruction patterns for a wavefront that has its SIMD to itself
+  (mpl_probe_issue): what bounds the scans of launches with fewer chains than the chip has SIMDs."""
+  import ctypes
+  import torch
+  from mplayers_amd import _lib
+  lib = _lib.load()
+  n = lib.mpl_probe_issue_count()
+  clocks = torch.zeros(n, dtype=torch.int64, device=dev)
+  stream = torch.cuda.current_stream().cuda_stream
+  _lib.check(lib.mpl_probe_issue(ctypes.c_void_p(clocks.data_ptr()), n, ctypes.c_void_p(stream)),
+             "probe_issue")
+  torch.cuda.synchronize()
+  c = clocks.cpu().tolist()
+  res = {"empty_region_clocks": c[0]}
+  for i in range(1, n):
+    slots = lib.mpl_probe_issue_slots(i)
+    res[lib.mpl_probe_issue_name(i).decode()] = round((c[i] - c[0]) / slots, 2)
   return res
 
 
@@ -472,6 +497,8 @@ def main():
   if a.peak_probe or (cfg["name"] == "C5" and a.scale == 1.0 and not a.no_peak_probe):
     # what this GPU sustains for traffic of the kernels' shapes, next to the published 8 TB/s
     out["measured_stream_rates"] = peak_probe(H, W, L, dev, reps=5 if a.peak_probe else 2)
+  if a.issue_probe:
+    out["issue_costs"] = issue_probe(dev)
   if a.module_probe and training:
     out["module_surface"] = module_probe(cfg, algs, unary, edge, dcost)
   if a.edge_probe:

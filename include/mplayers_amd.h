@@ -256,6 +256,18 @@ int mpl_mrf_energy(const mpl_shape* shape, int n_labelings, const float* unary,
 int mpl_probe_copy(int shape, int n_in, int n_out, const float* in, float* out, int height,
                    int width, int n_labels, void* stream);
 
+/* Issue probe (diagnostic, no counterpart in the reference): one wavefront, alone on its SIMD, runs
+ * a few hundred copies of each of mpl_probe_issue_count() instruction patterns between two reads of
+ * the shader clock and stores the elapsed clocks of pattern i in clocks[i] (device memory, room for
+ * n >= mpl_probe_issue_count() values; pattern 0 is an empty region, the overhead of the two reads).
+ * mpl_probe_issue_slots(i) is the number of issue slots pattern i was run for, idle slots
+ * included, mpl_probe_issue_name(i) what it is.  The scans of launches with fewer chains than the
+ * chip has SIMDs are bound by these costs. */
+int mpl_probe_issue_count(void);
+const char* mpl_probe_issue_name(int pattern);
+int mpl_probe_issue_slots(int pattern);
+int mpl_probe_issue(long long* clocks, int n, void* stream);
+
 /* Batched 2-D transpose src (batch, rows, cols) -> dst (batch, cols, rows), fp32: the layout change
  * between the network's (batch, labels, H, W) tensors and the kernels' (batch, H, W, labels), which
  * the reference's module does with permute().contiguous() (pytorch/MP_module.py:199,203,233).

@@ -1,4 +1,5 @@
-// Bandwidth probes: what the memory system sustains for traffic of the scans' shape.
+// Bandwidth probes: what the memory system sustains for traffic of the scans' shape; and, at the end
+// of the file, an issue probe: what instruction patterns cost a lone wavefront.
 //
 // The scan kernels are long-lived wavefronts, one per chain, that stream several planes in and out
 // one pixel vector at a time.  These kernels move the same bytes in the same shape without any of
@@ -87,6 +88,103 @@ void launch_probe(int shape, const float* in, float* out, int H, int W, int L, h
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Issue probe: what instruction patterns cost a wavefront that has its SIMD to itself.  One
+// wavefront runs a few hundred copies of each pattern between two reads of the shader clock; the
+// difference, less that of an empty region, divided by the number of issue slots is reported.
+// The scans of launches with fewer chains than the chip has SIMDs are bound by exactly these costs.
+// ------------------------------------------------------------------------------------------------
+struct IssuePattern {
+  const char* name;
+  int slots;  // instructions (idle slots included) between the two clock reads
+};
+const IssuePattern kIssuePatterns[] = {
+    {"empty region", 0},
+    {"vop2 add, independent", 480},
+    {"vop2 add, each needs the one before", 480},
+    {"vop2 multiply-add (v_fmac)", 480},
+    {"vop3 multiply-add (v_fma), three registers", 480},
+    {"vop3 multiply-add, two registers and a scalar", 480},
+    {"v_min3, three registers", 480},
+    {"comparison into a scalar mask", 480},
+    {"select on a scalar mask, registers", 480},
+    {"select on a scalar mask, inline constant", 480},
+    {"comparison, two idle slots, select (3 slots)", 480},
+    {"two comparisons and two selects interleaved (4 slots)", 480},
+    {"s_nop 0", 480},
+    {"s_nop 1", 480},
+    {"scalar add", 480},
+    {"v_readlane", 480},
+    {"two idle slots and a lane-shift minimum (2 slots)", 480},
+    {"lane-shift minimum and two independent adds (3 slots)", 480},
+    {"v_exp", 480},
+    {"v_rcp", 480},
+    {"ds_bpermute x8, one wait (9 slots)", 477},
+    {"ds_bpermute and wait (round trip, 2 slots)", 480},
+    {"ds_read_b32 and wait (round trip, 2 slots)", 480},
+    {"ds_add_f32, ds_wrxchg_rtn and wait, distinct addresses (3 slots)", 480},
+    {"ds_add_f32 of 64 lanes to one address and wait (2 slots)", 480},
+};
+constexpr int kNumIssuePatterns = (int)(sizeof(kIssuePatterns) / sizeof(kIssuePatterns[0]));
+
+#define MPL_ISSUE_TIMED(idx, body)                                                                \
+  {                                                                                               \
+    __builtin_amdgcn_s_barrier();                                                                 \
+    const long long t0 = clock64();                                                               \
+    asm volatile(body ::: "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "v18", "v19",  \
+                 "s44", "s45", "s46", "s47", "vcc", "memory");                                    \
+    const long long t1 = clock64();                                                               \
+    if (threadIdx.x == 0) out[idx] = t1 - t0;                                                     \
+  }
+
+__global__ void __launch_bounds__(kWave) issue_probe_kernel(long long* __restrict__ out) {
+  __shared__ float lds[256];
+  for (int i = threadIdx.x; i < 256; i += kWave) lds[i] = 0.f;
+  __syncthreads();
+  // v18: byte address of this lane's LDS word, v19: that of word 0 (no pattern writes them: an LDS
+  // access at a clobbered, unaligned address would fault); v10..v17: operands and results;
+  // s40..s43: masks and a scalar operand (whatever they hold: only the timing is read)
+  const unsigned own = (unsigned)(size_t)&lds[threadIdx.x], first = (unsigned)(size_t)&lds[0];
+  asm volatile(
+      "v_mov_b32 v18, %0\n v_mov_b32 v19, %1\n v_mov_b32 v10, 1.0\n v_mov_b32 v11, 1.0\n"
+      " v_mov_b32 v12, 1.0\n v_mov_b32 v13, 1.0\n v_mov_b32 v14, 1.0\n v_mov_b32 v15, 1.0\n"
+      " v_mov_b32 v16, 1.0\n v_mov_b32 v17, 1.0\n s_mov_b32 s40, 1\n s_mov_b32 s41, 1\n"
+      " s_mov_b32 s42, 1\n s_mov_b32 s43, 1"
+      :
+      : "v"(own), "v"(first)
+      : "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "v18", "v19", "s40", "s41", "s42",
+        "s43", "memory");
+  for (int rep = 0; rep < 2; ++rep) {  // (the second pass runs from a warm instruction cache)
+  MPL_ISSUE_TIMED(0, "")
+  MPL_ISSUE_TIMED(1, ".rept 120\n v_add_f32 v10, v10, v14\n v_add_f32 v11, v11, v14\n v_add_f32 v12, v12, v14\n v_add_f32 v13, v13, v14\n .endr")
+  MPL_ISSUE_TIMED(2, ".rept 480\n v_add_f32 v10, v10, v14\n .endr")
+  MPL_ISSUE_TIMED(3, ".rept 480\n v_fmac_f32 v11, v12, v13\n .endr")
+  MPL_ISSUE_TIMED(4, ".rept 480\n v_fma_f32 v10, v11, v12, v13\n .endr")
+  MPL_ISSUE_TIMED(5, ".rept 480\n v_fma_f32 v10, v11, v12, s40\n .endr")
+  MPL_ISSUE_TIMED(6, ".rept 480\n v_min3_f32 v10, v11, v12, v13\n .endr")
+  MPL_ISSUE_TIMED(7, ".rept 480\n v_cmp_eq_f32_e64 s[44:45], v10, v15\n .endr")
+  MPL_ISSUE_TIMED(8, ".rept 480\n v_cndmask_b32_e64 v10, v11, v12, s[40:41]\n .endr")
+  MPL_ISSUE_TIMED(9, ".rept 480\n v_cndmask_b32_e64 v10, v10, 3, s[40:41]\n .endr")
+  MPL_ISSUE_TIMED(10, ".rept 160\n v_cmp_eq_f32_e32 vcc, v10, v14\n s_nop 1\n v_cndmask_b32_e32 v16, 3, v16, vcc\n .endr")
+  MPL_ISSUE_TIMED(11, ".rept 120\n v_cmp_eq_f32_e64 s[44:45], v10, v14\n v_cmp_eq_f32_e64 s[46:47], v11, v14\n v_cndmask_b32_e64 v16, v16, 3, s[44:45]\n v_cndmask_b32_e64 v17, v17, 4, s[46:47]\n .endr")
+  MPL_ISSUE_TIMED(12, ".rept 480\n s_nop 0\n .endr")
+  MPL_ISSUE_TIMED(13, ".rept 480\n s_nop 1\n .endr")
+  MPL_ISSUE_TIMED(14, ".rept 480\n s_add_i32 s44, s40, 1\n .endr")
+  MPL_ISSUE_TIMED(15, ".rept 480\n v_readlane_b32 s44, v10, 3\n .endr")
+  MPL_ISSUE_TIMED(16, ".rept 240\n s_nop 1\n v_min_f32_dpp v10, v10, v10 row_shr:1 row_mask:0xf bank_mask:0xf\n .endr")
+  MPL_ISSUE_TIMED(17, ".rept 160\n v_min_f32_dpp v10, v10, v10 row_shr:1 row_mask:0xf bank_mask:0xf\n v_add_f32 v11, v11, v14\n v_add_f32 v12, v12, v14\n .endr")
+  MPL_ISSUE_TIMED(18, ".rept 480\n v_exp_f32 v10, v15\n .endr")
+  MPL_ISSUE_TIMED(19, ".rept 480\n v_rcp_f32 v10, v15\n .endr")
+  MPL_ISSUE_TIMED(20, ".rept 53\n ds_bpermute_b32 v10, v18, v15\n ds_bpermute_b32 v11, v18, v15\n ds_bpermute_b32 v12, v18, v15\n ds_bpermute_b32 v13, v18, v15\n ds_bpermute_b32 v10, v18, v15\n ds_bpermute_b32 v11, v18, v15\n ds_bpermute_b32 v12, v18, v15\n ds_bpermute_b32 v13, v18, v15\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(21, ".rept 240\n ds_bpermute_b32 v10, v18, v15\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(22, ".rept 240\n ds_read_b32 v10, v18\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(23, ".rept 160\n ds_add_f32 v18, v15\n ds_wrxchg_rtn_b32 v10, v18, v19\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(24, ".rept 240\n ds_add_f32 v19, v15\n s_waitcnt lgkmcnt(0)\n .endr")
+  }
+}
+#undef MPL_ISSUE_TIMED
+
 }  // namespace
 
 extern "C" {
@@ -112,6 +210,25 @@ int mpl_probe_copy(int shape, int n_in, int n_out, const float* in, float* out, 
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MPL_ELAUNCH, "probe_copy: %s", hipGetErrorString(e));
+  return MPL_OK;
+}
+
+int mpl_probe_issue_count(void) { return kNumIssuePatterns; }
+
+const char* mpl_probe_issue_name(int pattern) {
+  return pattern >= 0 && pattern < kNumIssuePatterns ? kIssuePatterns[pattern].name : "";
+}
+
+int mpl_probe_issue_slots(int pattern) {
+  return pattern >= 0 && pattern < kNumIssuePatterns ? kIssuePatterns[pattern].slots : -1;
+}
+
+int mpl_probe_issue(long long* clocks, int n, void* stream) {
+  if (clocks == nullptr) return fail(MPL_EINVAL, "probe_issue: null pointer");
+  if (n < kNumIssuePatterns) return fail(MPL_EINVAL, "probe_issue: room for %d results needed", kNumIssuePatterns);
+  issue_probe_kernel<<<1, kWave, 0, (hipStream_t)stream>>>(clocks);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MPL_ELAUNCH, "probe_issue: %s", hipGetErrorString(e));
   return MPL_OK;
 }
 

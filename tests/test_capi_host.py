@@ -222,6 +222,11 @@ def test_new_entry_points_validate_before_launching():
   assert lib.mpl_mrf_energy(ctypes.byref(shape), 0, one, one, null, one, one, null) == 0  # nothing to do
   assert lib.mpl_probe_copy(0, 2, 2, one, one, 4, 4, 8, null) != 0
   assert lib.mpl_probe_copy(0, 1, 1, one, one, 4, 4, 6, null) != 0
+  assert lib.mpl_probe_issue(null, 64, null) != 0
+  assert lib.mpl_probe_issue(one, 1, null) != 0
+  assert lib.mpl_probe_issue_count() > 1 and lib.mpl_probe_issue_slots(0) == 0
+  assert lib.mpl_probe_issue_slots(lib.mpl_probe_issue_count()) == -1
+  assert lib.mpl_probe_issue_name(1) != b"" and lib.mpl_probe_issue_name(-1) == b""
   assert lib.mpl_transpose(null, one, 1, 4, 4, null) != 0
   assert lib.mpl_transpose(one, one, 1, -1, 4, null) != 0
   assert lib.mpl_transpose(one, one, 0, 4, 4, null) == 0                                  # empty

@@ -230,6 +230,26 @@ def test_min_a_dir_and_initial_messages(gpu, oracle):
 
 
 @pytest.mark.gpu
+def test_issue_probe_reads_sane_costs(gpu):
+  """One plain vector instruction issues every 4 clocks for a lone wavefront and `s_nop 1` takes
+  the time of two: the unit in which the probe's other rows are read."""
+  import ctypes
+  import torch
+  from mplayers_amd import _lib
+  lib = _lib.load()
+  n = lib.mpl_probe_issue_count()
+  clocks = torch.zeros(n, dtype=torch.int64, device="cuda")
+  _lib.check(lib.mpl_probe_issue(ctypes.c_void_p(clocks.data_ptr()), n, None), "probe_issue")
+  torch.cuda.synchronize()
+  c = clocks.cpu().tolist()
+  cost = {lib.mpl_probe_issue_name(i).decode(): (c[i] - c[0]) / lib.mpl_probe_issue_slots(i)
+          for i in range(1, n)}
+  print(cost, flush=True)
+  assert 3.5 <= cost["vop2 add, independent"] <= 4.6
+  assert 7.0 <= cost["s_nop 1"] <= 9.0
+  assert all(v > 0 for v in cost.values())
+
+
 def test_copy_probe_moves_what_it_claims(gpu):
   """The bandwidth probe's kernels write the sum of their input planes (+ k for output plane k) to
   every element, whatever the access shape, and reject shapes they do not implement."""
