@@ -677,7 +677,7 @@ extern "C" {
 
 const char* mpl_last_error(void) { return g_err; }
 
-int mpl_version(void) { return 200; }
+int mpl_version(void) { return 201; }  // (2.01: MPL_F_FUSED_PAIRS_OFF, mpl_probe_issue)
 
 int mpl_set_option(int option, int value) {
   if (option == MPL_OPT_PACKED_SCANS) {
