@@ -283,7 +283,7 @@ const char* mpl_last_error(void);
  * these; the values are read atomically once per call.
  * MPL_OPT_PACKED_SCANS (default 1): launches with a 2-D table of at most 32 labels and more than
  * 1024 chains (2048 with 21 labels), and launches with a 1-D table of at most 8 labels and more than
- * 4096 chains or of at most 16 labels and more than 8192 chains, whose planes stay below 2 GiB, are scanned with several chains per wavefront; 0
+ * 6144 chains or of at most 16 labels and more than 10000 chains, whose planes stay below 2 GiB, are scanned with several chains per wavefront; 0
  * forces the one-chain-per-wavefront kernels, 2 packs whenever the label count (at most 32) allows
  * it.  The packed step scans every front label whatever the table, so it is not the default for
  * 1-D tables, which are nearly always bands; a caller whose 1-D tables of up to 32 labels are dense

@@ -536,16 +536,16 @@ constexpr int kPackedMaxL = 32;
 //  * its table is 2-D (a learned table, dense) and it has more chains than the 256 CUs have SIMDs;
 //    with 21 labels, whose one-chain-per-wavefront scans have a short step of their own, more
 //    chains than two wavefronts per SIMD,
-//  * its table is 1-D and it has at most 8 labels and more than 4096 chains, or at most 16 labels
-//    and more than 8192 chains.  The packed step is the dense one, L candidates per label, whatever
+//  * its table is 1-D and it has at most 8 labels and more than 6144 chains, or at most 16 labels
+//    and more than 10000 chains.  The packed step is the dense one, L candidates per label, whatever
 //    the table; nearly every 1-D table is a band (Potts, truncated linear or quadratic), whose step
 //    in the one-chain scans takes a few taps, and only the device knows which it is: these are the
 //    sizes from which packing pays for a band, too.  A caller with dense 1-D tables of up to 32
 //    labels and thousands of chains per launch passes MPL_F_PACKED_ALWAYS.
 constexpr int kPackedMinChains = 1025;
 constexpr int kPackedMinChains21 = 2049;
-constexpr int kPackedMinChains1d8 = 4097;    // at most 8 labels
-constexpr int kPackedMinChains1d16 = 8193;   // 9 to 16 labels
+constexpr int kPackedMinChains1d8 = 6145;    // at most 8 labels
+constexpr int kPackedMinChains1d16 = 10001;  // 9 to 16 labels
 // always: pack whatever the table and the number of chains (tests, comparisons, such callers)
 // chains per wavefront the packed scans would use for such a launch (below 2: they do not apply)
 int packed_chains_per_wave(int B, int H, int W, int L, bool ctx2d, int64_t chains, bool always);

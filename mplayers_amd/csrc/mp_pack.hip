@@ -610,7 +610,11 @@ int packed_chains_per_wave(int B, int H, int W, int L, bool ctx2d, int64_t chain
   //    1.62 and min(k, 3) 1.42 against 1.36; 4 labels, 5120 chains, dense 0.98 against 1.34;
   //    min(k, 3) with 16 labels: 5120 chains 4.6 against 3.3, 10240 chains 5.2 against 6.4, 40960
   //    chains 17.0 against 25.3 (TRWP, 10240 chains per launch: 21.1 against 25.2); with 12 labels
-  //    and 10240 chains 4.3 against 6.4; with 32 labels and 10240 chains 15.1 against 10.4.
+  //    and 10240 chains 4.3 against 6.4; with 32 labels and 10240 chains 15.1 against 10.4.  With
+  //    8 directions, whose diagonal chains are short, on 300 x 400: 8 labels, batch 1 (4196 chains)
+  //    1.05 against 0.61, batch 2 with 5 labels (8392 chains) 0.99 against 1.22, batch 4 (16784
+  //    chains) 1.40 against 2.02; 16 labels, batch 2 (8392 chains) 1.81 against 1.42, batch 4 2.11
+  //    against 2.56.
   if (!always) {
     if (ctx2d) {
       if (chains < (L == 21 ? kPackedMinChains21 : kPackedMinChains)) return 0;

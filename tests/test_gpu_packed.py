@@ -1,6 +1,6 @@
 """Scans with several chains per wavefront (at most 32 labels).  By default only launches with a
 2-D table and more than 1024 chains (2048 with 21 labels), or with a 1-D table of at most 8 / 16
-labels and more than 4096 / 8192 chains, take them, so the small cases are run with the policy forced (option value 2)
+labels and more than 6144 / 10000 chains, take them, so the small cases are run with the policy forced (option value 2)
 and one case is large enough to take them on its own; every result is checked against the oracle
 exactly like the one-chain-per-wavefront kernels."""
 import numpy as np
@@ -128,11 +128,11 @@ def test_band_table_of_many_chains_stays_unpacked(gpu, oracle):
 
 
 def test_few_labels_and_many_chains_pack_by_default(gpu, oracle):
-  """8 labels, 4928 chains in the launch: with at most 8 labels a 1-D table costs the packed step
+  """8 labels, 6528 chains in the launch: with at most 8 labels a 1-D table costs the packed step
   little more than a band would, and 8 chains share a wavefront."""
   from mplayers_amd import _lib
   rng = np.random.default_rng(9)
-  B, H, W, L, n_dir, n_iter = 16, 150, 4, 8, 4, 2
+  B, H, W, L, n_dir, n_iter = 16, 200, 4, 8, 4, 2
   ctx = (0.4 * np.minimum(np.arange(L), 2)).astype(np.float32)
   unary = rng.random((B, 1, H, W, L)).astype(np.float32)
   ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
