@@ -183,13 +183,13 @@ def peak_probe(H, W, L, dev, reps=5):
   """What this GPU sustains on planes of the workload's size, in GB/s of bytes moved: one-pass
   streaming kernels (the shape of the element-wise passes) and long-lived one-wavefront-per-chain
   kernels that move n_in planes in and n_out planes out pixel by pixel (the shape of the scans,
-  without their arithmetic): mpl_probe_copy."""
+  without their arithmetic): mplp_copy of the probe library."""
   import ctypes
   import torch
-  from mplayers_amd import _lib
+  from mplayers_amd import _probe
   if L % 4:
     return {"note": "the probe needs a label count that is a multiple of 4"}
-  lib = _lib.load()
+  lib = _probe.load()
   n = H * W * L
   src = torch.zeros(4 * n, dtype=torch.float32, device=dev)
   dst = torch.empty(3 * n, dtype=torch.float32, device=dev)
@@ -199,9 +199,9 @@ def peak_probe(H, W, L, dev, reps=5):
   for shape, sname in ((2, "stream"), (0, "rows"), (1, "columns")):
     for n_in, n_out in ((1, 1), (3, 0), (1, 3), (3, 2), (4, 3)):
       def run():
-        _lib.check(lib.mpl_probe_copy(shape, n_in, n_out, ctypes.c_void_p(src.data_ptr()),
-                                      ctypes.c_void_p(dst.data_ptr()), H, W, L,
-                                      ctypes.c_void_p(stream)), "probe_copy")
+        _probe.check(lib.mplp_copy(shape, n_in, n_out, ctypes.c_void_p(src.data_ptr()),
+                                   ctypes.c_void_p(dst.data_ptr()), H, W, L,
+                                   ctypes.c_void_p(stream)), "probe_copy")
       run()
       torch.cuda.synchronize()
       start.record()
@@ -216,22 +216,23 @@ def peak_probe(H, W, L, dev, reps=5):
 
 def issue_probe(dev):
   """Clocks per issue slot of instruction patterns for a wavefront that has its SIMD to itself
-  (mpl_probe_issue): what bounds the scans of launches with fewer chains than the chip has SIMDs."""
+  (mplp_issue of the probe library): what bounds the scans of launches with fewer chains than the
+  chip has SIMDs."""
   import ctypes
   import torch
-  from mplayers_amd import _lib
-  lib = _lib.load()
-  n = lib.mpl_probe_issue_count()
+  from mplayers_amd import _probe
+  lib = _probe.load()
+  n = lib.mplp_issue_count()
   clocks = torch.zeros(n, dtype=torch.int64, device=dev)
   stream = torch.cuda.current_stream().cuda_stream
-  _lib.check(lib.mpl_probe_issue(ctypes.c_void_p(clocks.data_ptr()), n, ctypes.c_void_p(stream)),
-             "probe_issue")
+  _probe.check(lib.mplp_issue(ctypes.c_void_p(clocks.data_ptr()), n, ctypes.c_void_p(stream)),
+               "probe_issue")
   torch.cuda.synchronize()
   c = clocks.cpu().tolist()
   res = {"empty_region_clocks": c[0]}
   for i in range(1, n):
-    slots = lib.mpl_probe_issue_slots(i)
-    res[lib.mpl_probe_issue_name(i).decode()] = round((c[i] - c[0]) / slots, 2)
+    slots = lib.mplp_issue_slots(i)
+    res[lib.mplp_issue_name(i).decode()] = round((c[i] - c[0]) / slots, 2)
   return res
 
 

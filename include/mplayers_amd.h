@@ -5,7 +5,8 @@
  * label axis innermost.  The caller owns and allocates every buffer, exactly as the reference's
  * operators require (pytorch/MP_module.py:26-50, 65-78); buffers marked "zero-filled" must come
  * in zeroed, as the reference's caller provides them.  `stream` is a hipStream_t (NULL = the
- * default stream).  Nothing here allocates device memory or synchronises with the host.
+ * default stream).  Nothing here allocates device memory, and nothing but mpl_profile_end(), which
+ * waits for the events of its bracket, synchronises with the host.
  *
  * Shapes:  B = batch * n_cv,  P = B*H*W pixels,  N = P*L.
  *   unary, cost_final, unary_update, dcost_final, dunary, dunary_update   (B, H, W, L)  fp32
@@ -65,8 +66,9 @@ typedef struct mpl_shape {
  * TRWP_hard_soft build does (MPLayers/TRWP_hard_soft/TRWP_backward.cu:104-111, 188-195, 258-265);
  * the TRWP and ISGMR builds skip them (MPLayers/TRWP/TRWP_backward.cu:111-112). */
 #define MPL_F_FUSED_PAIRS_OFF 0x20u
-/* TRWP calls: one launch per direction even where a launch has so few chains (at most 1024) that
- * the library would run both sweeps of a pair of opposite directions in one. */
+/* TRWP calls: one launch per direction even where a launch has so few chains (at most one per
+ * SIMD of the device) that the library would run both sweeps of a pair of opposite directions in
+ * one. */
 #define MPL_F_ALL 0x3fu
 
 /* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.
@@ -145,15 +147,13 @@ int mpl_soft_weighted_message_back(int n_trees, int n_disp, const float* dmessag
                                    const float* message, const uint8_t* message_soft_sum_min_ind,
                                    float* dmessage, void* stream);
 
-/* Device check of the wavefront primitives the kernels are built on (cross-lane shifts, min/sum
- * reductions, ballots).  out: 8 host ints, out[0] == 1 when every check passed.  Synchronises. */
-int mpl_selftest_wave_ops(int* out_host);
-
 /* Per-kernel timing for benchmarks (no counterpart in the reference, which times whole calls with
  * time.time(), MPLayers/main.py:271-313).  Between mpl_profile_begin() and mpl_profile_end() every
  * kernel launch of this library is bracketed by HIP events on its own stream; mpl_profile_end()
  * waits for them and fills stats[kind] for kind < n_stats.  Events cost a few microseconds per
- * launch; nothing is recorded outside such a bracket.  One bracket at a time per process. */
+ * launch; nothing is recorded outside such a bracket.  One bracket at a time per process: the
+ * bracket is process-wide state (calls on any thread and stream between begin and end are
+ * recorded into it), so a second begin before the end restarts it. */
 #define MPL_KERNEL_FWD_SWEEP 0      /* forward scan of one direction (TRWP) */
 #define MPL_KERNEL_BWD_SWEEP 1      /* reverse scan of one direction (TRWP) */
 #define MPL_KERNEL_BELIEF 2         /* S = unary + sum of messages (TRWP, once per call) */
@@ -244,30 +244,6 @@ int mpl_mrf_energy(const mpl_shape* shape, int n_labelings, const float* unary,
                    const float* context, const float* edge_weights, const uint8_t* labels,
                    double* energy, void* stream);
 
-/* Bandwidth probe (diagnostic, no counterpart in the reference): moves n_in planes of
- * (height, width, n_labels) fp32 from `in` to n_out planes at `out` (sum of the inputs, + k for
- * plane k) in the scans' access shape -- one long-lived wavefront per row (MPL_PROBE_ROWS) or per
- * column (MPL_PROBE_COLUMNS), one pixel vector per step, eight pixels in flight -- or as a one-pass
- * streaming kernel (MPL_PROBE_STREAM).  `in` holds n_in planes, `out` max(n_out, 1); (n_in, n_out)
- * is one of (1,1) (1,3) (3,0) (3,2) (4,3); n_labels a multiple of 4. */
-#define MPL_PROBE_ROWS 0
-#define MPL_PROBE_COLUMNS 1
-#define MPL_PROBE_STREAM 2
-int mpl_probe_copy(int shape, int n_in, int n_out, const float* in, float* out, int height,
-                   int width, int n_labels, void* stream);
-
-/* Issue probe (diagnostic, no counterpart in the reference): one wavefront, alone on its SIMD, runs
- * a few hundred copies of each of mpl_probe_issue_count() instruction patterns between two reads of
- * the shader clock and stores the elapsed clocks of pattern i in clocks[i] (device memory, room for
- * n >= mpl_probe_issue_count() values; pattern 0 is an empty region, the overhead of the two reads).
- * mpl_probe_issue_slots(i) is the number of issue slots pattern i was run for, idle slots
- * included, mpl_probe_issue_name(i) what it is.  The scans of launches with fewer chains than the
- * chip has SIMDs are bound by these costs. */
-int mpl_probe_issue_count(void);
-const char* mpl_probe_issue_name(int pattern);
-int mpl_probe_issue_slots(int pattern);
-int mpl_probe_issue(long long* clocks, int n, void* stream);
-
 /* Batched 2-D transpose src (batch, rows, cols) -> dst (batch, cols, rows), fp32: the layout change
  * between the network's (batch, labels, H, W) tensors and the kernels' (batch, H, W, labels), which
  * the reference's module does with permute().contiguous() (pytorch/MP_module.py:199,203,233).
@@ -281,9 +257,11 @@ const char* mpl_last_error(void);
 /* Process-wide defaults of what the per-call flags MPL_F_PACKED_* and MPL_F_FUSED_U_OFF select
  * (no counterpart in the reference).  A call that passes one of those flags is not affected by
  * these; the values are read atomically once per call.
- * MPL_OPT_PACKED_SCANS (default 1): launches with a 2-D table of at most 32 labels and more than
- * 1024 chains (2048 with 21 labels), and launches with a 1-D table of at most 8 labels and more than
- * 6144 chains or of at most 16 labels and more than 10000 chains, whose planes stay below 2 GiB, are scanned with several chains per wavefront; 0
+ * MPL_OPT_PACKED_SCANS (default 1): launches with a 2-D table of at most 32 labels and more
+ * chains than the device has SIMDs (four per compute unit; twice as many with 21 labels), and
+ * launches with a 1-D table of at most 8 labels and more than 6 chains per SIMD or of at most 16
+ * labels and more than 9, whose planes stay below 2 GiB, are scanned with several chains per
+ * wavefront (on an MI355X, 1024 SIMDs: more than 1024 / 2048 / 6144 / 9216 chains); 0
  * forces the one-chain-per-wavefront kernels, 2 packs whenever the label count (at most 32) allows
  * it.  The packed step scans every front label whatever the table, so it is not the default for
  * 1-D tables, which are nearly always bands; a caller whose 1-D tables of up to 32 labels are dense
@@ -295,6 +273,15 @@ const char* mpl_last_error(void);
  * storing it in a pass of its own; 0 always runs that pass (results agree to the parity tolerance,
  * bit for bit on inputs whose sums do not round). */
 #define MPL_OPT_FUSED_U 1
+/* MPL_OPT_BELIEF_REBUILD (default MPL_BELIEF_REBUILD_DEFAULT): the TRWP forward calls, hard and
+ * soft-weighted, keep unary + the sum of all messages as a plane that every sweep updates by
+ * differences, where the reference re-sums it before every sweep (TRWP_forward.cu:60-80).  Every
+ * `value` iterations the plane is re-summed from the messages as the reference sums them, so the
+ * rounding of at most that many iterations' updates is ever in it; 0: never; -1: the library
+ * chooses (calls of at most 64 direction sweeps, n_iter * n_dir, are not re-summed; longer ones
+ * every max(1, 32 / n_dir) iterations). */
+#define MPL_OPT_BELIEF_REBUILD 2
+#define MPL_BELIEF_REBUILD_DEFAULT (-1)
 int mpl_set_option(int option, int value);
 
 /* Library version: major * 100 + minor. */

@@ -1,4 +1,6 @@
-"""Compiles the HIP sources under csrc/ into libmplayers_hip.so (gfx950 only) with hipcc.
+"""Compiles the HIP sources under csrc/ into libmplayers_hip.so (gfx950 only) with hipcc, and the
+measurement probes (csrc/mp_probe.hip) into libmplayers_probe.so, which only the benchmark and the
+tests load.
 
 The scan kernels are instantiated once per R (labels per lane, 1..4); each instantiation is its
 own translation unit so that they compile in parallel.
@@ -12,6 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libmplayers_hip.so")
+PROBE_LIB = os.path.join(HERE, "libmplayers_probe.so")
+PROBE_UNITS = ("mp_probe",)  # objects of the probe library; every other unit is the product's
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-munsafe-fp-atomics", "-fno-honor-nans",
@@ -58,13 +62,26 @@ def build(verbose=False, extra_flags=(), lib_path=LIB, jobs=None):
         print(" ".join(cmd))
         if out.strip():
           print(out)
-  link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", lib_path]
-  out = _run(link)
-  if verbose:
-    print(" ".join(link))
-    if out.strip():
-      print(out)
+  link(lib_path=lib_path, verbose=verbose)
   return lib_path
+
+
+def link(lib_path=LIB, verbose=False):
+  """Links the objects that are there into the product library and the probe library."""
+  hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+  obj_dir = OBJ if lib_path == LIB else lib_path + ".build"
+  probe_path = PROBE_LIB if lib_path == LIB else lib_path.replace(".so", "_probe.so")
+  names = [name for name, _, _ in _units()]
+  groups = ((lib_path, [n for n in names if n not in PROBE_UNITS], ["-lpthread"]),
+            (probe_path, [n for n in names if n in PROBE_UNITS], []))
+  for path, members, libs in groups:
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + \
+        [os.path.join(obj_dir, n + ".o") for n in members] + libs + ["-o", path]
+    out = _run(cmd)
+    if verbose:
+      print(" ".join(cmd))
+      if out.strip():
+        print(out)
 
 
 if __name__ == "__main__":

@@ -6,12 +6,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hip.so"))
 
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
-           "mpl_selftest_wave_ops", "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
+           "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
            "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_edge_shift_static",
            "mpl_trwp_soft_forward",
            "mpl_trwp_soft_backward", "mpl_soft_weighted_message", "mpl_soft_weighted_message_back", "mpl_set_option",
-           "mpl_stereo_data_cost", "mpl_gradient_cues", "mpl_mrf_energy", "mpl_probe_copy", "mpl_transpose",
-           "mpl_probe_issue", "mpl_probe_issue_count", "mpl_probe_issue_name", "mpl_probe_issue_slots")
+           "mpl_stereo_data_cost", "mpl_gradient_cues", "mpl_mrf_energy", "mpl_transpose")
 
 KERNEL_KINDS = ("fwd_sweep", "bwd_sweep", "belief", "aggregate", "label", "combine", "other",
                 "fwd_sweep_all", "bwd_sweep_all", "unary_all")
@@ -66,20 +65,13 @@ def load():
   lib.mpl_stereo_data_cost.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, ci, vp, vp]
   lib.mpl_gradient_cues.argtypes = [vp, ci, ci, ci, ci, cf, vp, vp, vp]
   lib.mpl_mrf_energy.argtypes = [sp, ci, vp, vp, vp, vp, vp, vp]
-  lib.mpl_probe_copy.argtypes = [ci, ci, ci, vp, vp, ci, ci, ci, vp]
   lib.mpl_transpose.argtypes = [vp, vp, ci, ctypes.c_int64, ctypes.c_int64, vp]
-  lib.mpl_probe_issue.argtypes = [vp, ci, vp]
-  lib.mpl_probe_issue_count.argtypes = []
-  lib.mpl_probe_issue_name.argtypes = [ci]
-  lib.mpl_probe_issue_slots.argtypes = [ci]
-  lib.mpl_selftest_wave_ops.argtypes = [ctypes.POINTER(ci)]
   lib.mpl_n_chains.argtypes = [ci, ci, ci]
   lib.mpl_profile_begin.argtypes = []
   lib.mpl_profile_end.argtypes = [ctypes.POINTER(KernelStat), ci]
   for name in SYMBOLS:
     getattr(lib, name).restype = ci
   lib.mpl_last_error.restype = ctypes.c_char_p
-  lib.mpl_probe_issue_name.restype = ctypes.c_char_p
   if lib.mpl_version() // 100 != 2:
     raise RuntimeError("libmplayers_hip.so has ABI version %d, this package needs 2xx: rebuild it "
                        "with `python -m mplayers_amd._build`" % lib.mpl_version())
@@ -95,6 +87,8 @@ def load():
 
 OPT_PACKED_SCANS = 0
 OPT_FUSED_U = 1
+OPT_BELIEF_REBUILD = 2
+BELIEF_REBUILD_DEFAULT = -1
 
 
 def set_option(option, value):

@@ -399,41 +399,6 @@ __global__ void __launch_bounds__(256) isgmr_combine_kernel(const float* X, floa
 }
 
 // ------------------------------------------------------------------------------------------------
-// wave-primitive self test
-// ------------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(kWave) selftest_kernel(int* out) {
-  const int lane = threadIdx.x;
-  int ok = 1;
-  float x = (float)(lane * 3 % 17) + 100.f;
-  float up = wave_shl1(x, -1.f);
-  float dn = wave_shr1(x, -2.f);
-  float eu = lane < 63 ? (float)((lane + 1) * 3 % 17) + 100.f : -1.f;
-  float ed = lane > 0 ? (float)((lane - 1) * 3 % 17) + 100.f : -2.f;
-  if (up != eu || dn != ed) ok = 0;
-  float y = (float)((lane * 37 + 11) % 64);  // a permutation of 0..63
-  if (wave_min(y) != 0.f) ok = 0;
-  for (int special = 0; special < 64; special += 9)  // the minimum sits in every row and bank
-    if (wave_min(y + (lane == special ? -100.f : 0.f)) != (float)((special * 37 + 11) % 64) - 100.f)
-      ok = 0;
-  if (wave_min_fast(y) != 0.f) ok = 0;
-  for (int special = 0; special < 64; special += 7)
-    if (wave_min_fast(y + (lane == special ? -100.f : 0.f)) != (float)((special * 37 + 11) % 64) - 100.f)
-      ok = 0;
-  if (wave_min_fast(lane < 21 ? (float)(30 - lane) : INFINITY) != 10.f) ok = 0;
-  if (wave_sum((float)lane) != 2016.f) ok = 0;
-  bool pr[2] = {lane == 5 || lane == 40, lane == 40};
-  if (last_label<2>(pr, -1) != 81) ok = 0;
-  bool pn[2] = {false, false};
-  if (last_label<2>(pn, -7) != -7) ok = 0;
-  uint64_t b = ballot(ok != 0);
-  if (lane == 0) {
-    out[0] = (b == ~0ull) ? 1 : 0;
-    out[1] = (int)(b & 0xffffffffu);
-    out[2] = (int)(b >> 32);
-  }
-}
-
-// ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
 thread_local char g_err[512] = "";
@@ -446,7 +411,7 @@ struct ProfRec {
   hipEvent_t start, stop;
 };
 struct Profiler {
-  bool on = false;
+  std::atomic<bool> on{false};
   std::vector<ProfRec> recs;
   std::vector<hipEvent_t> pool;
   hipEvent_t get_event() {
@@ -467,7 +432,7 @@ struct Timed {
   hipStream_t st;
   hipEvent_t stop = nullptr;
   Timed(int kind, hipStream_t s, int sweeps = 1) : st(s) {
-    if (!g_prof.on) return;
+    if (!g_prof.on.load(std::memory_order_acquire)) return;
     std::lock_guard<std::mutex> lk(g_prof_mu);
     ProfRec r;
     r.kind = kind;
@@ -561,6 +526,7 @@ int labels_per_lane(int L) { return (L + kWave - 1) / kWave; }
 // process defaults of the per-call choices (mpl_set_option); a call reads them once
 std::atomic<int> g_packed_scans{1};  // MPL_OPT_PACKED_SCANS: 0 off, 1 by chain count, 2 always
 std::atomic<int> g_fused_u{1};       // MPL_OPT_FUSED_U
+std::atomic<int> g_belief_rebuild{MPL_BELIEF_REBUILD_DEFAULT};  // MPL_OPT_BELIEF_REBUILD
 
 // what one call does, from its flags and the process defaults
 struct CallOpts {
@@ -580,24 +546,31 @@ int read_flags(unsigned flags, const char* what, CallOpts* o) {
   return MPL_OK;
 }
 
-// TRWP launches of at most this many wavefronts (at most one per SIMD) run both sweeps of a pair of
-// opposite directions in one launch
-constexpr int kFusedPairMaxChains = 1024;
-
-// wavefronts of a one-direction launch: one per chain, or one per group of chains where the packed
-// scans take the launch
+// Chains per wavefront of the launch described by p (its directions filled in): the one place where
+// a launch is given to the packed scans (>= 2) or to the one-chain-per-wavefront kernels (0).
+// Everything that depends on that choice (the launcher, the number of wavefronts, whether the
+// Jacobi scans form U themselves) reads p.pack.
 template <typename Params>
-int launch_waves(const mpl_shape* s, const Params& p, const CallOpts& o) {
-  const int chains = p.block_prefix[p.n_dirs];
-  const int G = o.packed ? packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp,
-                                                  s->ctx2d != 0, chains, o.packed == 2)
-                         : 0;
-  return G >= 2 ? (chains + G - 1) / G : chains;
+int decide_pack(const mpl_shape* s, const Params& p, const CallOpts& o) {
+  if (!o.packed) return 0;
+  const int G = packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp, s->ctx2d != 0,
+                                       p.block_prefix[p.n_dirs], o.packed == 2);
+  return G >= 2 ? G : 0;
 }
 
-void launch_fwd(const SweepParams& p, bool train, bool jacobi, const CallOpts& o, hipStream_t st) {
+// wavefronts of a one-direction launch: one per chain, or one per group of p.pack chains
+template <typename Params>
+int launch_waves(const Params& p) {
+  const int chains = p.block_prefix[p.n_dirs];
+  return p.pack >= 2 ? (chains + p.pack - 1) / p.pack : chains;
+}
+
+void launch_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_FWD_SWEEP_ALL : MPL_KERNEL_FWD_SWEEP, st, p.fused_pair ? 2 : 1);
-  if (o.packed && launch_packed_fwd(p, train, jacobi, o.packed == 2, st)) return;
+  if (p.pack >= 2) {
+    launch_packed_fwd(p, train, jacobi, p.pack, st);  // (u_fused is never set together with pack)
+    return;
+  }
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_fwd<1>(p, train, jacobi, st); break;
     case 2: launch_sweep_fwd<2>(p, train, jacobi, st); break;
@@ -606,9 +579,12 @@ void launch_fwd(const SweepParams& p, bool train, bool jacobi, const CallOpts& o
   }
 }
 
-void launch_bwd(const BackParams& p, bool jacobi, const CallOpts& o, hipStream_t st) {
+void launch_bwd(const BackParams& p, bool jacobi, hipStream_t st) {
   Timed timed(jacobi ? MPL_KERNEL_BWD_SWEEP_ALL : MPL_KERNEL_BWD_SWEEP, st, p.fused_pair ? 2 : 1);
-  if (o.packed && launch_packed_bwd(p, jacobi, o.packed == 2, st)) return;
+  if (p.pack >= 2) {
+    launch_packed_bwd(p, jacobi, p.pack, st);
+    return;
+  }
   switch (labels_per_lane(p.L)) {
     case 1: launch_sweep_bwd<1>(p, jacobi, st); break;
     case 2: launch_sweep_bwd<2>(p, jacobi, st); break;
@@ -647,6 +623,32 @@ void zero_fill(float* dst, int64_t n, hipStream_t st) {
   zero_fill_kernel<<<(int)blocks, 256, 0, st>>>(dst, n);
 }
 
+// The sweeps keep the belief plane up to date by differences, S <- (S - m_old) + m_new, where the
+// reference re-sums unary + sum_k m_k before every sweep (UpdateUnaryKernel, TRWP_forward.cu:60-80):
+// the rounding of each update stays in the plane.  Between two iterations the plane holds S itself,
+// so it can be re-summed there exactly as the reference sums it, which bounds the drift of long
+// runs (the 50 iterations of energy minimisation) at what a few iterations accumulate.
+// Iterations between two re-summations for a call (0: none).  Left to the library (-1), calls of at
+// most kShortCallSweeps direction sweeps are not re-summed (what they accumulate is below the
+// rounding of the reference's own fp32 sums), longer ones whenever kSweepsPerRebuild sweeps have
+// passed.
+constexpr int kShortCallSweeps = 64;
+constexpr int kSweepsPerRebuild = 32;
+int belief_rebuild_interval(int n_dir, int n_iter) {
+  const int opt = g_belief_rebuild.load(std::memory_order_relaxed);
+  if (opt >= 0) return opt;
+  if ((int64_t)n_dir * n_iter <= kShortCallSweeps) return 0;
+  return kSweepsPerRebuild / n_dir > 1 ? kSweepsPerRebuild / n_dir : 1;
+}
+
+void rebuild_belief(const mpl_shape* s, const float* unary, const float* msg, float* S,
+                    hipStream_t st) {
+  Timed timed(MPL_KERNEL_BELIEF, st);
+  const int64_t N = (int64_t)s->batch * s->height * s->width * s->n_disp;
+  const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(S);
+  MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, S, (int*)nullptr);
+}
+
 // cost_final is not written before the final aggregation, so its first bytes carry the context
 // descriptor during the sweeps (no allocation, no state shared between streams).
 const CtxDesc* make_desc(const mpl_shape* s, const float* ctx, float* cost_final, hipStream_t st) {
@@ -661,6 +663,38 @@ const CtxDesc* make_desc(const mpl_shape* s, const float* ctx, float* cost_final
 }  // namespace
 
 namespace mpl {
+// SIMDs of the current device: four per compute unit.  Without a device (argument validation on a
+// host that has none) the MI355X's 256 compute units are assumed.
+const LaunchPolicy& launch_policy() {
+  constexpr int kMaxDevices = 64;
+  static LaunchPolicy table[kMaxDevices];
+  static std::atomic<int> ready[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+  if (ready[dev].load(std::memory_order_acquire) == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+      (void)hipGetLastError();
+      cus = 256;
+    }
+    LaunchPolicy pol;
+    pol.n_simd = 4 * cus;
+    pol.fused_pair_max_waves = pol.n_simd;
+    pol.packed_min_chains = pol.n_simd + 1;
+    pol.packed_min_chains21 = 2 * pol.n_simd + 1;
+    pol.packed_min_chains_1d8 = 6 * pol.n_simd + 1;
+    pol.packed_min_chains_1d16 = 9 * pol.n_simd + 1;
+    pol.direct_max_chains = 2 * pol.n_simd;
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lk(mu);
+    if (ready[dev].load(std::memory_order_relaxed) == 0) {
+      table[dev] = pol;
+      ready[dev].store(1, std::memory_order_release);
+    }
+  }
+  return table[dev];
+}
+
 int fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -677,7 +711,7 @@ extern "C" {
 
 const char* mpl_last_error(void) { return g_err; }
 
-int mpl_version(void) { return 201; }  // (2.01: MPL_F_FUSED_PAIRS_OFF, mpl_probe_issue)
+int mpl_version(void) { return 210; }  // (2.10: the probes left the library; MPL_OPT_BELIEF_REBUILD; CPU forward)
 
 int mpl_set_option(int option, int value) {
   if (option == MPL_OPT_PACKED_SCANS) {
@@ -690,6 +724,11 @@ int mpl_set_option(int option, int value) {
     g_fused_u.store(value, std::memory_order_relaxed);
     return MPL_OK;
   }
+  if (option == MPL_OPT_BELIEF_REBUILD) {
+    if (value < -1) return fail(MPL_EINVAL, "set_option: the belief rebuild interval is >= -1");
+    g_belief_rebuild.store(value, std::memory_order_relaxed);
+    return MPL_OK;
+  }
   return fail(MPL_EINVAL, "set_option: unknown option %d", option);
 }
 
@@ -700,13 +739,13 @@ int mpl_profile_begin(void) {
     g_prof.pool.push_back(r.stop);
   }
   g_prof.recs.clear();
-  g_prof.on = true;
+  g_prof.on.store(true, std::memory_order_release);
   return MPL_OK;
 }
 
 int mpl_profile_end(mpl_kernel_stat* stats, int n_stats) {
   std::lock_guard<std::mutex> lk(g_prof_mu);
-  g_prof.on = false;
+  g_prof.on.store(false, std::memory_order_release);
   for (int i = 0; i < n_stats; ++i) {
     stats[i].launches = 0;
     stats[i].total_ms = 0.0;
@@ -732,19 +771,6 @@ int mpl_profile_end(mpl_kernel_stat* stats, int n_stats) {
 int mpl_n_chains(int dir, int height, int width) {
   if (dir < 0 || dir >= kMaxDirs || height < 1 || width < 1) return -1;
   return make_dir(dir, height, width).n_chains;
-}
-
-int mpl_selftest_wave_ops(int* out_host) {
-  if (out_host == nullptr) return fail(MPL_EINVAL, "out_host is null");
-  int* d = nullptr;
-  if (hipMalloc(&d, 8 * sizeof(int)) != hipSuccess) return fail(MPL_ELAUNCH, "hipMalloc failed");
-  (void)hipMemset(d, 0, 8 * sizeof(int));
-  selftest_kernel<<<1, kWave>>>(d);
-  hipError_t e = hipDeviceSynchronize();
-  if (e == hipSuccess) e = hipMemcpy(out_host, d, 8 * sizeof(int), hipMemcpyDeviceToHost);
-  (void)hipFree(d);
-  if (e != hipSuccess) return fail(MPL_ELAUNCH, "selftest: %s", hipGetErrorString(e));
-  return MPL_OK;
 }
 
 int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
@@ -784,9 +810,12 @@ int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
   p.belief_out = unary_update;
   p.msg_in = msg;
   p.msg_out = msg;
+  const int rebuild = belief_rebuild_interval(s->n_dir, n_iter);
   for (int it = 0; it < n_iter; ++it) {
+    if (rebuild > 0 && it > 0 && it % rebuild == 0) rebuild_belief(s, unary, msg, unary_update, st);
     for (int d = 0; d < s->n_dir; ++d) {  // Gauss-Seidel over directions: TRWP_forward.cu:440-518
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
+      p.pack = decide_pack(s, p, opts);
       p.first_iter = (it == 0);
       p.pair_q = 1;
       p.belief = (uninit && it == 0 && d <= 1) ? unary : unary_update;
@@ -798,13 +827,13 @@ int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
       p.skip_s_store = skip_s(d);
       // few chains: the wavefront of a chain sweeps d and then d + 1 (the same pixels in reverse)
       p.fused_pair = (opts.fused_pairs && !(d & 1) &&
-                      launch_waves(s, p, opts) <= kFusedPairMaxChains) ? 1 : 0;
+                      launch_waves(p) <= launch_policy().fused_pair_max_waves) ? 1 : 0;
       p.skip_s_store2 = skip_s(d + 1);
       if (train) {
         p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
         p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       }
-      launch_fwd(p, train, false, opts, st);
+      launch_fwd(p, train, false, st);
       if (p.fused_pair) ++d;
     }
     if (label_all) {
@@ -857,10 +886,8 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
   // more directions the scans would read more than that pass moves.  (Not where the packed scans
   // of small label counts run: they are bound by the instructions of a step, and two more loads
   // per step cost them more than the pass.)
-  const bool packed_runs =
-      opts.packed && packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp, s->ctx2d != 0,
-                                            p.block_prefix[p.n_dirs], opts.packed == 2) >= 2;
-  const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && !packed_runs;
+  p.pack = decide_pack(s, p, opts);
+  const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && p.pack == 0;
   if (msg_uninit && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {
@@ -896,7 +923,7 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
       p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
     }
-    launch_fwd(p, train, true, opts, st);
+    launch_fwd(p, train, true, st);
     if (label_all) {
       Timed timed(MPL_KERNEL_LABEL, st);
       launch_labels(unary, nxt, s->n_dir, P, s->n_disp, factor, enable_min_a_dir, label_all + it * P, st);
@@ -949,6 +976,7 @@ int mpl_trwp_backward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
   for (int it = n_iter - 1; it >= 0; --it) {
     for (int d = s->n_dir - 1; d >= 0; --d) {  // TRWP_backward.cu:337-424
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
+      p.pack = decide_pack(s, p, opts);
       p.a_in = first ? dcost_final : dunary;  // CostAggregateKernelBack: every g_k starts as dcost
       p.first_touch = (it == n_iter - 1) && (d & 1);
       p.inv_from_a = (d & 1) ? 0 : 1;  // the launch before an even direction swept d + 1 = d ^ 1
@@ -959,9 +987,9 @@ int mpl_trwp_backward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       // few chains: the wavefront of a chain walks d (odd) and then d - 1 (same pixels, reversed)
       p.fused_pair = (opts.fused_pairs && (d & 1) &&
-                      launch_waves(s, p, opts) <= kFusedPairMaxChains) ? 1 : 0;
+                      launch_waves(p) <= launch_policy().fused_pair_max_waves) ? 1 : 0;
       p.skip_h2 = (it == 0) ? 1 : 0;
-      launch_bwd(p, false, opts, st);
+      launch_bwd(p, false, st);
       first = false;
       if (p.fused_pair) --d;
     }
@@ -1013,6 +1041,7 @@ int mpl_isgmr_backward(const mpl_shape* s, unsigned flags, int enable_sgm, float
   p.dctx = dcontext;
   p.same_label = (flags & MPL_F_DCONTEXT_SAME_LABEL) ? 1 : 0;
   fill_dirs(s, 0, s->n_dir, p.dirs, p.block_prefix, &p.n_dirs);
+  p.pack = decide_pack(s, p, opts);
   for (int it = n_iter - 1; it >= 0; --it) {
     const bool first = (it == n_iter - 1);
     p.gu_in = first ? dcost_final : gu_buf;  // gu_k = dcost_final for every k at the start
@@ -1020,7 +1049,7 @@ int mpl_isgmr_backward(const mpl_shape* s, unsigned flags, int enable_sgm, float
     p.gu_pair_share = first ? 0 : pair_share;
     p.idx_min = msg_min_index + (int64_t)it * s->n_dir * N;
     p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
-    launch_bwd(p, true, opts, st);
+    launch_bwd(p, true, st);
     Timed timed(MPL_KERNEL_COMBINE, st);
     const bool v4 = (N % 4 == 0) && aligned16(dmsg_update) && aligned16(gu_buf) &&
                     aligned16(dcost_final) && aligned16(dunary);
@@ -1060,7 +1089,9 @@ int mpl_trwp_soft_forward(const mpl_shape* s, unsigned flags, float rho, int n_i
   p.belief_out = unary_update;
   p.msg_in = msg;
   p.msg_out = msg;
+  const int rebuild = belief_rebuild_interval(s->n_dir, n_iter);
   for (int it = 0; it < n_iter; ++it) {
+    if (rebuild > 0 && it > 0 && it % rebuild == 0) rebuild_belief(s, unary, msg, unary_update, st);
     for (int d = 0; d < s->n_dir; ++d) {  // TRWP_forward_soft.cu:441-520
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
       if (train) {
@@ -1069,7 +1100,7 @@ int mpl_trwp_soft_forward(const mpl_shape* s, unsigned flags, float rho, int n_i
       }
       // few chains of at most 32 labels: the wavefront of a chain sweeps d and then d + 1
       p.fused_pair = (opts.fused_pairs && s->n_disp <= 32 &&
-                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+                      p.block_prefix[p.n_dirs] <= launch_policy().fused_pair_max_waves) ? 1 : 0;
       Timed timed(MPL_KERNEL_FWD_SWEEP, st, p.fused_pair ? 2 : 1);
       launch_soft_fwd(p, train, st);
       if (p.fused_pair) ++d;
@@ -1128,7 +1159,7 @@ int mpl_trwp_soft_backward(const mpl_shape* s, unsigned flags, float rho, int n_
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
       // few chains of at most 32 labels: the wavefront of a chain walks d (odd) and then d - 1
       p.fused_pair = (opts.fused_pairs && s->n_disp <= 32 &&
-                      p.block_prefix[p.n_dirs] <= kFusedPairMaxChains) ? 1 : 0;
+                      p.block_prefix[p.n_dirs] <= launch_policy().fused_pair_max_waves) ? 1 : 0;
       Timed timed(MPL_KERNEL_BWD_SWEEP, st, p.fused_pair ? 2 : 1);
       launch_soft_bwd(p, st);
       first = false;

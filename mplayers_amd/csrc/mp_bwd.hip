@@ -30,8 +30,7 @@ namespace {
 // One label per lane otherwise (DIRECT): the step is bound by its own latency, and one atomic for
 // the scatter, one exchange and one atomic for the histogram are the shortest way through it.
 constexpr int kNear = 3;
-// launches of at most this many chains (two wavefronts per SIMD) are taken to be latency-bound
-constexpr int kDirectMaxChains = 2048;
+// (launches of at most LaunchPolicy::direct_max_chains chains are taken to be latency-bound)
 
 template <int R>
 struct PixB {
@@ -262,12 +261,16 @@ __global__ void __launch_bounds__(kWave) sweep_bwd_kernel(const BackParams p) {
           // The table entry is there before the atomics are issued, so the sum of dedge below runs
           // while they are under way.  The LDS executes the instructions of a wavefront in their
           // order: the exchange finds the sums complete without a wait in between, and the
-          // histogram's atomic, which nothing waits for, queues up behind it.
+          // histogram's atomic, which nothing waits for, queues up behind it.  The three are
+          // relaxed atomics to different addresses per lane, which the compiler may reorder: the
+          // fences at wavefront scope forbid that and emit no instruction.
           __builtin_amdgcn_wave_barrier();
           if (valid[0]) {
             atomicAdd(&sc_s[fd], g);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             __builtin_amdgcn_wave_barrier();
             scn[0] = atomicExch(&sc_s[lane], 0.f);  // read and clear
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
             __builtin_amdgcn_wave_barrier();
             if (DC && (same || cd != fd)) atomicAdd(&hist_s[ci], w * g);
           }
@@ -496,7 +499,7 @@ void launch_vmg(const BackParams& p, bool jacobi, hipStream_t st) {
     // shortcuts), 2-D tables (their argmin labels are spread over all labels), and 33 to 64 labels
     // while the launch is latency-bound (40 labels, 1200 chains per launch 3.4 against 4.7 ms, but
     // 64 labels, 3200 chains 9.0 against 7.5).
-    if (p.L <= kPackedMaxL || p.ctx2d || blocks <= kDirectMaxChains) {
+    if (p.L <= kPackedMaxL || p.ctx2d || blocks <= launch_policy().direct_max_chains) {
       if (jacobi)
         sweep_bwd_kernel<R, VEC, MASK, true, true, GRAD><<<blocks, kWave, lds, st>>>(p);
       else

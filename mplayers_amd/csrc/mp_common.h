@@ -467,7 +467,8 @@ struct SweepParams {
   const CtxDesc* desc;             // may be null: dense path
   uint8_t* idx_min;                // (n_dir_total, N) of this iteration, or null
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
-  int pack;                        // packed scans (mp_pack.hip): chains per wavefront
+  int pack;                        // packed scans (mp_pack.hip): chains per wavefront; 0: one chain per
+                                   // wavefront.  Decided once per launch by the host (mp_api.hip)
   int pair_q;                      // Gauss-Seidel: belief plane holds Q between the sweeps of a pair
   int skip_s_store;                // Gauss-Seidel: last sweep of the call, nobody reads S after it
   int fused_pair;                  // Gauss-Seidel: every wavefront sweeps dirs[0], then dirs[0] ^ 1
@@ -528,29 +529,44 @@ void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t
 template <int R>
 void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 
-// a_s (kMaxL floats) + the context: (L,L) for 2-D tables and for the one-label-per-lane dense path
+// Launch policy of the current device.  The scans put one wavefront on a chain, so which kernel a
+// launch takes depends on how many wavefronts' worth of chains it has per SIMD (four SIMDs per
+// compute unit): the thresholds are multiples of the device's SIMD count, read from its properties
+// once per device.  The multiples were measured on an MI355X (256 compute units, 1024 SIMDs).
+struct LaunchPolicy {
+  int n_simd;
+  // Gauss-Seidel launches of at most this many wavefronts (one per SIMD) run both sweeps of a pair
+  // of opposite directions in one launch
+  int fused_pair_max_waves;
+  // A launch is packed (mp_pack.hip: several chains per wavefront, at most kPackedMaxL labels) by
+  // default when
+  //  * its table is 2-D (a learned table, dense) and it has more chains than SIMDs; with 21 labels,
+  //    whose one-chain-per-wavefront scans have a short step of their own, more chains than two
+  //    wavefronts per SIMD,
+  //  * its table is 1-D and it has at most 8 labels and more than 6 chains per SIMD, or at most 16
+  //    labels and more than 9.  The packed step is the dense one, L candidates per label, whatever
+  //    the table; nearly every 1-D table is a band (Potts, truncated linear or quadratic), whose step
+  //    in the one-chain scans takes a few taps, and only the device knows which it is: these are the
+  //    sizes from which packing pays for a band, too.  A caller with dense 1-D tables of up to 32
+  //    labels and thousands of chains per launch passes MPL_F_PACKED_ALWAYS.
+  int packed_min_chains;       // 2-D table
+  int packed_min_chains21;     // 2-D table, 21 labels
+  int packed_min_chains_1d8;   // 1-D table, at most 8 labels
+  int packed_min_chains_1d16;  // 1-D table, 9 to 16 labels
+  // reverse scans with one label per lane: launches of at most this many chains (two wavefronts per
+  // SIMD) are taken to be bound by the latency of a step (mp_bwd.hip)
+  int direct_max_chains;
+};
+const LaunchPolicy& launch_policy();  // mp_api.hip
+
 // packed scans for small label counts (mp_pack.hip): several chains per wavefront.
-// The launchers return false, without launching, when the problem does not qualify.
 constexpr int kPackedMaxL = 32;
-// A launch is packed by default when
-//  * its table is 2-D (a learned table, dense) and it has more chains than the 256 CUs have SIMDs;
-//    with 21 labels, whose one-chain-per-wavefront scans have a short step of their own, more
-//    chains than two wavefronts per SIMD,
-//  * its table is 1-D and it has at most 8 labels and more than 6144 chains, or at most 16 labels
-//    and more than 10000 chains.  The packed step is the dense one, L candidates per label, whatever
-//    the table; nearly every 1-D table is a band (Potts, truncated linear or quadratic), whose step
-//    in the one-chain scans takes a few taps, and only the device knows which it is: these are the
-//    sizes from which packing pays for a band, too.  A caller with dense 1-D tables of up to 32
-//    labels and thousands of chains per launch passes MPL_F_PACKED_ALWAYS.
-constexpr int kPackedMinChains = 1025;
-constexpr int kPackedMinChains21 = 2049;
-constexpr int kPackedMinChains1d8 = 6145;    // at most 8 labels
-constexpr int kPackedMinChains1d16 = 10001;  // 9 to 16 labels
+// chains per wavefront the packed scans would use for such a launch (below 2: they do not apply);
 // always: pack whatever the table and the number of chains (tests, comparisons, such callers)
-// chains per wavefront the packed scans would use for such a launch (below 2: they do not apply)
 int packed_chains_per_wave(int B, int H, int W, int L, bool ctx2d, int64_t chains, bool always);
-bool launch_packed_fwd(const SweepParams& p, bool train, bool jacobi, bool always, hipStream_t st);
-bool launch_packed_bwd(const BackParams& p, bool jacobi, bool always, hipStream_t st);
+// G: what packed_chains_per_wave returned for the launch (>= 2)
+void launch_packed_fwd(const SweepParams& p, bool train, bool jacobi, int G, hipStream_t st);
+void launch_packed_bwd(const BackParams& p, bool jacobi, int G, hipStream_t st);
 
 // soft-weighted TRWP (mp_soft.hip): one direction per launch, L <= 64
 void launch_soft_fwd(const SweepParams& p, bool train, hipStream_t st);

@@ -573,13 +573,6 @@ __global__ void __launch_bounds__(kWave) packed_bwd_kernel(const BackParams p) {
 
 // prefix sums of wavefronts per direction for G chains per wavefront
 template <typename Params>
-int64_t chains_in_launch(const Params& p) {
-  int64_t c = 0;
-  for (int i = 0; i < p.n_dirs; ++i) c += (int64_t)p.B * make_dir(p.dirs[i], p.H, p.W).n_chains;
-  return c;
-}
-
-template <typename Params>
 Params with_wave_prefix(const Params& p, int G) {
   Params q = p;
   q.pack = G;
@@ -616,20 +609,18 @@ int packed_chains_per_wave(int B, int H, int W, int L, bool ctx2d, int64_t chain
   //    chains) 1.40 against 2.02; 16 labels, batch 2 (8392 chains) 1.81 against 1.42, batch 4 2.11
   //    against 2.56.
   if (!always) {
+    const LaunchPolicy& pol = launch_policy();
     if (ctx2d) {
-      if (chains < (L == 21 ? kPackedMinChains21 : kPackedMinChains)) return 0;
+      if (chains < (L == 21 ? pol.packed_min_chains21 : pol.packed_min_chains)) return 0;
     } else {
-      if (L > 16 || chains < (L <= 8 ? kPackedMinChains1d8 : kPackedMinChains1d16)) return 0;
+      if (L > 16 || chains < (L <= 8 ? pol.packed_min_chains_1d8 : pol.packed_min_chains_1d16)) return 0;
     }
   }
   int G = kWave / L;
   return G > 16 ? 16 : G;
 }
 
-bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, bool always, hipStream_t st) {
-  if (p0.u_fused) return false;  // (set for more than 32 labels only)
-  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, p0.ctx2d != 0, chains_in_launch(p0), always);
-  if (G < 2) return false;
+void launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, int G, hipStream_t st) {
   const SweepParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = sizeof(float) * (3 * kRedFloats + p.L * p.L);
@@ -652,12 +643,9 @@ bool launch_packed_fwd(const SweepParams& p0, bool train, bool jacobi, bool alwa
   else
     MPL_PACKED_FWD(0);
 #undef MPL_PACKED_FWD
-  return true;
 }
 
-bool launch_packed_bwd(const BackParams& p0, bool jacobi, bool always, hipStream_t st) {
-  const int G = packed_chains_per_wave(p0.B, p0.H, p0.W, p0.L, p0.ctx2d != 0, chains_in_launch(p0), always);
-  if (G < 2) return false;
+void launch_packed_bwd(const BackParams& p0, bool jacobi, int G, hipStream_t st) {
   const BackParams p = with_wave_prefix(p0, G);
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = sizeof(float) * (4 * kRedFloats + p.L * p.L * (1 + G));
@@ -682,7 +670,6 @@ bool launch_packed_bwd(const BackParams& p0, bool jacobi, bool always, hipStream
     default: MPL_PACKED_BWD(3); break;
   }
 #undef MPL_PACKED_BWD
-  return true;
 }
 
 }  // namespace mpl

@@ -6,13 +6,29 @@
 // the arithmetic (n_in planes read and summed, n_out planes written, register prefetch ring), and a
 // one-pass streaming kernel moves them the way an element-wise kernel does, so the scans can be
 // rated against what the hardware delivers for their access pattern rather than against the data
-// sheet alone.  Diagnostics only; no counterpart in the reference.
+// sheet alone.  Diagnostics only; no counterpart in the reference.  Built into a library of its own
+// (libmplayers_probe.so, mp_probe.h) that only the benchmark and the tests load.
+
+#include <stdarg.h>
+#include <stdio.h>
 
 #include "mp_common.h"
+#include "mp_probe.h"
 
 using namespace mpl;
 
 namespace {
+
+constexpr int kEinval = -1, kElaunch = -2;
+thread_local char g_probe_err[256] = "";
+int pfail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int pfail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_probe_err, sizeof(g_probe_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
@@ -77,10 +93,10 @@ void launch_probe(int shape, const float* in, float* out, int H, int W, int L, h
   const int64_t plane = (int64_t)H * W * units;
   const v4f* src = reinterpret_cast<const v4f*>(in);
   v4f* dst = reinterpret_cast<v4f*>(out);
-  if (shape == MPL_PROBE_ROWS) {
+  if (shape == MPLP_ROWS) {
     chain_copy_kernel<NIN, NOUT><<<H, kWave, 0, st>>>(src, dst, plane, units, (int64_t)W * units,
                                                       units, W);
-  } else if (shape == MPL_PROBE_COLUMNS) {
+  } else if (shape == MPLP_COLUMNS) {
     chain_copy_kernel<NIN, NOUT><<<W, kWave, 0, st>>>(src, dst, plane, units, units,
                                                       (int64_t)W * units, H);
   } else {
@@ -128,12 +144,19 @@ const IssuePattern kIssuePatterns[] = {
 };
 constexpr int kNumIssuePatterns = (int)(sizeof(kIssuePatterns) / sizeof(kIssuePatterns[0]));
 
+// %0: byte address of this lane's LDS word, %1: that of word 0.  They are operands of every
+// statement, so whatever the compiler does with its registers between two statements, an LDS
+// access of a pattern never sees an address it did not get from the compiler.  v10..v17 and the
+// scalar registers only feed arithmetic whose result is not read: what they hold does not matter.
 #define MPL_ISSUE_TIMED(idx, body)                                                                \
   {                                                                                               \
     __builtin_amdgcn_s_barrier();                                                                 \
     const long long t0 = clock64();                                                               \
-    asm volatile(body ::: "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "v18", "v19",  \
-                 "s44", "s45", "s46", "s47", "vcc", "memory");                                    \
+    asm volatile(body                                                                             \
+                 :                                                                                \
+                 : "v"(own), "v"(first)                                                           \
+                 : "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "s40", "s41", "s42",  \
+                   "s43", "s44", "s45", "s46", "s47", "vcc", "memory");                           \
     const long long t1 = clock64();                                                               \
     if (threadIdx.x == 0) out[idx] = t1 - t0;                                                     \
   }
@@ -142,19 +165,15 @@ __global__ void __launch_bounds__(kWave) issue_probe_kernel(long long* __restric
   __shared__ float lds[256];
   for (int i = threadIdx.x; i < 256; i += kWave) lds[i] = 0.f;
   __syncthreads();
-  // v18: byte address of this lane's LDS word, v19: that of word 0 (no pattern writes them: an LDS
-  // access at a clobbered, unaligned address would fault); v10..v17: operands and results;
-  // s40..s43: masks and a scalar operand (whatever they hold: only the timing is read)
   const unsigned own = (unsigned)(size_t)&lds[threadIdx.x], first = (unsigned)(size_t)&lds[0];
+  // ordinary values in the registers the patterns compute on (nothing depends on their surviving)
   asm volatile(
-      "v_mov_b32 v18, %0\n v_mov_b32 v19, %1\n v_mov_b32 v10, 1.0\n v_mov_b32 v11, 1.0\n"
-      " v_mov_b32 v12, 1.0\n v_mov_b32 v13, 1.0\n v_mov_b32 v14, 1.0\n v_mov_b32 v15, 1.0\n"
-      " v_mov_b32 v16, 1.0\n v_mov_b32 v17, 1.0\n s_mov_b32 s40, 1\n s_mov_b32 s41, 1\n"
-      " s_mov_b32 s42, 1\n s_mov_b32 s43, 1"
+      "v_mov_b32 v10, 1.0\n v_mov_b32 v11, 1.0\n v_mov_b32 v12, 1.0\n v_mov_b32 v13, 1.0\n"
+      " v_mov_b32 v14, 1.0\n v_mov_b32 v15, 1.0\n v_mov_b32 v16, 1.0\n v_mov_b32 v17, 1.0\n"
+      " s_mov_b32 s40, 1\n s_mov_b32 s41, 1\n s_mov_b32 s42, 1\n s_mov_b32 s43, 1"
       :
-      : "v"(own), "v"(first)
-      : "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "v18", "v19", "s40", "s41", "s42",
-        "s43", "memory");
+      :
+      : "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "s40", "s41", "s42", "s43");
   for (int rep = 0; rep < 2; ++rep) {  // (the second pass runs from a warm instruction cache)
   MPL_ISSUE_TIMED(0, "")
   MPL_ISSUE_TIMED(1, ".rept 120\n v_add_f32 v10, v10, v14\n v_add_f32 v11, v11, v14\n v_add_f32 v12, v12, v14\n v_add_f32 v13, v13, v14\n .endr")
@@ -176,27 +195,73 @@ __global__ void __launch_bounds__(kWave) issue_probe_kernel(long long* __restric
   MPL_ISSUE_TIMED(17, ".rept 160\n v_min_f32_dpp v10, v10, v10 row_shr:1 row_mask:0xf bank_mask:0xf\n v_add_f32 v11, v11, v14\n v_add_f32 v12, v12, v14\n .endr")
   MPL_ISSUE_TIMED(18, ".rept 480\n v_exp_f32 v10, v15\n .endr")
   MPL_ISSUE_TIMED(19, ".rept 480\n v_rcp_f32 v10, v15\n .endr")
-  MPL_ISSUE_TIMED(20, ".rept 53\n ds_bpermute_b32 v10, v18, v15\n ds_bpermute_b32 v11, v18, v15\n ds_bpermute_b32 v12, v18, v15\n ds_bpermute_b32 v13, v18, v15\n ds_bpermute_b32 v10, v18, v15\n ds_bpermute_b32 v11, v18, v15\n ds_bpermute_b32 v12, v18, v15\n ds_bpermute_b32 v13, v18, v15\n s_waitcnt lgkmcnt(0)\n .endr")
-  MPL_ISSUE_TIMED(21, ".rept 240\n ds_bpermute_b32 v10, v18, v15\n s_waitcnt lgkmcnt(0)\n .endr")
-  MPL_ISSUE_TIMED(22, ".rept 240\n ds_read_b32 v10, v18\n s_waitcnt lgkmcnt(0)\n .endr")
-  MPL_ISSUE_TIMED(23, ".rept 160\n ds_add_f32 v18, v15\n ds_wrxchg_rtn_b32 v10, v18, v19\n s_waitcnt lgkmcnt(0)\n .endr")
-  MPL_ISSUE_TIMED(24, ".rept 240\n ds_add_f32 v19, v15\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(20, ".rept 53\n ds_bpermute_b32 v10, %0, v15\n ds_bpermute_b32 v11, %0, v15\n ds_bpermute_b32 v12, %0, v15\n ds_bpermute_b32 v13, %0, v15\n ds_bpermute_b32 v10, %0, v15\n ds_bpermute_b32 v11, %0, v15\n ds_bpermute_b32 v12, %0, v15\n ds_bpermute_b32 v13, %0, v15\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(21, ".rept 240\n ds_bpermute_b32 v10, %0, v15\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(22, ".rept 240\n ds_read_b32 v10, %0\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(23, ".rept 160\n ds_add_f32 %0, v15\n ds_wrxchg_rtn_b32 v10, %0, %1\n s_waitcnt lgkmcnt(0)\n .endr")
+  MPL_ISSUE_TIMED(24, ".rept 240\n ds_add_f32 %1, v15\n s_waitcnt lgkmcnt(0)\n .endr")
   }
 }
 #undef MPL_ISSUE_TIMED
+
+// ------------------------------------------------------------------------------------------------
+// wave-primitive self test
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(kWave) selftest_kernel(int* out) {
+  const int lane = threadIdx.x;
+  int ok = 1;
+  float x = (float)(lane * 3 % 17) + 100.f;
+  float up = wave_shl1(x, -1.f);
+  float dn = wave_shr1(x, -2.f);
+  float eu = lane < 63 ? (float)((lane + 1) * 3 % 17) + 100.f : -1.f;
+  float ed = lane > 0 ? (float)((lane - 1) * 3 % 17) + 100.f : -2.f;
+  if (up != eu || dn != ed) ok = 0;
+  float y = (float)((lane * 37 + 11) % 64);  // a permutation of 0..63
+  if (wave_min(y) != 0.f) ok = 0;
+  for (int special = 0; special < 64; special += 9)  // the minimum sits in every row and bank
+    if (wave_min(y + (lane == special ? -100.f : 0.f)) != (float)((special * 37 + 11) % 64) - 100.f)
+      ok = 0;
+  if (wave_min_fast(y) != 0.f) ok = 0;
+  for (int special = 0; special < 64; special += 7)
+    if (wave_min_fast(y + (lane == special ? -100.f : 0.f)) != (float)((special * 37 + 11) % 64) - 100.f)
+      ok = 0;
+  if (wave_min_fast(lane < 21 ? (float)(30 - lane) : INFINITY) != 10.f) ok = 0;
+  if (wave_sum((float)lane) != 2016.f) ok = 0;
+  bool pr[2] = {lane == 5 || lane == 40, lane == 40};
+  if (last_label<2>(pr, -1) != 81) ok = 0;
+  bool pn[2] = {false, false};
+  if (last_label<2>(pn, -7) != -7) ok = 0;
+  uint64_t b = ballot(ok != 0);
+  if (lane == 0) {
+    out[0] = (b == ~0ull) ? 1 : 0;
+    out[1] = (int)(b & 0xffffffffu);
+    out[2] = (int)(b >> 32);
+  }
+}
 
 }  // namespace
 
 extern "C" {
 
-int mpl_probe_copy(int shape, int n_in, int n_out, const float* in, float* out, int height,
+const char* mplp_last_error(void) { return g_probe_err; }
+
+int mplp_selftest_wave_ops(int* out, void* stream) {
+  if (out == nullptr) return pfail(kEinval, "selftest: null pointer");
+  selftest_kernel<<<1, kWave, 0, (hipStream_t)stream>>>(out);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return pfail(kElaunch, "selftest: %s", hipGetErrorString(e));
+  return 0;
+}
+
+
+int mplp_copy(int shape, int n_in, int n_out, const float* in, float* out, int height,
                    int width, int n_labels, void* stream) {
-  if (in == nullptr || out == nullptr) return fail(MPL_EINVAL, "probe_copy: null pointer");
-  if (shape < 0 || shape > MPL_PROBE_STREAM) return fail(MPL_EINVAL, "probe_copy: unknown shape");
+  if (in == nullptr || out == nullptr) return pfail(kEinval, "probe_copy: null pointer");
+  if (shape < 0 || shape > MPLP_STREAM) return pfail(kEinval, "probe_copy: unknown shape");
   if (height < 1 || width < 1 || n_labels < 4 || n_labels > 256 || (n_labels & 3))
-    return fail(MPL_EINVAL, "probe_copy: n_labels must be a multiple of 4 in [4, 256]");
+    return pfail(kEinval, "probe_copy: n_labels must be a multiple of 4 in [4, 256]");
   if ((int64_t)height * width * n_labels / 4 / 256 > 0x7fffffff)
-    return fail(MPL_EINVAL, "probe_copy: plane too large");
+    return pfail(kEinval, "probe_copy: plane too large");
   hipStream_t st = (hipStream_t)stream;
   const int key = n_in * 10 + n_out;
   switch (key) {
@@ -206,30 +271,30 @@ int mpl_probe_copy(int shape, int n_in, int n_out, const float* in, float* out, 
     case 32: launch_probe<3, 2>(shape, in, out, height, width, n_labels, st); break;
     case 43: launch_probe<4, 3>(shape, in, out, height, width, n_labels, st); break;
     default:
-      return fail(MPL_EINVAL, "probe_copy: (n_in, n_out) must be one of (1,1) (1,3) (3,0) (3,2) (4,3)");
+      return pfail(kEinval, "probe_copy: (n_in, n_out) must be one of (1,1) (1,3) (3,0) (3,2) (4,3)");
   }
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(MPL_ELAUNCH, "probe_copy: %s", hipGetErrorString(e));
-  return MPL_OK;
+  if (e != hipSuccess) return pfail(kElaunch, "probe_copy: %s", hipGetErrorString(e));
+  return 0;
 }
 
-int mpl_probe_issue_count(void) { return kNumIssuePatterns; }
+int mplp_issue_count(void) { return kNumIssuePatterns; }
 
-const char* mpl_probe_issue_name(int pattern) {
+const char* mplp_issue_name(int pattern) {
   return pattern >= 0 && pattern < kNumIssuePatterns ? kIssuePatterns[pattern].name : "";
 }
 
-int mpl_probe_issue_slots(int pattern) {
+int mplp_issue_slots(int pattern) {
   return pattern >= 0 && pattern < kNumIssuePatterns ? kIssuePatterns[pattern].slots : -1;
 }
 
-int mpl_probe_issue(long long* clocks, int n, void* stream) {
-  if (clocks == nullptr) return fail(MPL_EINVAL, "probe_issue: null pointer");
-  if (n < kNumIssuePatterns) return fail(MPL_EINVAL, "probe_issue: room for %d results needed", kNumIssuePatterns);
+int mplp_issue(long long* clocks, int n, void* stream) {
+  if (clocks == nullptr) return pfail(kEinval, "probe_issue: null pointer");
+  if (n < kNumIssuePatterns) return pfail(kEinval, "probe_issue: room for %d results needed", kNumIssuePatterns);
   issue_probe_kernel<<<1, kWave, 0, (hipStream_t)stream>>>(clocks);
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(MPL_ELAUNCH, "probe_issue: %s", hipGetErrorString(e));
-  return MPL_OK;
+  if (e != hipSuccess) return pfail(kElaunch, "probe_issue: %s", hipGetErrorString(e));
+  return 0;
 }
 
 }  // extern "C"

@@ -204,8 +204,35 @@ def test_product_never_touches_the_oracle_or_scratch_files():
   assert not re.search(r"(^|[\"'/\s])_work/", bench)
 
 
+def test_probe_library_is_separate_and_validates():
+  """The measurement probes live in a library of their own (csrc/mp_probe.h): the product
+  library exports none of them, and they answer bad arguments on the host."""
+  import ctypes
+  from mplayers_amd import _lib, _probe
+  product = _lib.load()
+  for name in ("mpl_probe_copy", "mpl_probe_issue", "mpl_selftest_wave_ops", "mplp_copy",
+               "mplp_issue", "mplp_selftest_wave_ops"):
+    assert not hasattr(product, name), name
+  lib = _probe.load()
+  text = open(os.path.join(ROOT, "mplayers_amd", "csrc", "mp_probe.h")).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  for name in sorted(set(re.findall(r"\b(mplp_[a-z0-9_]+)\s*\(", text))):
+    assert hasattr(lib, name), name
+  null = ctypes.c_void_p(None)
+  one = ctypes.c_void_p(16)   # never dereferenced: every call below fails validation first
+  assert lib.mplp_copy(0, 2, 2, one, one, 4, 4, 8, null) != 0
+  assert lib.mplp_copy(0, 1, 1, one, one, 4, 4, 6, null) != 0
+  assert lib.mplp_issue(null, 64, null) != 0
+  assert lib.mplp_issue(one, 1, null) != 0
+  assert lib.mplp_issue_count() > 1 and lib.mplp_issue_slots(0) == 0
+  assert lib.mplp_issue_slots(lib.mplp_issue_count()) == -1
+  assert lib.mplp_issue_name(1) != b"" and lib.mplp_issue_name(-1) == b""
+  assert lib.mplp_selftest_wave_ops(null, null) != 0
+  assert b"" != lib.mplp_last_error()
+
+
 def test_new_entry_points_validate_before_launching():
-  """Terms, probe and transpose entry points answer bad arguments with MPL_EINVAL on the host."""
+  """Terms and transpose entry points answer bad arguments with MPL_EINVAL on the host."""
   import ctypes
   from mplayers_amd import _lib
   lib = _lib.load()
@@ -220,13 +247,6 @@ def test_new_entry_points_validate_before_launching():
   shape = _lib.Shape(4, 1, 4, 4, 8, 0)
   assert lib.mpl_mrf_energy(ctypes.byref(shape), 1, one, one, null, null, one, null) != 0
   assert lib.mpl_mrf_energy(ctypes.byref(shape), 0, one, one, null, one, one, null) == 0  # nothing to do
-  assert lib.mpl_probe_copy(0, 2, 2, one, one, 4, 4, 8, null) != 0
-  assert lib.mpl_probe_copy(0, 1, 1, one, one, 4, 4, 6, null) != 0
-  assert lib.mpl_probe_issue(null, 64, null) != 0
-  assert lib.mpl_probe_issue(one, 1, null) != 0
-  assert lib.mpl_probe_issue_count() > 1 and lib.mpl_probe_issue_slots(0) == 0
-  assert lib.mpl_probe_issue_slots(lib.mpl_probe_issue_count()) == -1
-  assert lib.mpl_probe_issue_name(1) != b"" and lib.mpl_probe_issue_name(-1) == b""
   assert lib.mpl_transpose(null, one, 1, 4, 4, null) != 0
   assert lib.mpl_transpose(one, one, 1, -1, 4, null) != 0
   assert lib.mpl_transpose(one, one, 0, 4, 4, null) == 0                                  # empty
