@@ -1,7 +1,8 @@
 /*
  * C ABI of libmplayers_hip.so: min-sum message passing (TRWP, ISGMR) on grid MRFs for gfx950.
  *
- * Every pointer is a DEVICE pointer unless said otherwise; all tensors are contiguous with the
+ * Every pointer is a DEVICE pointer unless said otherwise (the mpl_*_forward_cpu calls take host
+ * pointers); all tensors are contiguous with the
  * label axis innermost.  The caller owns and allocates every buffer, exactly as the reference's
  * operators require (pytorch/MP_module.py:26-50, 65-78); buffers marked "zero-filled" must come
  * in zeroed, as the reference's caller provides them.  `stream` is a hipStream_t (NULL = the
@@ -112,6 +113,25 @@ int mpl_isgmr_backward(const mpl_shape* shape, unsigned flags, int enable_sgm, f
                        const uint8_t* msg_norm_index, float* dunary, float* dcontext,
                        float* dedge_weights, float* dmsg, float* dunary_update,
                        float* dmsg_update, void* stream);
+
+/* The CPU branch of lib_*.TRWP.forward and lib_*.ISGMR.forward: what the reference's operators run
+ * when their tensors are not on the GPU (ForwardCPU, MPLayers/TRWP/TRWP.cpp:172-243 reached from
+ * :275-282, MPLayers/ISGMR/ISGMR.cpp:190-298 reached from :330-339).  HOST pointers; the calls run
+ * on the calling thread and on up to MPL_OPT_CPU_THREADS worker threads and return when done.
+ * That path has its own semantics, reproduced bit for bit: forward only, every edge weight 1, no
+ * argmin indices; the pairwise table of direction d is read at context + d * n_disp * n_disp, so
+ * `context` holds (n_dir - 1) * n_disp^2 floats plus one table (n_disp^2 with ctx2d, else n_disp);
+ * value = rho * (unary + sum_k m_k) - m_inv + ctx in that order; labels are 0 for 256 labels
+ * (the reference's unsigned char loop counter, common.cpp:152).  label_all may be NULL.
+ * mpl_isgmr_forward_cpu with enable_sgm REPLACES `unary` by the sum of the new messages after every
+ * iteration and clears `msg` (ISGMR.cpp:255-261): unary is an in/out tensor there.  msg_update is
+ * the second message buffer (zero-filled by the caller, as `msg`).  There is no CPU backward
+ * (TRWP.cpp:315-316). */
+int mpl_trwp_forward_cpu(const mpl_shape* shape, float rho, int n_iter, const float* unary,
+                         const float* context, float* msg, float* cost_final, uint8_t* label_all);
+int mpl_isgmr_forward_cpu(const mpl_shape* shape, int enable_sgm, float rho, int n_iter,
+                          float* unary, const float* context, float* msg, float* cost_final,
+                          float* msg_update, uint8_t* label_all);
 
 /* Soft-weighted TRWP: replaces lib_*.TRWP_hard_soft.forward_soft, MPLayers/TRWP_hard_soft/TRWP.cpp:
  * 313-349 (ForwardSoft) -> TRWP_forward_soft.cu:378-559.  The min over front labels becomes the
@@ -282,6 +302,9 @@ const char* mpl_last_error(void);
  * every max(1, 32 / n_dir) iterations). */
 #define MPL_OPT_BELIEF_REBUILD 2
 #define MPL_BELIEF_REBUILD_DEFAULT (-1)
+/* MPL_OPT_CPU_THREADS (default 0: 16, the reference's NUM_THREADS, tools/cpp/utils.h:17): threads
+ * the mpl_*_forward_cpu calls spread their chains over. */
+#define MPL_OPT_CPU_THREADS 3
 int mpl_set_option(int option, int value);
 
 /* Library version: major * 100 + minor. */

@@ -36,6 +36,12 @@ def _units():
   return units
 
 
+# host-only sources (the CPU forward path), compiled with the host compiler; no fused multiply-adds,
+# so that the arithmetic is the reference's own (g++ -O2 on x86-64 contracts nothing)
+HOST_UNITS = [("mp_cpu", os.path.join("cpu", "mp_cpu.cpp"))]
+HOST_FLAGS = ["-O3", "-ffp-contract=off", "-std=c++17", "-fPIC", "-pthread", "-Wall", "-Wextra"]
+
+
 def _run(cmd):
   proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
   out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
@@ -56,6 +62,10 @@ def build(verbose=False, extra_flags=(), lib_path=LIB, jobs=None):
     objs.append(obj)
     cmds.append([hipcc] + HIPCC_FLAGS + list(extra_flags) + defs +
                 ["-c", os.path.join(CSRC, src), "-o", obj])
+  cxx = os.environ.get("CXX", "g++")
+  for name, src in HOST_UNITS:
+    cmds.append([cxx] + HOST_FLAGS + ["-c", os.path.join(CSRC, src), "-o",
+                                      os.path.join(obj_dir, name + ".o")])
   with ThreadPoolExecutor(max_workers=jobs) as pool:
     for cmd, out in zip(cmds, pool.map(_run, cmds)):
       if verbose:
@@ -72,7 +82,8 @@ def link(lib_path=LIB, verbose=False):
   obj_dir = OBJ if lib_path == LIB else lib_path + ".build"
   probe_path = PROBE_LIB if lib_path == LIB else lib_path.replace(".so", "_probe.so")
   names = [name for name, _, _ in _units()]
-  groups = ((lib_path, [n for n in names if n not in PROBE_UNITS], ["-lpthread"]),
+  host = [name for name, _ in HOST_UNITS]
+  groups = ((lib_path, [n for n in names if n not in PROBE_UNITS] + host, ["-lpthread"]),
             (probe_path, [n for n in names if n in PROBE_UNITS], []))
   for path, members, libs in groups:
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + \

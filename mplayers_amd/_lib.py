@@ -6,6 +6,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hip.so"))
 
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
+           "mpl_trwp_forward_cpu", "mpl_isgmr_forward_cpu",
            "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
            "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_edge_shift_static",
            "mpl_trwp_soft_forward",
@@ -55,6 +56,8 @@ def load():
   lib.mpl_trwp_backward.argtypes = [sp, cu, cf, ci] + [vp] * 11
   lib.mpl_isgmr_forward.argtypes = [sp, cu, ci, cf, ci, ci] + [vp] * 11
   lib.mpl_isgmr_backward.argtypes = [sp, cu, ci, cf, ci] + [vp] * 12
+  lib.mpl_trwp_forward_cpu.argtypes = [sp, cf, ci] + [vp] * 5
+  lib.mpl_isgmr_forward_cpu.argtypes = [sp, ci, cf, ci] + [vp] * 6
   lib.mpl_trwp_soft_forward.argtypes = [sp, cu, cf, ci] + [vp] * 10
   lib.mpl_trwp_soft_backward.argtypes = [sp, cu, cf, ci] + [vp] * 11
   lib.mpl_soft_weighted_message.argtypes = [ci, ci, vp, vp, vp, vp]
@@ -88,6 +91,7 @@ def load():
 OPT_PACKED_SCANS = 0
 OPT_FUSED_U = 1
 OPT_BELIEF_REBUILD = 2
+OPT_CPU_THREADS = 3
 BELIEF_REBUILD_DEFAULT = -1
 
 

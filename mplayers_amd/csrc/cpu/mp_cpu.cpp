@@ -51,7 +51,9 @@ int n_threads() {
 template <typename Fn>
 void parallel_for(int64_t n, int64_t block, const Fn& fn) {
   const int64_t n_blocks = (n + block - 1) / block;
-  const int workers = (int)std::min<int64_t>(n_threads(), n_blocks);
+  // (no more threads than the host has hardware threads: the results do not depend on the count)
+  const int hw = (int)std::thread::hardware_concurrency();
+  const int workers = (int)std::min<int64_t>(std::min(n_threads(), hw > 0 ? hw : 1), n_blocks);
   std::atomic<int64_t> next{0};
   auto body = [&]() {
     for (;;) {
@@ -123,7 +125,11 @@ void sweep(const Grid& g, int dir, float rho, const float* unary, const float* m
     const int64_t bv = job / n_chains;
     const int start = starts[(size_t)(job - bv * n_chains)];
     int h = start / g.W, w = start - (start / g.W) * g.W;
-    std::vector<float> base((size_t)L), sum((size_t)L), out((size_t)L);
+    thread_local std::vector<float> scratch;
+    if (scratch.size() < 3 * (size_t)L) scratch.resize(3 * (size_t)L);
+    float* base = scratch.data();
+    float* sum = base + L;
+    float* out = sum + L;
     for (;;) {
       const int fh = h, fw = w;
       h += hs;

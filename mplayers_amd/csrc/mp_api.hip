@@ -729,6 +729,7 @@ int mpl_set_option(int option, int value) {
     g_belief_rebuild.store(value, std::memory_order_relaxed);
     return MPL_OK;
   }
+  if (option == MPL_OPT_CPU_THREADS) return set_cpu_threads(value);
   return fail(MPL_EINVAL, "set_option: unknown option %d", option);
 }
 

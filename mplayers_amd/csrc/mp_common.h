@@ -523,6 +523,9 @@ struct BackParams {
 // records the message mpl_last_error() returns on this thread and returns `code`
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 
+// MPL_OPT_CPU_THREADS (cpu/mp_cpu.cpp)
+int set_cpu_threads(int n);
+
 // launchers, one translation unit per R so that the instantiations compile in parallel
 template <int R>
 void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st);

@@ -6,10 +6,15 @@ MPLayers/ISGMR/ISGMR.cpp:300-313, 344-356, 400-401): caller-allocated, zero-fill
 are filled in place; an empty index / label tensor switches that output off.  They hand raw device
 pointers and the current HIP stream to the C ABI of libmplayers_hip.so.
 
+CPU tensors take the CPU forward of the library (mpl_trwp_forward_cpu / mpl_isgmr_forward_cpu), as
+the reference's operators run ForwardCPU for them (TRWP.cpp:275-282, ISGMR.cpp:330-339), with
+that path's own semantics: no edge weights, no indices, the table of direction d at
+context + d * L * L.
+
 Deviations from the reference, all towards failing loudly: more labels than 256 (the reference
-prints a message and returns zero-filled outputs, TRWP.cpp:269-273), CPU tensors (the reference
-runs its CPU loop, or prints "Does not support CPU backward", :315-316) and non-contiguous tensors
-raise RuntimeError.
+prints a message and returns zero-filled outputs, TRWP.cpp:269-273), a backward call on CPU tensors
+(the reference prints "Does not support CPU backward" and returns, :315-316), tensors on different
+devices and non-contiguous tensors raise RuntimeError.
 """
 import torch
 
@@ -20,11 +25,13 @@ def _ptr(t):
   return None if t is None or t.numel() == 0 else t.data_ptr()
 
 
-def _check(name, t, dtype, numel=None):
+def _check(name, t, dtype, numel=None, cuda=True):
   if not isinstance(t, torch.Tensor):
     raise TypeError("%s must be a tensor" % name)
-  if not t.is_cuda:
-    raise RuntimeError("%s is not on the GPU: these operators only run as HIP kernels" % name)
+  if cuda and not t.is_cuda:
+    raise RuntimeError("%s is not on the GPU like the other tensors of the call" % name)
+  if not cuda and t.is_cuda:
+    raise RuntimeError("%s is on the GPU, the other tensors of the call are not" % name)
   if not t.is_contiguous():
     raise RuntimeError("%s must be contiguous" % name)  # CHECK_CONTIGUOUS, cudaUtils.hpp:10
   if t.dtype != dtype:
@@ -87,6 +94,37 @@ class _Op(object):
     return shape, P, N
 
 
+def _no_cpu_backward(t):
+  if isinstance(t, torch.Tensor) and not t.is_cuda:
+    raise RuntimeError("Does not support CPU backward.")  # TRWP.cpp:315-316, ISGMR.cpp:377-378
+
+
+def _forward_cpu(mode, enable_sgm, rho, n_iter, unary, context, msg, cost_final, msg_update,
+                 label_all):
+  """ForwardCPU of the reference (TRWP.cpp:172-243, ISGMR.cpp:190-298) through the library's CPU
+  entry points.  edge_weights, the index tensors and unary_update play no part in that path."""
+  lib = _lib.load()
+  shape, P, L, ctx2d = _Op._shape_from_msg(msg)
+  N = P * L
+  f32 = torch.float32
+  _check("unary", unary, f32, N, cuda=False)
+  # the table of direction d is read at context + d * L * L
+  _check("context", context, f32, (shape.n_dir - 1) * L * L + _context_numel(L, ctx2d), cuda=False)
+  _check("msg", msg, f32, shape.n_dir * N, cuda=False)
+  _check("cost_final", cost_final, f32, N, cuda=False)
+  if label_all.numel() > 0:
+    _check("label_all", label_all, torch.uint8, n_iter * P, cuda=False)
+  if mode == "TRWP":
+    rc = lib.mpl_trwp_forward_cpu(shape, float(rho), int(n_iter), _ptr(unary), _ptr(context),
+                                  _ptr(msg), _ptr(cost_final), _ptr(label_all))
+  else:
+    _check("msg_update", msg_update, f32, shape.n_dir * N, cuda=False)
+    rc = lib.mpl_isgmr_forward_cpu(shape, int(enable_sgm), float(rho), int(n_iter), _ptr(unary),
+                                   _ptr(context), _ptr(msg), _ptr(cost_final), _ptr(msg_update),
+                                   _ptr(label_all))
+  _lib.check(rc, mode + ".forward (CPU)")
+
+
 class TRWP(object):
   """Drop-in for the reference's `lib_stereo.TRWP` / `lib_seg.TRWP` extension modules."""
 
@@ -96,6 +134,8 @@ class TRWP(object):
     """msg_uninit (not in the reference): True declares that `msg` holds no initial messages --
     they start at zero and the library writes every element, so the caller need not clear it.
     flags (not in the reference): further per-call MPL_F_* bits of the C ABI."""
+    if isinstance(unary, torch.Tensor) and not unary.is_cuda:
+      return _forward_cpu("TRWP", 0, rho, n_iter, unary, context, msg, cost_final, None, label_all)
     lib = _lib.load()
     shape, _, _ = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
                                      msg_norm_index, unary_update, label_all, n_iter)
@@ -112,6 +152,7 @@ class TRWP(object):
                dcontext, dedge_weights, dmsg, dunary_update, flags=0):
     """dcontext / dedge_weights: None or an empty tensor when that gradient is not wanted (not in
     the reference, which always computes both); flags: per-call MPL_F_* bits of the C ABI."""
+    _no_cpu_backward(dcost_final)
     lib = _lib.load()
     shape, n_iter, P, L, ctx2d = _Op._shape_from_index(msg_min_index)
     N = P * L
@@ -144,6 +185,9 @@ class ISGMR(object):
               cost_final, msg_min_index, msg_norm_index, unary_update, msg_update, label_all,
               msg_uninit=False, flags=0):
     """msg_uninit, flags (not in the reference): see TRWP.forward."""
+    if isinstance(unary, torch.Tensor) and not unary.is_cuda:
+      return _forward_cpu("ISGMR", enable_sgm, rho, n_iter, unary, context, msg, cost_final,
+                          msg_update, label_all)
     lib = _lib.load()
     shape, _, N = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
                                      msg_norm_index, unary_update, label_all, n_iter)
@@ -162,6 +206,7 @@ class ISGMR(object):
                msg_norm_index, dunary, dcontext, dedge_weights, dmsg, dunary_update, dmsg_update,
                flags=0):
     """dcontext / dedge_weights / flags: see TRWP.backward."""
+    _no_cpu_backward(dcost_final)
     lib = _lib.load()
     shape, n_iter, P, L, ctx2d = _Op._shape_from_index(msg_min_index)
     N = P * L

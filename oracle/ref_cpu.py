@@ -29,11 +29,12 @@ def module(name):
   return _mods[name]
 
 
-def forward(mode, unary, context, n_dir, n_iter, rho, saving_label=False):
+def forward(mode, unary, context, n_dir, n_iter, rho, saving_label=False, enable_sgm=False):
   """Run the reference ForwardCPU.  unary (B,cv,H,W,L) fp32, context a (n_dir,L,L)-strided
-  table (the CPU path reads `context + dir*L*L`, TRWP.cpp:205).  Returns msg, cost_final, label_all."""
+  table (the CPU path reads `context + dir*L*L`, TRWP.cpp:205).  Returns msg, cost_final, label_all
+  and unary_out (the SGM flag of ISGMR overwrites the unary tensor, ISGMR.cpp:255-261)."""
   import torch
-  unary = torch.as_tensor(unary, dtype=torch.float32).contiguous()
+  unary = torch.tensor(unary, dtype=torch.float32).contiguous()  # (a copy: may be overwritten)
   context = torch.as_tensor(context, dtype=torch.float32).contiguous()
   b, cv, h, w, L = unary.shape
   assert context.numel() >= n_dir * L * L
@@ -48,6 +49,7 @@ def forward(mode, unary, context, n_dir, n_iter, rho, saving_label=False):
                                empty_u8, empty_u8, scratch, label)
   else:
     msg_update = torch.zeros_like(msg)
-    module("ref_ISGMR").forward(0, float(rho), int(n_iter), 0, unary, context, edge, msg, cost,
-                                empty_u8, empty_u8, scratch, msg_update, label)
-  return dict(msg=msg.numpy(), cost_final=cost.numpy(), label_all=label.numpy())
+    module("ref_ISGMR").forward(int(bool(enable_sgm)), float(rho), int(n_iter), 0, unary, context,
+                                edge, msg, cost, empty_u8, empty_u8, scratch, msg_update, label)
+  return dict(msg=msg.numpy(), cost_final=cost.numpy(), label_all=label.numpy(),
+              unary_out=unary.numpy())

@@ -6,7 +6,8 @@ container (the reference tree does not travel):
     make -C oracle ref && python3 tests/golden/make_refcpu_golden.py
 
 Each fixture holds: mode, rho, n_dir, n_iter, unary (B,cv,H,W,L), context (n_dir,L,L) and the
-reference's msg, cost_final and label_all.  Inputs are integer valued in half of the cases so
+reference's msg, cost_final and label_all (the later ones also unary_out, the unary tensor after
+the call, which the SGM flag overwrites).  Fixtures that exist are kept unless --all is given.  Inputs are integer valued in half of the cases so
 that every fp32 operation is exact and comparisons can be bitwise.
 """
 import os
@@ -26,6 +27,11 @@ CASES = [
     ("isgmr_d4_l16", "ISGMR", 1.0, 4, 3, 1, 8, 12, 16, False, True),
     ("isgmr_d8_l21_int", "ISGMR", 1.0, 8, 3, 2, 5, 6, 21, True, False),
     ("isgmr_d16_l6", "ISGMR", 1.0, 16, 2, 1, 10, 11, 6, False, True),
+    # the SGM flag of the ISGMR operator (unary read at the current pixel and replaced after
+    # every iteration, ISGMR.cpp:72-77, 255-261) and the label loop at 256 labels (common.cpp:152)
+    ("sgm_d4_l8", "SGM", 1.0, 4, 2, 2, 6, 7, 8, False, True),
+    ("sgm_d8_l21_int", "SGM", 1.0, 8, 3, 1, 5, 6, 21, True, False),
+    ("trwp_d4_l256", "TRWP", 0.5, 4, 1, 1, 3, 4, 256, False, True),
 ]
 
 
@@ -46,10 +52,19 @@ def main():
     else:
       context = rng.integers(0, 6, (n_dir, L, L)).astype(np.float32) if integer else \
           rng.random((n_dir, L, L)).astype(np.float32)
-    out = ref_cpu.forward(mode, unary, context, n_dir, n_iter, rho, saving_label=True)
-    np.savez_compressed(os.path.join(HERE, "refcpu_%s.npz" % name), mode=mode, rho=rho,
+    path = os.path.join(HERE, "refcpu_%s.npz" % name)
+    if os.path.exists(path) and "--all" not in sys.argv:
+      continue  # fixtures already written are kept as they are
+    if name == "trwp_d4_l256":
+      context = context[:, :1, :].copy()  # one row per direction is all a 1-D table needs ...
+      context = np.concatenate([context.reshape(n_dir, L), np.zeros((n_dir, L * L - L), np.float32)],
+                               axis=1).reshape(n_dir, L, L)  # ... at the stride of a full table
+    out = ref_cpu.forward(mode, unary, context, n_dir, n_iter, rho, saving_label=True,
+                          enable_sgm=(mode == "SGM"))
+    np.savez_compressed(path, mode=mode, rho=rho,
                         n_dir=n_dir, n_iter=n_iter, unary=unary, context=context,
-                        msg=out["msg"], cost_final=out["cost_final"], label_all=out["label_all"])
+                        msg=out["msg"], cost_final=out["cost_final"], label_all=out["label_all"],
+                        unary_out=out["unary_out"])
     print(name, out["msg"].shape, float(np.abs(out["msg"]).max()))
 
 

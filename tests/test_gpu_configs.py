@@ -10,6 +10,11 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+# (the fixtures of the SGM flag pin the CPU forward alone, tests/test_cpu_forward.py: that flag
+# rewrites the unary tensor on the reference's CPU path, which neither the GPU semantics nor the
+# oracle's restatement of the CPU loop nest do)
+REFCPU_FIXTURES = [p for p in sorted(glob.glob(os.path.join(GOLDEN, "refcpu_*.npz")))
+                   if "refcpu_sgm" not in p]
 
 
 CONFIG_CASES = [
@@ -60,7 +65,7 @@ def test_config_matches_oracle(gpu, oracle, name, mode, scale, n_iter):
   assert abs(g[0].astype(np.float64).sum() - dcost.astype(np.float64).sum()) <= 1e-3 * np.abs(dcost).sum() ** 0.5 + 1e-2
 
 
-@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "refcpu_*.npz"))),
+@pytest.mark.parametrize("path", REFCPU_FIXTURES,
                          ids=lambda p: os.path.basename(p)[7:-4])
 def test_reference_cpu_fixtures(gpu, path):
   """Outputs of the reference's own compiled CPU forward (tests/golden/make_refcpu_golden.py).
