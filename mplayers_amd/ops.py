@@ -135,6 +135,8 @@ class TRWP(object):
     they start at zero and the library writes every element, so the caller need not clear it.
     flags (not in the reference): further per-call MPL_F_* bits of the C ABI."""
     if isinstance(unary, torch.Tensor) and not unary.is_cuda:
+      if msg_uninit:
+        msg.zero_()
       return _forward_cpu("TRWP", 0, rho, n_iter, unary, context, msg, cost_final, None, label_all)
     lib = _lib.load()
     shape, _, _ = _Op._check_forward(unary, context, edge_weights, msg, cost_final, msg_min_index,
@@ -186,6 +188,9 @@ class ISGMR(object):
               msg_uninit=False, flags=0):
     """msg_uninit, flags (not in the reference): see TRWP.forward."""
     if isinstance(unary, torch.Tensor) and not unary.is_cuda:
+      if msg_uninit:
+        msg.zero_()
+        msg_update.zero_()
       return _forward_cpu("ISGMR", enable_sgm, rho, n_iter, unary, context, msg, cost_final,
                           msg_update, label_all)
     lib = _lib.load()

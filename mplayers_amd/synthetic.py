@@ -90,11 +90,21 @@ CONFIGS = {
 }
 
 
-def make_config(name, seed=0, scale=1.0, mode=None, n_dir=None):
+def make_config(name, seed=0, scale=1.0, mode=None, n_dir=None, context=None, n_labels=None,
+                batch=None, n_iter=None):
   """Builds the inputs of configuration `name` (C1..C5).  scale < 1 shrinks H and W (parity tests
   at sizes a CPU checker finishes in seconds); mode overrides TRWP/ISGMR for the two-algorithm
-  configurations.  Returns a dict with the config fields plus unary, context, edge_weights."""
+  configurations.  n_labels, batch, n_iter run the same problem at another size; context
+  ("dense1d" / "dense2d") replaces the pairwise table by a learned-style dense one: random entries
+  in [0, 1), zero at offset 0 / on the diagonal (2-D: upper triangle, the part that is read).
+  Returns a dict with the config fields plus unary, context, edge_weights."""
   cfg = dict(CONFIGS[name])
+  if n_labels is not None:
+    cfg["L"] = int(n_labels)
+  if batch is not None:
+    cfg["B"] = int(batch)
+  if n_iter is not None:
+    cfg["n_iter"] = int(n_iter)
   if mode is not None:
     cfg["mode"] = mode
     cfg["rho"] = 0.5 if mode == "TRWP" else 1.0
@@ -110,9 +120,9 @@ def make_config(name, seed=0, scale=1.0, mode=None, n_dir=None):
     cfg["context"] = truncated_linear(L, 4, 0.5)
     cfg["edge_weights"] = torch.ones(n_dir, B, 1, H, W)
   elif name in ("C2", "C5"):
-    cfg["unary"] = stereo_unary(H, W, L, gen)
+    cfg["unary"] = torch.cat([stereo_unary(H, W, L, gen) for _ in range(B)], 0)
     cfg["context"] = truncated_linear(L, 2, 0.25) if name == "C2" else truncated_linear(L, 3, 0.3)
-    cfg["edge_weights"] = image_edge_weights(H, W, n_dir, gen)
+    cfg["edge_weights"] = torch.cat([image_edge_weights(H, W, n_dir, gen) for _ in range(B)], 1)
   elif name == "C3":
     cfg["unary"] = denoise_unary(H, W, L, gen)
     cfg["context"] = truncated_quadratic(L, 200, 25.0)
@@ -124,6 +134,16 @@ def make_config(name, seed=0, scale=1.0, mode=None, n_dir=None):
     cfg["edge_weights"] = ew.unsqueeze(1).permute(2, 0, 1, 3, 4).contiguous()
   else:
     raise KeyError(name)
+  if context == "dense1d":
+    c = torch.rand(L, generator=gen)
+    c[0] = 0.0
+    cfg["context"] = c
+  elif context == "dense2d":
+    if L != 21:
+      raise ValueError("the operators take a 2-D table with 21 labels only, as the reference does")
+    cfg["context"] = torch.triu(torch.rand(L, L, generator=gen), diagonal=1)
+  elif context is not None:
+    raise KeyError(context)
   cfg["units"] = B * H * W * L * cfg["n_iter"]
   return cfg
 

@@ -202,7 +202,7 @@ def test_large_config_properties_at_full_size(gpu, mode):
   from mplayers_amd import lib_stereo, synthetic
   cfg = synthetic.make_config("C5", seed=0, mode=mode)
   B, H, W, L, n_dir = cfg["B"], cfg["H"], cfg["W"], cfg["L"], cfg["n_dir"]
-  n_iter, rho = 2, cfg["rho"]
+  n_iter, rho = cfg["n_iter"], cfg["rho"]  # the 5 iterations the configuration states
   dev = "cuda:0"
   unary = cfg["unary"].to(dev)
   ctx = cfg["context"].to(dev)
@@ -321,7 +321,7 @@ def test_full_size_rows_match_oracle(gpu, oracle, mode):
   dev = "cuda:0"
   _check_rows(gpu, oracle, mode, cfg["unary"].to(dev), cfg["context"].to(dev),
               cfg["edge_weights"][:2].contiguous().to(dev), synthetic.upstream_grad(cfg).to(dev),
-              2, cfg["rho"], "full-size rows")
+              cfg["n_iter"], cfg["rho"], "full-size rows")
 
 
 @pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
@@ -370,7 +370,7 @@ def test_full_size_chains_match_oracle(gpu, oracle, mode, pair):
   cfg = synthetic.make_config("C5", seed=0, mode=mode)
   B, H, W, L = cfg["B"], cfg["H"], cfg["W"], cfg["L"]
   n_dir = 4 if pair < 4 else 8
-  n_iter, rho = 2, cfg["rho"]
+  n_iter, rho = cfg["n_iter"], cfg["rho"]
   dev = "cuda:0"
   unary = cfg["unary"].to(dev)
   ctx = cfg["context"].to(dev)
@@ -440,3 +440,130 @@ def test_full_size_chains_match_oracle(gpu, oracle, mode, pair):
     got_de = dedge[[pair, pair + 1]][:, :, :, hh, ww].cpu().numpy()[:, :, :, None]
     assert np.abs(got_du - du).max() <= 1e-4 * max(1.0, np.abs(du).max()), (h0, w0)
     assert np.abs(got_de - de).max() <= 1e-4 * max(1.0, np.abs(de).max()), (h0, w0)
+
+
+@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
+def test_module_at_full_size_equals_the_operators(gpu, mode):
+  """The large configuration as stated (1500 x 2000, 192 labels, 8 directions, 5 iterations)
+  through MPModule, the path a user of the layer takes: uninitialised buffers and messages that
+  start at zero by declaration.  Its cost and its gradients must be the ones the operators give
+  on zero-filled tensors under the reference's contract, bit for bit (dcontext, summed with float
+  atomics, to 1e-4), and the size-independent properties must hold."""
+  import torch
+  from mplayers_amd import MPModule, lib_stereo, synthetic
+  cfg = synthetic.make_config("C5", seed=0, mode=mode)
+  B, H, W, L, n_dir, n_iter, rho = (cfg[k] for k in ("B", "H", "W", "L", "n_dir", "n_iter", "rho"))
+  dev = "cuda:0"
+  args = argparse.Namespace(mpnet_mrf_mode=mode, mpnet_max_iter=n_iter, mpnet_n_dirs=n_dir,
+                            n_classes=L, mpnet_term_weight=1.0, mpnet_smoothness_train="",
+                            mpnet_diag_value=0, enable_symmetric=True)
+  mod = MPModule(args, enable_saving_label=True).cuda().train()
+  table = torch.nn.Parameter(cfg["context"].to(dev))
+  mod.set_label_context(table, np.arange(1, L), [0])
+  print("module at full size", mode, flush=True)
+  u = cfg["unary"].to(dev).permute(0, 1, 4, 2, 3).contiguous().requires_grad_(True)  # (B, cv, L, H, W)
+  e = cfg["edge_weights"][:, :, 0].permute(1, 0, 2, 3).contiguous().to(dev).requires_grad_(True)
+  g = synthetic.upstream_grad(cfg).to(dev)
+  cost, _, labels, _, _ = mod(u, e)
+  cost.backward(g.permute(0, 1, 4, 2, 3))
+  torch.cuda.synchronize()
+  cost_m = cost.detach().permute(0, 1, 3, 4, 2).contiguous()
+  du_m = u.grad.permute(0, 1, 3, 4, 2).contiguous()
+  de_m = e.grad.permute(1, 0, 2, 3).unsqueeze(2).contiguous()
+  dc_m = table.grad.clone()
+  assert torch.equal(cost_m.argmin(dim=-1).to(torch.uint8), labels[-1])
+  total = float(g.double().sum())
+  assert abs(float(du_m.double().sum()) - total) <= 1e-6 * float(g.double().abs().sum())
+  assert float(dc_m[0]) == 0.0 and bool(torch.isfinite(dc_m).all())
+  del cost, u, mod
+  torch.cuda.empty_cache()
+  # the operators on zero-filled tensors, flags = 0
+  unary = cfg["unary"].to(dev)
+  ctx = cfg["context"].to(dev)
+  ew = cfg["edge_weights"].to(dev)
+  msg = torch.zeros(n_dir, B, 1, H, W, L, device=dev)
+  cost = torch.zeros(B, 1, H, W, L, device=dev)
+  scratch = torch.zeros(B, 1, H, W, L, device=dev)
+  imin = torch.zeros(n_iter, n_dir, B, 1, H, W, L, dtype=torch.uint8, device=dev)
+  inorm = torch.zeros(n_iter, n_dir, B, 1, H, W, dtype=torch.uint8, device=dev)
+  empty = torch.empty(0, dtype=torch.uint8)
+  dunary = torch.zeros_like(cost)
+  dedge = torch.zeros(n_dir, B, 1, H, W, device=dev)
+  dctx = torch.zeros(L, device=dev)
+  if mode == "TRWP":
+    lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch, empty)
+    lib_stereo.TRWP.backward(rho, ctx, ew, g, imin, inorm, dunary, dctx, dedge, msg, scratch)
+  else:
+    msg_tmp = torch.zeros_like(msg)
+    lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch,
+                             msg_tmp, empty)
+    lib_stereo.ISGMR.backward(0, rho, ctx, ew, g, imin, inorm, dunary, dctx, dedge, msg, scratch,
+                              msg_tmp)
+  torch.cuda.synchronize()
+  assert torch.equal(cost_m, cost)
+  assert torch.equal(du_m, dunary)
+  assert torch.equal(de_m, dedge)
+  assert float((dc_m - dctx).abs().max()) <= 1e-4 * max(1.0, float(dctx.abs().max()))
+  print("peak memory %.1f GB" % (torch.cuda.max_memory_allocated() / 1e9), flush=True)
+  assert torch.cuda.max_memory_allocated() < 288e9
+
+
+@pytest.mark.parametrize("mode,L", [("TRWP", 21), ("ISGMR", 12), ("TRWP", 70)])
+def test_module_with_two_cost_volumes(gpu, oracle, mode, L):
+  """cv = 2: two cost volumes per batch item share the pairwise table and run as independent
+  problems (batch * cv of them, MP_module.py:36).  The module passes edge weights per batch item,
+  so they are left out here (the reference's (B, n_dir, H, W) maps do not cover a second volume);
+  the autograd Function takes them per volume."""
+  import torch
+  from mplayers_amd import MPModule
+  from mplayers_amd.MP_module import ISGMRFunction, TRWPFunction
+  rng = np.random.default_rng(L + 5)
+  B, cv, H, W, n_dir, n_iter = 2, 2, 6, 7, 4 if mode == "TRWP" else 8, 2
+  rho = 0.5 if mode == "TRWP" else 1.0
+  args = argparse.Namespace(mpnet_mrf_mode=mode, mpnet_max_iter=n_iter, mpnet_n_dirs=n_dir,
+                            n_classes=L, mpnet_term_weight=1.0, mpnet_smoothness_train="",
+                            mpnet_diag_value=0, enable_symmetric=True)
+  mod = MPModule(args, enable_saving_label=True).cuda().train()
+  if L == 21:
+    ctx = np.triu(rng.random((L, L)), 1).astype(np.float32)
+    loc, diag = np.triu_indices(L, k=1), [range(L), range(L)]
+  else:
+    ctx = np.concatenate([[0], rng.random(L - 1)]).astype(np.float32)
+    loc, diag = np.arange(1, L), [0]
+  table = torch.nn.Parameter(torch.from_numpy(ctx).cuda())
+  mod.set_label_context(table, loc, diag)
+  unary = rng.standard_normal((B, cv, L, H, W)).astype(np.float32)
+  dcost = rng.standard_normal((B, cv, L, H, W)).astype(np.float32)
+  u = torch.from_numpy(unary).cuda().requires_grad_(True)
+  cost, _, labels, _, _ = mod(u, None)
+  cost.backward(torch.from_numpy(dcost).cuda())
+  torch.cuda.synchronize()
+  un = np.ascontiguousarray(unary.transpose(0, 1, 3, 4, 2))
+  dn = np.ascontiguousarray(dcost.transpose(0, 1, 3, 4, 2))
+  ref = oracle.forward(mode, un, ctx, None, n_dir, n_iter, rho, saving_label=True, want_gaps=True)
+  got = cost.detach().cpu().numpy().transpose(0, 1, 3, 4, 2)
+  gpu.assert_values_close(got, ref["cost_final"], what="cost_final")
+  tol = 2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max()))
+  gpu.assert_labels_match_off_ties(labels.cpu().numpy(), ref["label_all"], ref["gap_label"], tol)
+  du, dc, _ = oracle.backward(mode, ctx, None, dn, ref["msg_min_index"], ref["msg_norm_index"], rho)
+  gu = u.grad.cpu().numpy().transpose(0, 1, 3, 4, 2)
+  assert np.abs(gu - du).max() <= 1e-4 * max(1.0, float(np.abs(du).max()))
+  assert np.abs(table.grad.cpu().numpy() - dc).max() <= 1e-4 * max(1.0, float(np.abs(dc).max()))
+  # the second volume is an independent problem: alone it gives the same numbers
+  u1 = torch.from_numpy(unary[:, 1:2]).cuda()
+  cost1 = mod(u1, None)[0]
+  assert torch.equal(cost1, cost[:, 1:2])
+  # the Function with edge weights per volume
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, cv, H, W))).astype(np.float32)
+  fn = TRWPFunction if mode == "TRWP" else ISGMRFunction
+  mod.args.training = True
+  uf = torch.from_numpy(un).cuda().requires_grad_(True)
+  ef = torch.from_numpy(ew).cuda().requires_grad_(True)
+  cf, _ = fn.apply(uf, table.detach(), ef, mod.args)
+  cf.backward(torch.from_numpy(dn).cuda())
+  torch.cuda.synchronize()
+  ref = oracle.forward(mode, un, ctx, ew, n_dir, n_iter, rho)
+  gpu.assert_values_close(cf.detach().cpu().numpy(), ref["cost_final"], what="cost_final (ew)")
+  du, _, de = oracle.backward(mode, ctx, ew, dn, ref["msg_min_index"], ref["msg_norm_index"], rho)
+  assert np.abs(uf.grad.cpu().numpy() - du).max() <= 1e-4 * max(1.0, float(np.abs(du).max()))
+  assert np.abs(ef.grad.cpu().numpy() - de).max() <= 1e-4 * max(1.0, float(np.abs(de).max()))
