@@ -68,6 +68,10 @@ def parse():
                        "1-D table of random entries, or a 2-D (L, L) table (at most 64 labels); the "
                        "scans then take their O(L^2) step and the roofline reported is the VALU one "
                        "(2 L lane-operations per label and direction sweep); not the headline workload")
+  ap.add_argument("--no-dense-flag", action="store_true",
+                  help="with --context: do not declare the table dense (one wavefront per chain)")
+  ap.add_argument("--split-waves", type=int, default=None,
+                  help="with --context: force this many wavefronts per chain (MPL_OPT_DENSE_SPLIT_WAVES)")
   ap.add_argument("--labels", type=int, default=None, help="run the configuration with this many labels")
   ap.add_argument("--batch", type=int, default=None, help="run the configuration at this batch size")
   ap.add_argument("--n-iter", type=int, default=None, help="run this many iterations")
@@ -335,11 +339,11 @@ class Workload(object):
   pass of every selected algorithm through the operators, exactly as the reference's callers
   drive them."""
 
-  def __init__(self, cfg, algs, training, dev, dunary_only=False, trwp_flags=0):
+  def __init__(self, cfg, algs, training, dev, dunary_only=False, trwp_flags=0, fwd_flags=0):
     import torch
     from mplayers_amd import synthetic
     self.cfg, self.algs, self.training = cfg, algs, training
-    self.dunary_only, self.trwp_flags = dunary_only, trwp_flags
+    self.dunary_only, self.trwp_flags, self.fwd_flags = dunary_only, trwp_flags, fwd_flags
     B, H, W, L, n_dir, n_iter = (cfg[k] for k in ("B", "H", "W", "L", "n_dir", "n_iter"))
     self.unary = cfg["unary"].to(dev)
     self.context = cfg["context"].to(dev)
@@ -389,13 +393,15 @@ class Workload(object):
                                                   w.dscratch)
       elif alg == "TRWP":
         lib_stereo.TRWP.forward(rho, n_iter, 0, w.unary, w.context, w.edge, w.msg, w.cost, w.imin,
-                                w.inorm, w.belief, w.empty, msg_uninit=uninit, flags=w.trwp_flags)
+                                w.inorm, w.belief, w.empty, msg_uninit=uninit,
+                                flags=w.trwp_flags | w.fwd_flags)
         if w.training:
           lib_stereo.TRWP.backward(rho, w.context, w.edge, w.dcost, w.imin, w.inorm, w.dunary,
                                    w.dctx, w.dedge, w.dmsg, w.dscratch, flags=w.trwp_flags)
       else:
         lib_stereo.ISGMR.forward(0, rho, n_iter, 0, w.unary, w.context, w.edge, w.msg, w.cost,
-                                 w.imin, w.inorm, w.belief, w.msg_tmp, w.empty, msg_uninit=uninit)
+                                 w.imin, w.inorm, w.belief, w.msg_tmp, w.empty, msg_uninit=uninit,
+                                 flags=w.fwd_flags)
         if w.training:
           lib_stereo.ISGMR.backward(0, rho, w.context, w.edge, w.dcost, w.imin, w.inorm, w.dunary,
                                     w.dctx, w.dedge, w.dmsg, w.dscratch, w.dmsg_tmp)
@@ -488,7 +494,12 @@ def main():
 
   uninit = bool(a.msg_uninit)
   trwp_flags = _lib.F_FUSED_PAIRS_OFF if a.no_fused_pairs else 0
-  work = Workload(cfg, algs, training, dev, dunary_only=a.dunary_only, trwp_flags=trwp_flags)
+  # a dense table is declared to the library (MPL_F_DENSE_TABLE) as a caller who trains one does
+  fwd_flags = _lib.F_DENSE_TABLE if (a.context is not None and not a.no_dense_flag) else 0
+  if a.split_waves is not None:
+    _lib.set_option(_lib.OPT_DENSE_SPLIT_WAVES, a.split_waves)
+  work = Workload(cfg, algs, training, dev, dunary_only=a.dunary_only, trwp_flags=trwp_flags,
+                  fwd_flags=fwd_flags)
   unary, edge, dcost = work.unary, work.edge, work.dcost
 
   if a.copy_probe:
@@ -557,7 +568,8 @@ def main():
                                              "fwd+bwd" if training else "fwd", B, H, W, L, n_dir,
                                              n_iter),
                  "scale": a.scale,
-                 "pairwise_table": a.context or "as the configuration states",
+                 "pairwise_table": (a.context + (", declared dense (MPL_F_DENSE_TABLE)" if fwd_flags
+                                                 else "")) if a.context else "as the configuration states",
                  "initial_messages": ("zero by declaration (MPL_F_MSG_UNINIT): the library writes "
                                       "every element itself" if uninit else
                                       "the reference's operator contract: `msg` cleared by the "

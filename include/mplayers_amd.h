@@ -70,7 +70,15 @@ typedef struct mpl_shape {
 /* TRWP calls: one launch per direction even where a launch has so few chains (at most one per
  * SIMD of the device) that the library would run both sweeps of a pair of opposite directions in
  * one. */
-#define MPL_F_ALL 0x3fu
+#define MPL_F_DENSE_TABLE 0x40u
+/* forward calls: the caller declares that its 1-D pairwise table is dense (a learned table, an
+ * untruncated one): no constant tail that the O(L) band scan could use, so the scans take their
+ * O(L^2) step.  With more than 64 labels, launches with fewer chains than about three per SIMD then
+ * put several wavefronts on every chain, each scanning a share of the front labels of a pixel.
+ * The kind of the table is otherwise only known on the device, after the launch is sized.  The
+ * results are the same bit for bit with and without the flag, whatever the table; a band table
+ * runs slower with it (its launches take the dense step). */
+#define MPL_F_ALL 0x7fu
 
 /* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.
  * msg: initial messages in, final normalised messages out.  msg_min_index/msg_norm_index NULL =>
@@ -305,6 +313,10 @@ const char* mpl_last_error(void);
 /* MPL_OPT_CPU_THREADS (default 0: 16, the reference's NUM_THREADS, tools/cpp/utils.h:17): threads
  * the mpl_*_forward_cpu calls spread their chains over. */
 #define MPL_OPT_CPU_THREADS 3
+/* MPL_OPT_DENSE_SPLIT_WAVES (default 0: the library chooses per launch): wavefronts per chain of
+ * the forward launches that MPL_F_DENSE_TABLE splits, at most 8 and at most what leaves every
+ * wavefront a front label (1: never split).  For tests and measurements. */
+#define MPL_OPT_DENSE_SPLIT_WAVES 4
 int mpl_set_option(int option, int value);
 
 /* Library version: major * 100 + minor. */

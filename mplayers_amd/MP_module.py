@@ -13,7 +13,7 @@ Tensor layouts (as in the reference):
 import torch
 import torch.nn as nn
 
-from . import lib_seg, lib_stereo
+from . import _lib, lib_seg, lib_stereo
 from .label_context import create_label_context
 from .layout import labels_first, labels_last
 
@@ -80,6 +80,12 @@ def _backward_buffers(dcost_final, message_index, with_message_tmp, need_context
   return buf
 
 
+def _table_flags(args):
+  """MPL_F_DENSE_TABLE when the module says its pairwise table is dense (not in the reference: the
+  kind of the table is only known on the device otherwise, see include/mplayers_amd.h)."""
+  return _lib.F_DENSE_TABLE if getattr(args, "dense_table", False) else 0
+
+
 class TRWPFunction(torch.autograd.Function):
   """Tree-reweighted message passing, Gauss-Seidel over directions (MP_module.py:17-86)."""
 
@@ -94,7 +100,7 @@ class TRWPFunction(torch.autograd.Function):
     _ops_for(n_disp).TRWP.forward(rho, n_iter, int(args.enable_min_a_dir), unary, label_context,
                                   edge_weights, buf["message"], buf["cost_final"],
                                   buf["message_index"], buf["cost_index"], buf["unary_update"],
-                                  buf["label_all"], msg_uninit=True)
+                                  buf["label_all"], msg_uninit=True, flags=_table_flags(args))
     ctx.intermediate_results = (rho, buf["message_index"], buf["cost_index"], label_context,
                                 edge_weights, enable_edge_weights)
     return buf["cost_final"], buf["label_all"]
@@ -131,7 +137,7 @@ class ISGMRFunction(torch.autograd.Function):
                                    unary, label_context, edge_weights, buf["message"],
                                    buf["cost_final"], buf["message_index"], buf["cost_index"],
                                    buf["unary_update"], buf["message_tmp"], buf["label_all"],
-                                   msg_uninit=True)
+                                   msg_uninit=True, flags=_table_flags(args))
     ctx.intermediate_results = (args.enable_sgm, rho, buf["message_index"], buf["cost_index"],
                                 label_context, edge_weights, enable_edge_weights)
     return buf["cost_final"], buf["label_all"]
@@ -218,6 +224,9 @@ class MPModule(torch.nn.Module):
       assert self.args.mpnet_max_iter == 1
     label_context = self._effective_label_context()
     self.args.training = self.training
+    # a table that is being learned is dense in general; args.mpnet_dense_table overrides the guess
+    dense = getattr(self.args, "mpnet_dense_table", None)
+    self.args.dense_table = bool(self.label_context.requires_grad if dense is None else dense)
     if self.args.mpnet_mrf_mode in {'ISGMR', 'SGM'}:
       cost_final, cost_all = ISGMRFunction.apply(unary, label_context, edge_weights, self.args)
     elif self.args.mpnet_mrf_mode == 'TRWP':

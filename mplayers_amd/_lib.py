@@ -30,6 +30,7 @@ F_PACKED_ALWAYS = 0x04
 F_FUSED_U_OFF = 0x08
 F_DCONTEXT_SAME_LABEL = 0x10
 F_FUSED_PAIRS_OFF = 0x20
+F_DENSE_TABLE = 0x40
 
 
 class KernelStat(ctypes.Structure):
@@ -92,6 +93,7 @@ OPT_PACKED_SCANS = 0
 OPT_FUSED_U = 1
 OPT_BELIEF_REBUILD = 2
 OPT_CPU_THREADS = 3
+OPT_DENSE_SPLIT_WAVES = 4
 BELIEF_REBUILD_DEFAULT = -1
 
 

@@ -527,12 +527,14 @@ int labels_per_lane(int L) { return (L + kWave - 1) / kWave; }
 std::atomic<int> g_packed_scans{1};  // MPL_OPT_PACKED_SCANS: 0 off, 1 by chain count, 2 always
 std::atomic<int> g_fused_u{1};       // MPL_OPT_FUSED_U
 std::atomic<int> g_belief_rebuild{MPL_BELIEF_REBUILD_DEFAULT};  // MPL_OPT_BELIEF_REBUILD
+std::atomic<int> g_split_waves{0};   // MPL_OPT_DENSE_SPLIT_WAVES: 0 = by the model of choose_split
 
 // what one call does, from its flags and the process defaults
 struct CallOpts {
   int packed;   // 0 off, 1 by chain count, 2 always
   bool fused_u;
   bool fused_pairs;
+  bool dense_table;
 };
 
 int read_flags(unsigned flags, const char* what, CallOpts* o) {
@@ -543,6 +545,7 @@ int read_flags(unsigned flags, const char* what, CallOpts* o) {
               : (flags & MPL_F_PACKED_ALWAYS) ? 2 : g_packed_scans.load(std::memory_order_relaxed);
   o->fused_u = (flags & MPL_F_FUSED_U_OFF) ? false : g_fused_u.load(std::memory_order_relaxed) != 0;
   o->fused_pairs = (flags & MPL_F_FUSED_PAIRS_OFF) == 0;
+  o->dense_table = (flags & MPL_F_DENSE_TABLE) != 0;
   return MPL_OK;
 }
 
@@ -556,6 +559,36 @@ int decide_pack(const mpl_shape* s, const Params& p, const CallOpts& o) {
   const int G = packed_chains_per_wave(s->batch, s->height, s->width, s->n_disp, s->ctx2d != 0,
                                        p.block_prefix[p.n_dirs], o.packed == 2);
   return G >= 2 ? G : 0;
+}
+
+// Wavefronts per chain for the forward scan of a launch whose caller declared a dense 1-D table
+// (MPL_F_DENSE_TABLE) with several labels per lane.  Four wavefronts, one on every SIMD of a
+// compute unit, each scanning a quarter of the front labels: the only count that keeps the SIMDs
+// of a unit evenly loaded, which matters because the wavefronts of a chain meet at a barrier every
+// pixel (2, 3, 6 and 8 wavefronts were measured slower than 4 at every size, 6 and 8 slower than
+// one).  A wavefront that shares its SIMD with others hides the wait states of the scan's
+// broadcasts and lane shifts, so the split gains more than the idle SIMDs it fills; it stops
+// paying once one wavefront per chain loads every SIMD evenly.  Measured on 192 labels, forward
+// scan, one wavefront against four (ms per launch): keeping argmin labels, 384 chains 11.6 / 5.8,
+// 768 chains 30.1 / 15.7, 1248 chains 55.3 / 40.2, 1536 chains 34.5 / 29.3, 2496 chains
+// 79.5 / 76.2, 3072 chains 48.3 / 55.7; without them 384 chains 6.6 / 3.9, 1248 chains
+// 34.0 / 29.8, 1536 chains 21.2 / 21.8, 2496 chains 51.3 / 57.2.
+template <typename Params>
+int choose_split(const mpl_shape* s, const Params& p, const CallOpts& o, bool train) {
+  if (!o.dense_table || s->ctx2d || s->n_disp <= kWave || p.pack >= 2) return 0;
+  const int L = s->n_disp, R = labels_per_lane(L);
+  const int forced = g_split_waves.load(std::memory_order_relaxed);
+  int w = 4;
+  if (forced > 0) {
+    w = forced;
+  } else {
+    const int64_t chains = p.block_prefix[p.n_dirs];
+    const int n_simd = launch_policy().n_simd;
+    if (2 * chains > (train ? 5 : 3) * (int64_t)n_simd) return 0;  // 2.5 / 1.5 chains per SIMD
+  }
+  // every wavefront needs a share of the front labels (they are visited R at a time)
+  while (w > 1 && (w - 1) * (((L + R * w - 1) / (R * w)) * R) >= L) --w;
+  return w >= 2 ? w : 0;
 }
 
 // wavefronts of a one-direction launch: one per chain, or one per group of p.pack chains
@@ -730,6 +763,11 @@ int mpl_set_option(int option, int value) {
     return MPL_OK;
   }
   if (option == MPL_OPT_CPU_THREADS) return set_cpu_threads(value);
+  if (option == MPL_OPT_DENSE_SPLIT_WAVES) {
+    if (value < 0 || value > 8) return fail(MPL_EINVAL, "set_option: 0 to 8 wavefronts per chain");
+    g_split_waves.store(value, std::memory_order_relaxed);
+    return MPL_OK;
+  }
   return fail(MPL_EINVAL, "set_option: unknown option %d", option);
 }
 
@@ -817,6 +855,7 @@ int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
     for (int d = 0; d < s->n_dir; ++d) {  // Gauss-Seidel over directions: TRWP_forward.cu:440-518
       fill_dirs(s, d, 1, p.dirs, p.block_prefix, &p.n_dirs);
       p.pack = decide_pack(s, p, opts);
+      p.split = choose_split(s, p, opts, train);
       p.first_iter = (it == 0);
       p.pair_q = 1;
       p.belief = (uninit && it == 0 && d <= 1) ? unary : unary_update;
@@ -888,6 +927,7 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
   // of small label counts run: they are bound by the instructions of a step, and two more loads
   // per step cost them more than the pass.)
   p.pack = decide_pack(s, p, opts);
+  p.split = choose_split(s, p, opts, train);
   const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && p.pack == 0;
   if (msg_uninit && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
   float* have = msg;  // the buffer that holds the current messages

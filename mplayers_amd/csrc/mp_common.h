@@ -469,6 +469,8 @@ struct SweepParams {
   uint8_t* idx_norm;               // (n_dir_total, P) of this iteration, or null
   int pack;                        // packed scans (mp_pack.hip): chains per wavefront; 0: one chain per
                                    // wavefront.  Decided once per launch by the host (mp_api.hip)
+  int split;                       // dense 1-D table, several labels per lane, few chains: wavefronts
+                                   // per chain that share the front labels of a pixel (0, 1: one)
   int pair_q;                      // Gauss-Seidel: belief plane holds Q between the sweeps of a pair
   int skip_s_store;                // Gauss-Seidel: last sweep of the call, nobody reads S after it
   int fused_pair;                  // Gauss-Seidel: every wavefront sweeps dirs[0], then dirs[0] ^ 1

@@ -67,22 +67,25 @@ __device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&val
 // label (c[|cd - (fd+1)|] of label cd is c[|(cd-1) - fd|] of label cd - 1; c[fd+1] enters at
 // label 0).  `<=` on the ascending scan keeps the largest front label among equals, as the
 // reference's descending scan with `<` does.
+// The scan covers the front labels fd_lo .. fd_hi - 1 (fd_lo a multiple of R): all of them, or the
+// share of one wavefront where several scan a pixel together (split_combine below).
 template <int R, bool TRAIN, bool WHOLE>  // WHOLE: L is a multiple of R
 __device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L, int lab0,
-                                             const float* ctx_s, float (&v)[R], int (&fd_idx)[R]) {
+                                             const float* ctx_s, float (&v)[R], int (&fd_idx)[R],
+                                             const int fd_lo, const int fd_hi) {
   float c_own[R], cv[R];  // c[label] of the lane's labels; the sliding c[|label - fd|]
 #pragma unroll
   for (int j = 0; j < R; ++j) {
-    const int l = lab0 + j;
-    c_own[j] = ctx_s[l < L ? l : L - 1];
-    cv[j] = c_own[j];
+    const int l = lab0 + j < L ? lab0 + j : L - 1;
+    c_own[j] = ctx_s[l];
+    cv[j] = fd_lo == 0 ? c_own[j] : ctx_s[l > fd_lo ? l - fd_lo : fd_lo - l];
     v[j] = INFINITY;
     fd_idx[j] = L - 1;
   }
   // the weight in a vector register: a multiply-add takes one scalar operand, and that is a[fd]
   float wv = w;
   asm volatile("" : "+v"(wv));
-  for (int fd0 = 0; fd0 < L; fd0 += R) {
+  for (int fd0 = fd_lo; fd0 < fd_hi; fd0 += R) {
     const int src = fd0 / R;  // the lane that owns front labels fd0 .. fd0 + R - 1
 #pragma unroll
     for (int u = 0; u < R; ++u) {
@@ -107,6 +110,43 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L
 #pragma unroll
         for (int j = R - 1; j > 0; --j) cv[j] = cv[j - 1];
         cv[0] = in0;
+      }
+    }
+  }
+}
+
+// Several wavefronts on one chain (launches with far fewer chains than the chip has SIMDs, dense
+// table): every wavefront of the workgroup walks the chain and holds the same state, but scans only
+// its share of the front labels of a pixel; the partial minima (and their labels) meet in LDS,
+// one slot per wavefront, and every wavefront folds all of them in the order of the front labels
+// (`<=`: the later share wins ties, as the one scan over all front labels does), so the state stays
+// identical in all of them, bit for bit what one wavefront computes.  Two sets of slots alternate:
+// a wavefront that runs ahead writes the other set, and it cannot reach this set again before the
+// barrier of the next step, which every wavefront passes only after it has read this one.
+template <int R, bool TRAIN>
+__device__ __forceinline__ void split_combine(float* xchg, int n_waves, int wave, int lane, int parity,
+                                              float (&v)[R], int (&fd_idx)[R]) {
+  constexpr int S = TRAIN ? 2 * R : R;  // dwords per lane and slot
+  float* set = xchg + (size_t)parity * n_waves * kWave * S;
+  float* mine = set + ((size_t)wave * kWave + lane) * S;
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    mine[j] = v[j];
+    if (TRAIN) mine[R + j] = __builtin_bit_cast(float, fd_idx[j]);
+  }
+  __syncthreads();
+  for (int k = 0; k < n_waves; ++k) {
+    const float* theirs = set + ((size_t)k * kWave + lane) * S;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const float pv = theirs[j];
+      if (TRAIN) {
+        const int pi = __builtin_bit_cast(int, theirs[R + j]);
+        const bool take = (k == 0) || (pv <= v[j]);
+        v[j] = take ? pv : v[j];
+        fd_idx[j] = take ? pi : fd_idx[j];
+      } else {
+        v[j] = k == 0 ? pv : fminf(v[j], pv);
       }
     }
   }
@@ -382,12 +422,14 @@ __device__ __forceinline__ void linear_step(const float (&a)[R], float w, float 
 }
 
 // One chain.  KT: > 0 band with compile-time K, 0 band with run-time K, -1 dense, -21 dense with
-// exactly 21 labels, -2 truncated linear context of any width (linear_step).
+// exactly 21 labels, -2 truncated linear context of any width (linear_step), -3 dense 1-D table with
+// the front labels split over the wavefronts of the workgroup (split_combine; xchg: its LDS slots).
 // VEC: L % R == 0 (vector accesses).  MASK: some lanes own labels >= L.
 template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI, int KT>
 __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
                                               const ChainCtx& ch, float* a_s, const float* ctx_s,
-                                              const bool skip_s_store) {
+                                              const bool skip_s_store, float* xchg = nullptr) {
+  constexpr bool SPLIT = (KT == -3);
   const int L = p.L;
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t P = (int64_t)p.B * HW;
@@ -416,10 +458,18 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
                                   TRAIN ? (int)HW : 0);
   const float rho = p.rho;
   const float inf = INFINITY;
-  const int lane = threadIdx.x;
+  const int lane = SPLIT ? (int)(threadIdx.x & (kWave - 1)) : (int)threadIdx.x;
   const int lab0 = R * lane;
   const int foff = lab0 * 4;  // byte offset of this lane's block inside a pixel's float vector
   const int n = ch.n;
+  // SPLIT: the wavefronts of the workgroup share the front labels; the first one stores
+  const int wave = SPLIT ? uniform_i((int)(threadIdx.x / kWave)) : 0;
+  const int n_waves = SPLIT ? (int)(blockDim.x / kWave) : 1;
+  const bool store_ok = !SPLIT || wave == 0;
+  // front labels per wavefront: a multiple of R (the scan visits them R at a time)
+  const int fd_chunk = SPLIT ? ((L + R * n_waves - 1) / (R * n_waves)) * R : L;
+  const int fd_lo = SPLIT ? min(wave * fd_chunk, L) : 0;
+  const int fd_hi = SPLIT ? min(fd_lo + fd_chunk, L) : L;
 
   bool valid[R];
 #pragma unroll
@@ -528,13 +578,20 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       }
       uf[j] = valid[j] ? un : inf;
     }
+    if constexpr (SPLIT) {
+      // the first wavefront is about to overwrite the start pixel's entry of the belief plane, in
+      // place: not before every wavefront of the chain has read it
+      wait_vmem<0>();
+      __syncthreads();
+    }
     const unsigned so0 = (unsigned)ch.pix0 * (unsigned)vbytes;
-    const int vo0 = (int)(lane_ok ? so0 + (unsigned)foff : kDeadWide);
+    const int vo0 = (int)((lane_ok && store_ok) ? so0 + (unsigned)foff : kDeadWide);
+    const int nrec0 = store_ok ? (int)(so0 + (unsigned)vbytes) : 0;
     if (!JACOBI && p.pair_q && !skip_s_store) {
       if constexpr (VEC)
         buf_store<R, true>(rSo, vo0, 0u, conv);
       else
-        buf_store<R, VEC>(make_rsrc(bSo, (int)(so0 + (unsigned)vbytes)), foff, so0, conv);
+        buf_store<R, VEC>(make_rsrc(bSo, nrec0), foff, so0, conv);
     }
     if (JACOBI || p.zero_start) {
       float z[R];
@@ -543,7 +600,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       if constexpr (VEC)
         buf_store<R, true>(rMo, vo0, 0u, z);
       else
-        buf_store<R, VEC>(make_rsrc(bMo, (int)(so0 + (unsigned)vbytes)), foff, so0, z);
+        buf_store<R, VEC>(make_rsrc(bMo, nrec0), foff, so0, z);
     }
   }
 
@@ -643,10 +700,12 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
           dense_step_r1<TRAIN>(a[0], L, w, lane, ctx_s, v[0], fd_idx[0]);
         }
       } else if (live) {
-        if constexpr (R > 1)  // (2-D tables exist for one label per lane only)
-          dense1d_step<R, TRAIN, VEC>(a, w, L, lab0, ctx_s, v, fd_idx);
-        else
+        if constexpr (R > 1) {  // (2-D tables exist for one label per lane only)
+          dense1d_step<R, TRAIN, VEC>(a, w, L, lab0, ctx_s, v, fd_idx, fd_lo, fd_hi);
+          if constexpr (SPLIT) split_combine<R, TRAIN>(xchg, n_waves, wave, lane, t & 1, v, fd_idx);
+        } else {
           dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
+        }
       } else {
 #pragma unroll
         for (int j = 0; j < R; ++j) {
@@ -672,17 +731,17 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       const unsigned so = sp * (unsigned)vbytes;
       const unsigned sob = sp * (unsigned)L;
       if constexpr (VEC) {
-        const bool on = lane_ok && live;  // nothing is stored past the end
+        const bool on = lane_ok && live && store_ok;  // nothing is stored past the end
         const int vo = (int)(on ? so + (unsigned)foff : kDeadWide);
         buf_store<R, true>(rMo, vo, 0u, m);
         if (!JACOBI) buf_store<R, true>(rSo, vo, 0u, sn);
         if (TRAIN) buf_store_u8<R, true>(rImin, (int)(on ? sob + (unsigned)lab0 : kDeadWide), 0u, fd_idx);
       } else {
-        const int nrec = live ? (int)(so + (unsigned)vbytes) : 0;
+        const int nrec = (live && store_ok) ? (int)(so + (unsigned)vbytes) : 0;
         buf_store<R, VEC>(make_rsrc(bMo, nrec), foff, so, m);
         if (!JACOBI) buf_store<R, VEC>(make_rsrc(bSo, skip_s_store ? 0 : nrec), foff, so, sn);
         if (TRAIN)
-          buf_store_u8<R, VEC>(make_rsrc(bImin, live ? (int)(sob + (unsigned)L) : 0), lab0, sob, fd_idx);
+          buf_store_u8<R, VEC>(make_rsrc(bImin, (live && store_ok) ? (int)(sob + (unsigned)L) : 0), lab0, sob, fd_idx);
       }
       if (TRAIN) {
         bool pr[R];
@@ -690,7 +749,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         for (int j = 0; j < R; ++j) pr[j] = valid[j] && (v[j] == nmin);
         const int nidx = last_label<R>(pr, L - 1);
         // every lane stores the same byte to the same address
-        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm, live ? (int)sp : kDeadOffset, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)nidx, dInorm, (live && store_ok) ? (int)sp : kDeadOffset, 0, 0);
       }
       st_p += ch.pstep;
   };
@@ -802,8 +861,80 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
   }
 }
 
+// A dense 1-D table in a launch with far fewer chains than the chip has SIMDs (p.split wavefronts
+// per chain, chosen by the host; several labels per lane only).  Every wavefront of the workgroup
+// runs the chain; see split_combine.
+constexpr int kSplitMaxWaves = 8;
+template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI>
+__global__ void __launch_bounds__(kSplitMaxWaves * kWave) sweep_fwd_split_kernel(const SweepParams p) {
+  extern __shared__ float smem[];
+  float* a_s = smem;            // kMaxL floats (unused by this scan)
+  float* ctx_s = smem + kMaxL;  // L floats
+  float* xchg = ctx_s + ((p.L + 3) & ~3);
+  const int L = p.L;
+  const ChainCtx ch = locate_chain(p);
+  if (!JACOBI && !p.pair_q && ch.n < 2) return;  // nothing to write (the same for every wavefront)
+  CtxDesc desc;
+  desc.band_k = 0;  // the dense scan is exact for any table; the descriptor only says whether
+  desc.c0_is_min = 0;  // the initial messages are zero
+  desc.cmax = 0.f;
+  desc.msg_nonzero = p.desc != nullptr ? p.desc->msg_nonzero : 1;
+  desc.linear = 0;
+  desc.slope = 0.f;
+  for (int i = threadIdx.x; i < L; i += blockDim.x) ctx_s[i] = p.ctx[i];
+  __syncthreads();
+  const int halves = (!JACOBI && p.fused_pair) ? 2 : 1;
+#pragma clang loop unroll(disable)
+  for (int half = 0; half < halves; ++half) {
+    ChainCtx c = ch;
+    bool skip_s = p.skip_s_store != 0;
+    if (half) {
+      c.dir = ch.dir ^ 1;
+      c.pix0 = ch.pix0 + (ch.n - 1) * ch.pstep;
+      c.pstep = -ch.pstep;
+      skip_s = p.skip_s_store2 != 0;
+      wait_vmem<0>();
+      __syncthreads();
+    }
+    run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -3>(p, desc, c, a_s, ctx_s, skip_s, xchg);
+  }
+}
+
+inline size_t split_lds_bytes(int L, int R, int waves, bool train) {
+  return sizeof(float) * (kMaxL + ((L + 3) & ~3) + (size_t)2 * waves * kWave * (train ? 2 * R : R));
+}
+
+template <int R, bool VEC, bool MASK>
+void launch_vm_split(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+  const int blocks = p.block_prefix[p.n_dirs];
+  const int threads = p.split * kWave;
+  const size_t lds = split_lds_bytes(p.L, R, p.split, train);
+  const int mode = jacobi ? (p.u_fused ? 2 : 1) : 0;
+  if (train) {
+    if (mode == 2)
+      sweep_fwd_split_kernel<R, VEC, MASK, true, 2><<<blocks, threads, lds, st>>>(p);
+    else if (mode == 1)
+      sweep_fwd_split_kernel<R, VEC, MASK, true, 1><<<blocks, threads, lds, st>>>(p);
+    else
+      sweep_fwd_split_kernel<R, VEC, MASK, true, 0><<<blocks, threads, lds, st>>>(p);
+  } else {
+    if (mode == 2)
+      sweep_fwd_split_kernel<R, VEC, MASK, false, 2><<<blocks, threads, lds, st>>>(p);
+    else if (mode == 1)
+      sweep_fwd_split_kernel<R, VEC, MASK, false, 1><<<blocks, threads, lds, st>>>(p);
+    else
+      sweep_fwd_split_kernel<R, VEC, MASK, false, 0><<<blocks, threads, lds, st>>>(p);
+  }
+}
+
 template <int R, bool VEC, bool MASK>
 void launch_vm(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+  if constexpr (R > 1) {
+    if (p.split >= 2 && !p.ctx2d) {
+      launch_vm_split<R, VEC, MASK>(p, train, jacobi, st);
+      return;
+    }
+  }
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = fwd_lds_bytes(p.L, p.ctx2d);
   const int mode = jacobi ? (p.u_fused ? 2 : 1) : 0;
