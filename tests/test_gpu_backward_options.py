@@ -109,3 +109,79 @@ def test_per_call_flags_override_the_process_default(gpu, oracle):
   assert np.array_equal(always_default[0], always_by_flag[0])
   assert not np.array_equal(off_default[2], always_default[2])
   assert np.abs(off_default[2] - always_default[2]).max() <= 1e-4 * np.abs(off_default[2]).max()
+
+
+@pytest.mark.parametrize("mode,L", [("TRWP", 21), ("ISGMR", 12), ("TRWP", 96)])
+@pytest.mark.parametrize("with_edge_weights", [True, False])
+def test_module_with_a_frozen_table(gpu, mode, L, with_edge_weights):
+  """autograd's needs_input_grad decides which gradients the backward operators are asked for:
+  with a table that is not trained and edge weights that need no gradient the module hands the
+  operators no dcontext / dedge_weights tensor.  dunary must be the bits of the run that computes
+  everything, and the gradients that were not asked for come back as None."""
+  import argparse
+  import torch
+  from mplayers_amd import MPModule
+  rng = np.random.default_rng(L + 1)
+  B, H, W, n_dir, n_iter = 2, 6, 7, 4, 2
+  args = argparse.Namespace(mpnet_mrf_mode=mode, mpnet_max_iter=n_iter, mpnet_n_dirs=n_dir,
+                            n_classes=L, mpnet_term_weight=1.0, mpnet_smoothness_train="",
+                            mpnet_diag_value=0, enable_symmetric=True)
+  if L == 21:
+    ctx = np.triu(rng.random((L, L)), 1).astype(np.float32)
+    loc, diag = np.triu_indices(L, k=1), [range(L), range(L)]
+  else:
+    ctx = np.concatenate([[0], rng.random(L - 1)]).astype(np.float32)
+    loc, diag = np.arange(1, L), [0]
+  unary = torch.from_numpy(rng.standard_normal((B, 1, L, H, W)).astype(np.float32)).cuda()
+  ew = torch.from_numpy((0.1 + 0.9 * rng.random((B, n_dir, H, W))).astype(np.float32)).cuda()
+  dcost = torch.from_numpy(rng.standard_normal((B, 1, L, H, W)).astype(np.float32)).cuda()
+
+  def run(train_table, train_edges):
+    mod = MPModule(args).cuda().train()
+    table = torch.nn.Parameter(torch.from_numpy(ctx).cuda(), requires_grad=train_table)
+    mod.set_label_context(table, loc, diag)
+    u = unary.clone().requires_grad_(True)
+    e = ew.clone().requires_grad_(train_edges) if with_edge_weights else None
+    cost = mod(u, e)[0]
+    cost.backward(dcost)
+    torch.cuda.synchronize()
+    return cost.detach(), u.grad, table.grad, (e.grad if e is not None else None)
+
+  full = run(True, True)
+  frozen = run(False, False)
+  assert torch.equal(frozen[0], full[0])
+  assert torch.equal(frozen[1], full[1])
+  assert frozen[2] is None and frozen[3] is None
+  assert full[2] is not None and float(full[2].abs().max()) > 0
+  assert (full[3] is not None) == with_edge_weights
+  table_only = run(True, False)
+  assert torch.equal(table_only[1], full[1]) and table_only[3] is None
+  assert float((table_only[2] - full[2]).abs().max()) <= 1e-5 * max(1.0, float(full[2].abs().max()))
+
+
+def test_hard_soft_module_with_a_frozen_table(gpu):
+  """The hard path of the hard/soft module (which asks for the same-label dcontext terms) with
+  and without a trained table: the same dunary bits, no table gradient when it is frozen."""
+  import argparse
+  import torch
+  from mplayers_amd.MP_module_hard_soft import MPModule as MPModule_hard_soft
+  rng = np.random.default_rng(77)
+  B, L, H, W, n_dir, n_iter = 2, 21, 6, 7, 4, 2
+  unary = torch.from_numpy(rng.standard_normal((B, 1, L, H, W)).astype(np.float32)).cuda()
+  dcost = torch.from_numpy(rng.standard_normal((B, 1, L, H, W)).astype(np.float32)).cuda()
+  outs = []
+  for smoothness_train in ("on", ""):
+    args = argparse.Namespace(mpnet_mrf_mode="TRWP", mpnet_max_iter=n_iter, mpnet_n_dirs=n_dir,
+                              n_classes=L, mpnet_term_weight=1.0,
+                              mpnet_smoothness_train=smoothness_train, mpnet_smoothness_mode="Potts",
+                              mpnet_smoothness_trunct_value=-1, mpnet_smoothness_trunct_loc=-1,
+                              mpnet_diag_value=0, enable_symmetric=True, mpnet_enable_soft=False,
+                              enable_cuda=True)
+    mod = MPModule_hard_soft(args, enable_create_label_context=True).cuda().train()
+    u = unary.clone().requires_grad_(True)
+    cost = mod(u, None)[0]
+    cost.backward(dcost)
+    torch.cuda.synchronize()
+    outs.append((cost.detach(), u.grad, mod.label_context.grad))
+  assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+  assert outs[0][2] is not None and outs[1][2] is None

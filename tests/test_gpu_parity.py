@@ -196,6 +196,19 @@ def test_backward_of_many_short_chains(gpu, oracle, mode, L, kind):
     scale = max(1.0, float(np.abs(r).max()))
     assert np.abs(g - r).max() <= 1e-4 * scale, (name, float(np.abs(g - r).max()), scale)
   assert got[1][0] == 0
+  if mode == "TRWP":
+    # the hard backward of the TRWP_hard_soft build on the same launches: entry 0 of the table
+    # also collects the pairs whose front label is their own (one label per lane, popular-target
+    # shortcuts: the accumulator of label 0 is gathered twice and halved at the flush)
+    ref = oracle.backward(mode, ctx.astype(np.float64), ew.astype(np.float64),
+                          dcost.astype(np.float64), fwd["msg_min_index"], fwd["msg_norm_index"],
+                          rho, same_label=True)
+    got = gpu.gpu_backward(mode, ctx, ew, dcost, fwd["msg_min_index"], fwd["msg_norm_index"], rho,
+                           garbage_scratch=True, hard_soft=True)
+    assert abs(ref[1][0]) > 1e-3
+    for g, r, name in zip(got, ref, ("dunary", "dcontext", "dedge_weights")):
+      scale = max(1.0, float(np.abs(r).max()))
+      assert np.abs(g - r).max() <= 1e-4 * scale, (name, float(np.abs(g - r).max()), scale)
 
 
 def test_sgm_flag(gpu, oracle):
