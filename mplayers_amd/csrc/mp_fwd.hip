@@ -85,33 +85,42 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L
   // the weight in a vector register: a multiply-add takes one scalar operand, and that is a[fd]
   float wv = w;
   asm volatile("" : "+v"(wv));
-  for (int fd0 = fd_lo; fd0 < fd_hi; fd0 += R) {
-    const int src = fd0 / R;  // the lane that owns front labels fd0 .. fd0 + R - 1
+  // one front label: fd = fd0 + u is owned by lane src = fd0 / R, register u
+  auto visit = [&](const int fd, const int u, const int src) __attribute__((always_inline)) {
+    const float af = readlane_f(a[u], src);
+    // c[fd + 1]: the next label's own entry (past the last label the value is never used)
+    const float cn = u + 1 < R ? readlane_f(c_own[u + 1 < R ? u + 1 : 0], src)
+                               : readlane_f(c_own[0], (src + 1) & 63);
 #pragma unroll
-    for (int u = 0; u < R; ++u) {
-      const int fd = fd0 + u;
-      if (WHOLE || fd < L) {  // wave-uniform
-        const float af = readlane_f(a[u], src);
-        // c[fd + 1]: the next label's own entry (past the last label the value is never used)
-        const float cn = u + 1 < R ? readlane_f(c_own[u + 1 < R ? u + 1 : 0], src)
-                                   : readlane_f(c_own[0], (src + 1) & 63);
-#pragma unroll
-        for (int j = 0; j < R; ++j) {
-          const float val = fmaf(wv, cv[j], af);
-          if (TRAIN) {
-            const bool take = val <= v[j];
-            v[j] = take ? val : v[j];
-            fd_idx[j] = take ? fd : fd_idx[j];
-          } else {
-            v[j] = fminf(v[j], val);
-          }
-        }
-        const float in0 = wave_shr1(cv[R - 1], cn);
-#pragma unroll
-        for (int j = R - 1; j > 0; --j) cv[j] = cv[j - 1];
-        cv[0] = in0;
+    for (int j = 0; j < R; ++j) {
+      const float val = fmaf(wv, cv[j], af);
+      if (TRAIN) {
+        // (the minimum and the comparison are independent instructions; a select of the value
+        // would wait for the comparison's lane mask like the select of the label does)
+        const bool take = val <= v[j];
+        v[j] = fminf(v[j], val);
+        fd_idx[j] = take ? fd : fd_idx[j];
+      } else {
+        v[j] = fminf(v[j], val);
       }
     }
+    const float in0 = wave_shr1(cv[R - 1], cn);
+#pragma unroll
+    for (int j = R - 1; j > 0; --j) cv[j] = cv[j - 1];
+    cv[0] = in0;
+  };
+  // Two rounds of R front labels per trip: after R one-label shifts the sliding values sit in
+  // registers the shifts created, after 2 R they can be back in the ones the trip started with,
+  // so the loop carries no register moves.
+  int fd0 = fd_lo;
+  for (; fd0 + 2 * R <= fd_hi; fd0 += 2 * R) {
+#pragma unroll
+    for (int u = 0; u < 2 * R; ++u) visit(fd0 + u, u % R, (fd0 + u) / R);
+  }
+  for (; fd0 < fd_hi; fd0 += R) {
+#pragma unroll
+    for (int u = 0; u < R; ++u)
+      if (WHOLE || fd0 + u < fd_hi) visit(fd0 + u, u, fd0 / R);  // wave-uniform
   }
 }
 
