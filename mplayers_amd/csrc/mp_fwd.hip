@@ -113,14 +113,15 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L
   // registers the shifts created, after 2 R they can be back in the ones the trip started with,
   // so the loop carries no register moves.
   int fd0 = fd_lo;
-  for (; fd0 + 2 * R <= fd_hi; fd0 += 2 * R) {
+  int src0 = fd_lo / R;  // the lane that owns front label fd0 (counted along: no division per trip)
+  for (; fd0 + 2 * R <= fd_hi; fd0 += 2 * R, src0 += 2) {
 #pragma unroll
-    for (int u = 0; u < 2 * R; ++u) visit(fd0 + u, u % R, (fd0 + u) / R);
+    for (int u = 0; u < 2 * R; ++u) visit(fd0 + u, u % R, src0 + u / R);
   }
-  for (; fd0 < fd_hi; fd0 += R) {
+  for (; fd0 < fd_hi; fd0 += R, ++src0) {
 #pragma unroll
     for (int u = 0; u < R; ++u)
-      if (WHOLE || fd0 + u < fd_hi) visit(fd0 + u, u, fd0 / R);  // wave-uniform
+      if (WHOLE || fd0 + u < fd_hi) visit(fd0 + u, u, src0);  // wave-uniform
   }
 }
 
@@ -476,9 +477,12 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   const int n_waves = SPLIT ? (int)(blockDim.x / kWave) : 1;
   const bool store_ok = !SPLIT || wave == 0;
   // front labels per wavefront: a multiple of R (the scan visits them R at a time)
-  const int fd_chunk = SPLIT ? ((L + R * n_waves - 1) / (R * n_waves)) * R : L;
-  const int fd_lo = SPLIT ? min(wave * fd_chunk, L) : 0;
-  const int fd_hi = SPLIT ? min(fd_lo + fd_chunk, L) : L;
+  // (the division by the number of wavefronts runs on the vector unit: without the explicit
+  // read-back the bounds, and with them the loop counter of the scan and every lane index it
+  // forms, would stay in vector registers)
+  const int fd_chunk = SPLIT ? uniform_i(((L + R * n_waves - 1) / (R * n_waves)) * R) : L;
+  const int fd_lo = SPLIT ? uniform_i(min(wave * fd_chunk, L)) : 0;
+  const int fd_hi = SPLIT ? uniform_i(min(fd_lo + fd_chunk, L)) : L;
 
   bool valid[R];
 #pragma unroll
