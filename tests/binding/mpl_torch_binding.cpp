@@ -17,8 +17,10 @@ namespace {
 
 // CHECK_CONTIGUOUS of the reference (tools/cuda/cudaUtils.hpp:10) plus what the reference leaves
 // unchecked and the C ABI relies on: device, dtype and size of every tensor
-void check(const at::Tensor& t, const char* name, at::ScalarType dtype, int64_t numel) {
-  TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor (this build has no CPU path)");
+void check(const at::Tensor& t, const char* name, at::ScalarType dtype, int64_t numel,
+           bool cuda = true) {
+  TORCH_CHECK(t.is_cuda() == cuda, name, cuda ? " must be a GPU tensor like the rest of the call"
+                                              : " must be a CPU tensor like the rest of the call");
   TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
   TORCH_CHECK(t.scalar_type() == dtype, name, " has the wrong dtype");
   TORCH_CHECK(t.numel() >= numel, name, " has ", t.numel(), " elements, ", numel, " needed");
@@ -92,6 +94,22 @@ void check_backward(const mpl_shape& s, int n_iter, const at::Tensor& context,
   check(dedge_weights, "dedge_weights", at::kFloat, s.n_dir * P);
 }
 
+// Tensors that are not on the GPU: ForwardCPU of the reference (TRWP.cpp:172-243 reached from
+// :275-282, ISGMR.cpp:190-298 from :330-339) through the library's CPU entry points.  That path
+// reads one pairwise table per direction at context + d * n_disp^2 and ignores edge weights,
+// indices and unary_update.
+void check_forward_cpu(const mpl_shape& s, int n_iter, const at::Tensor& unary,
+                       const at::Tensor& context, const at::Tensor& msg,
+                       const at::Tensor& cost_final, const at::Tensor& label_all) {
+  const int64_t P = pixels(s), N = P * s.n_disp;
+  check(unary, "unary", at::kFloat, N, false);
+  check(context, "context", at::kFloat,
+        (int64_t)(s.n_dir - 1) * s.n_disp * s.n_disp + context_numel(s), false);
+  check(msg, "msg", at::kFloat, s.n_dir * N, false);
+  check(cost_final, "cost_final", at::kFloat, N, false);
+  if (label_all.numel() > 0) check(label_all, "label_all", at::kByte, (int64_t)n_iter * P, false);
+}
+
 void* current_stream(const at::Tensor& t) {
   return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream();
 }
@@ -103,6 +121,14 @@ void Forward(const float rho, const int n_iter, const int enable_min_a_dir, cons
              at::Tensor cost_final, at::Tensor msg_min_index, at::Tensor msg_norm_index,
              at::Tensor unary_update, at::Tensor label_all) {
   const mpl_shape s = shape_of(msg);
+  if (!unary.is_cuda()) {
+    check_forward_cpu(s, n_iter, unary, context, msg, cost_final, label_all);
+    const int rc = mpl_trwp_forward_cpu(&s, rho, n_iter, unary.data_ptr<float>(),
+                                        context.data_ptr<float>(), msg.data_ptr<float>(),
+                                        cost_final.data_ptr<float>(), u8_or_null(label_all));
+    TORCH_CHECK(rc == MPL_OK, "TRWP.forward: ", mpl_last_error());
+    return;
+  }
   check_forward(s, n_iter, unary, context, edge_weights, msg, cost_final, msg_min_index,
                 msg_norm_index, unary_update, label_all);
   const c10::DeviceGuard guard(unary.device());
@@ -120,6 +146,8 @@ void Backward(const float rho, const at::Tensor context, const at::Tensor edge_w
               const at::Tensor dcost_final, const at::Tensor msg_min_index,
               const at::Tensor msg_norm_index, at::Tensor dunary, at::Tensor dcontext,
               at::Tensor dedge_weights, at::Tensor dmsg, at::Tensor dunary_update) {
+  // (the reference prints this and returns, TRWP.cpp:315-316)
+  TORCH_CHECK(dcost_final.is_cuda(), "Does not support CPU backward.");
   int n_iter = 0;
   const mpl_shape s = shape_of_index(msg_min_index, &n_iter);
   check_backward(s, n_iter, context, edge_weights, dcost_final, msg_min_index, msg_norm_index,
@@ -145,6 +173,16 @@ void Forward(const int enable_sgm, const float rho, const int n_iter, const int 
              at::Tensor msg_norm_index, at::Tensor unary_update, at::Tensor msg_update,
              at::Tensor label_all) {
   const mpl_shape s = shape_of(msg);
+  if (!unary.is_cuda()) {
+    check_forward_cpu(s, n_iter, unary, context, msg, cost_final, label_all);
+    check(msg_update, "msg_update", at::kFloat, s.n_dir * pixels(s) * s.n_disp, false);
+    const int rc = mpl_isgmr_forward_cpu(&s, enable_sgm, rho, n_iter, unary.data_ptr<float>(),
+                                         context.data_ptr<float>(), msg.data_ptr<float>(),
+                                         cost_final.data_ptr<float>(), msg_update.data_ptr<float>(),
+                                         u8_or_null(label_all));
+    TORCH_CHECK(rc == MPL_OK, "ISGMR.forward: ", mpl_last_error());
+    return;
+  }
   check_forward(s, n_iter, unary, context, edge_weights, msg, cost_final, msg_min_index,
                 msg_norm_index, unary_update, label_all);
   check(msg_update, "msg_update", at::kFloat, s.n_dir * pixels(s) * s.n_disp);
@@ -165,6 +203,7 @@ void Backward(const int enable_sgm, const float rho, const at::Tensor context,
               const at::Tensor msg_min_index, const at::Tensor msg_norm_index, at::Tensor dunary,
               at::Tensor dcontext, at::Tensor dedge_weights, at::Tensor dmsg,
               at::Tensor dunary_update, at::Tensor dmsg_update) {
+  TORCH_CHECK(dcost_final.is_cuda(), "Does not support CPU backward.");  // ISGMR.cpp:377-378
   int n_iter = 0;
   const mpl_shape s = shape_of_index(msg_min_index, &n_iter);
   check_backward(s, n_iter, context, edge_weights, dcost_final, msg_min_index, msg_norm_index,

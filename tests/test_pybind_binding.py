@@ -30,19 +30,46 @@ def _load(pkg):
   return ns
 
 
-def test_binding_modules_load_and_refuse_cpu_tensors():
+def test_binding_modules_load_and_take_cpu_tensors_like_the_reference():
+  """CPU tensors run the reference's ForwardCPU semantics through the library's CPU entry points
+  (bit-exact against a fixture of the reference's own compiled CPU code); a CPU backward is
+  refused with the reference's message."""
   import torch
   for pkg in ("lib_stereo", "lib_seg"):
     ops = _load(pkg)
     for mod in (ops.TRWP, ops.ISGMR):
       assert callable(mod.forward) and callable(mod.backward)
+  golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+  e8 = torch.empty(0, dtype=torch.uint8)
+  for name, mod in (("refcpu_trwp_d8_l21.npz", _load("lib_seg").TRWP),
+                    ("refcpu_isgmr_d4_l16.npz", _load("lib_stereo").ISGMR)):
+    z = np.load(os.path.join(golden, name))
+    u = torch.tensor(z["unary"])
+    n_dir, n_iter, rho = int(z["n_dir"]), int(z["n_iter"]), float(z["rho"])
+    msg = torch.zeros((n_dir,) + tuple(u.shape))
+    cost, scratch = torch.zeros_like(u), torch.zeros_like(u)
+    label = torch.zeros((n_iter,) + tuple(u.shape[:-1]), dtype=torch.uint8)
+    if str(z["mode"]) == "TRWP":
+      mod.forward(rho, n_iter, 0, u, torch.tensor(z["context"]), torch.empty(0), msg, cost, e8, e8,
+                  scratch, label)
+    else:
+      mod.forward(0, rho, n_iter, 0, u, torch.tensor(z["context"]), torch.empty(0), msg, cost, e8,
+                  e8, scratch, torch.zeros_like(msg), label)
+    assert np.array_equal(msg.numpy(), z["msg"]) and np.array_equal(cost.numpy(), z["cost_final"])
+    assert np.array_equal(label.numpy(), z["label_all"])
+  ops = _load("lib_stereo")
   L = 4
   u = torch.zeros(1, 1, 2, 2, L)
-  e8 = torch.empty(0, dtype=torch.uint8)
-  with pytest.raises(RuntimeError, match="GPU tensor"):
+  # a 1-D table alone is too short for the CPU path (one table per direction)
+  with pytest.raises(RuntimeError, match="context"):
     ops.TRWP.forward(0.5, 1, 0, u, torch.zeros(L), torch.ones(4, 1, 1, 2, 2),
                      torch.zeros(4, 1, 1, 2, 2, L), torch.zeros_like(u), e8, e8,
                      torch.zeros_like(u), e8)
+  idx = torch.zeros(1, 4, 1, 1, 2, 2, L, dtype=torch.uint8)
+  with pytest.raises(RuntimeError, match="Does not support CPU backward"):
+    ops.TRWP.backward(0.5, torch.zeros(L), torch.ones(4, 1, 1, 2, 2), u, idx, idx[..., 0].contiguous(),
+                      torch.zeros_like(u), torch.zeros(L), torch.zeros(4, 1, 1, 2, 2),
+                      torch.zeros(4, 1, 1, 2, 2, L), torch.zeros_like(u))
   # positional arguments only, in the reference's order: a wrong count is a TypeError
   with pytest.raises(TypeError):
     ops.ISGMR.forward(0.5, 1, 0, u)
