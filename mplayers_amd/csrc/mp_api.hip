@@ -121,7 +121,9 @@ template <int V, int ND>
 __global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ unary,
                                                      const float* __restrict__ msg, int n_dir_rt,
                                                      int64_t N, float* __restrict__ S,
-                                                     int* nonzero_flag) {
+                                                     int* nonzero_flag, const int* only_if = nullptr) {
+  // (only_if: a flag an earlier kernel of the stream has set or left clear; clear: nothing to do)
+  if (only_if != nullptr && *only_if == 0) return;
   const int n_dir = ND > 0 ? ND : n_dir_rt;
   bool any = false;  // some message of this thread's elements is not zero
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
@@ -153,6 +155,35 @@ __global__ void __launch_bounds__(256) belief_kernel(const float* __restrict__ u
   if (nonzero_flag != nullptr && any) *nonzero_flag = 1;  // every writer stores the same value
 }
 
+// Sets *flag when some element of the n_dir message planes is not zero (every writer stores the
+// same value).  The reference's callers pass cleared message tensors; knowing that on the device
+// lets the first sweeps read the unary terms in place of planes that would have to be built first.
+template <int V, int ND>
+__global__ void __launch_bounds__(256) check_nonzero_kernel(const float* __restrict__ msg,
+                                                            int n_dir_rt, int64_t N, int* flag) {
+  const int n_dir = ND > 0 ? ND : n_dir_rt;
+  bool any = false;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
+       i += (int64_t)gridDim.x * blockDim.x * V) {
+    if constexpr (ND > 0) {
+      Pack<V> m[ND];
+#pragma unroll
+      for (int k = 0; k < ND; ++k) m[k] = ld_pack<V>(msg + (int64_t)k * N + i);
+#pragma unroll
+      for (int k = 0; k < ND; ++k)
+#pragma unroll
+        for (int j = 0; j < V; ++j) any = any || (m[k].v[j] != 0.f);
+    } else {
+      for (int k = 0; k < n_dir; ++k) {
+        const Pack<V> m = ld_pack<V>(msg + (int64_t)k * N + i);
+#pragma unroll
+        for (int j = 0; j < V; ++j) any = any || (m.v[j] != 0.f);
+      }
+    }
+  }
+  if (any) *flag = 1;
+}
+
 // ISGMR: every direction of an iteration reads the old messages only through
 //   U_d = rho * (unary + sum_k m_k - m_d) - m_{d^1}      (UpdateUnaryKernel, ISGMR_forward.cu:101-121)
 // so U_d is stored once per iteration (in place of m_d, or into the other message buffer) before
@@ -161,7 +192,8 @@ template <int V, int ND>
 __global__ void __launch_bounds__(256) isgmr_unary_kernel(const float* __restrict__ unary,
                                                           const float* msg, float* out,
                                                           int n_dir_rt, int64_t N, float rho,
-                                                          int pair_share) {
+                                                          int pair_share, const int* only_if = nullptr) {
+  if (only_if != nullptr && *only_if == 0) return;  // (see belief_kernel)
   constexpr int KD = ND > 0 ? ND : kMaxDirs;
   const int n_dir = ND > 0 ? ND : n_dir_rt;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < N;
@@ -838,14 +870,27 @@ int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
   // flag stays 0), and the first sweep of every direction writes the zero of its chain starts.
   const bool uninit = msg_uninit && desc != nullptr;
   if (msg_uninit && !uninit) zero_fill(msg, (int64_t)s->n_dir * N, st);
+  // The reference's contract: `msg` holds the initial messages, which its callers always clear.
+  // With more labels than the packed scans take, the messages are first only looked at (n_dir
+  // planes in, nothing out): when they are all zero the belief plane is not built (the kernel
+  // that builds it finds the flag clear and ends) and the first pair of sweeps does what it does
+  // for messages declared zero, choosing on the device (SweepParams::zero_first).
+  const bool probe_zero = !uninit && desc != nullptr && s->n_disp > kPackedMaxL;
   if (!uninit) {
     Timed timed(MPL_KERNEL_BELIEF, st);
     const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(unary_update);
     int* flag = desc != nullptr ? &const_cast<CtxDesc*>(desc)->msg_nonzero : nullptr;
-    MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update, flag);
+    if (probe_zero) {
+      MPL_EW_LAUNCH(check_nonzero_kernel, v4, s->n_dir, N, st, msg, s->n_dir, N, flag);
+      MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update,
+                    (int*)nullptr, (const int*)flag);
+    } else {
+      MPL_EW_LAUNCH(belief_kernel, v4, s->n_dir, N, st, unary, msg, s->n_dir, N, unary_update, flag);
+    }
   }
 
   SweepParams p = base_fwd_params(s, rho, edge_weights, context, desc);
+  p.belief_zero = unary;
   p.belief_out = unary_update;
   p.msg_in = msg;
   p.msg_out = msg;
@@ -860,6 +905,7 @@ int mpl_trwp_forward(const mpl_shape* s, unsigned flags, float rho, int n_iter,
       p.pair_q = 1;
       p.belief = (uninit && it == 0 && d <= 1) ? unary : unary_update;
       p.zero_start = (uninit && it == 0) ? 1 : 0;
+      p.zero_first = (probe_zero && it == 0 && d <= 1) ? 1 : 0;
       auto skip_s = [&](int dd) {
         return (((it == n_iter - 1) && (dd == s->n_dir - 1)) ||  // cost_final is re-summed
                 (uninit && it == 0 && dd == 0)) ? 1 : 0;
@@ -930,6 +976,13 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
   p.split = choose_split(s, p, opts, train);
   const bool fuse_u = opts.fused_u && s->n_dir == 4 && rho == 1.f && p.pack == 0;
   if (msg_uninit && !unary_as_u) zero_fill(msg, (int64_t)s->n_dir * N, st);
+  // The reference's contract at rho = 1, one chain per wavefront: the initial messages are looked
+  // at first (n_dir planes in, nothing out); when they are all zero, as the reference's callers
+  // pass them, the first iteration's U pass finds the flag clear and ends, and its scans read the
+  // unary terms, chosen on the device (SweepParams::zero_first).
+  const bool probe_zero = !msg_uninit && rho == 1.f && desc != nullptr && s->n_disp > kPackedMaxL &&
+                          p.pack == 0;
+  p.belief_zero = unary;
   float* have = msg;  // the buffer that holds the current messages
   for (int it = 0; it < n_iter; ++it) {
     // Jacobi over directions (ISGMR_forward.cu:506-622): every direction reads the old messages,
@@ -954,8 +1007,15 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
     } else {
       Timed timed(MPL_KERNEL_UNARY_ALL, st);
       const bool v4 = (N % 4 == 0) && aligned16(unary) && aligned16(msg) && aligned16(msg_update);
+      const int* only_if = nullptr;
+      if (probe_zero && it == 0) {
+        int* flag = &const_cast<CtxDesc*>(desc)->msg_nonzero;
+        MPL_EW_LAUNCH(check_nonzero_kernel, v4, s->n_dir, N, st, have, s->n_dir, N, flag);
+        only_if = flag;
+        p.zero_first = 1;
+      }
       MPL_EW_LAUNCH(isgmr_unary_kernel, v4, s->n_dir, N, st, unary, have, ubuf, s->n_dir, N, rho,
-                    p.u_pair_share);
+                    p.u_pair_share, only_if);
       p.msg_in = ubuf;
       p.u_stride = N;
     }
@@ -965,6 +1025,7 @@ int mpl_isgmr_forward(const mpl_shape* s, unsigned flags, int enable_sgm, float 
       p.idx_norm = msg_norm_index + (int64_t)it * s->n_dir * P;
     }
     launch_fwd(p, train, true, st);
+    p.zero_first = 0;
     if (label_all) {
       Timed timed(MPL_KERNEL_LABEL, st);
       launch_labels(unary, nxt, s->n_dir, P, s->n_disp, factor, enable_min_a_dir, label_all + it * P, st);

@@ -484,6 +484,12 @@ struct SweepParams {
                                    // holds the old messages themselves; the scans form U on the fly
   int zero_start;                  // Gauss-Seidel: store zeros at the chain start of msg_out (the
                                    // caller's buffer is undefined and this is its first sweep)
+  int zero_first;                  // first sweeps over messages the device found to be all zero
+                                   // (CtxDesc::msg_nonzero == 0): `belief_zero` stands for the plane the
+                                   // sweep would read (Gauss-Seidel, first pair of directions: the belief
+                                   // plane, which then need not exist; Jacobi, first iteration: U), and
+                                   // the even sweep of that pair stores no plane
+  const float* belief_zero;        // the unary terms
   float* edge_label;               // soft TRWP: (n_dir_total, P, L, L) duals of this iteration, or null
 };
 

@@ -438,9 +438,15 @@ __device__ __forceinline__ void linear_step(const float (&a)[R], float w, float 
 template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI, int KT>
 __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
                                               const ChainCtx& ch, float* a_s, const float* ctx_s,
-                                              const bool skip_s_store, float* xchg = nullptr) {
+                                              const bool skip_s_store_in, float* xchg = nullptr) {
   constexpr bool SPLIT = (KT == -3);
   const int L = p.L;
+  // The caller's initial messages turned out to be all zero (the usual case: the reference's
+  // callers pass a cleared tensor) and this is a sweep that can profit: S = Q = U = unary, so the
+  // unary terms are read in place of the plane, and the even sweep of the first pair has nothing to
+  // store (the odd one reads the unary terms again).  Wave-uniform, the same for every chain.
+  const bool zfirst = JACOBI != 2 && p.zero_first && desc.msg_nonzero == 0;
+  const bool skip_s_store = skip_s_store_in || (!JACOBI && zfirst && (ch.dir & 1) == 0);
   const int64_t HW = (int64_t)p.H * p.W;
   const int64_t P = (int64_t)p.B * HW;
   const int64_t N = P * L;
@@ -456,7 +462,9 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // stores U, five planes in and two out per iteration, is not run)
   const int oth = (dir & ~1) ^ 2;  // the even direction of the other pair
   const float* __restrict__ bS =
-      (JACOBI == 1 ? p.msg_in + (int64_t)(p.u_pair_share ? (dir & ~1) : dir) * p.u_stride : p.belief) + img_e;
+      (zfirst ? p.belief_zero
+              : (JACOBI == 1 ? p.msg_in + (int64_t)(p.u_pair_share ? (dir & ~1) : dir) * p.u_stride
+                             : p.belief)) + img_e;
   const float* __restrict__ bMd = p.msg_in + (int64_t)(JACOBI == 2 ? oth : dir) * N + img_e;
   const float* __restrict__ bMi = p.msg_in + (int64_t)(JACOBI == 2 ? oth + 1 : (dir ^ 1)) * N + img_e;
   float* __restrict__ bMo = p.msg_out + (int64_t)dir * N + img_e;

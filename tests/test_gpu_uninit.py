@@ -101,3 +101,32 @@ def test_module_allocates_without_clearing(gpu):
       lib_stereo.ISGMR.forward(0, rho, n_iter, 0, u, context, e, msg, ref, empty, empty,
                                torch.empty_like(u), torch.empty_like(msg), empty)
     assert torch.equal(cost, ref.permute(0, 1, 4, 2, 3).contiguous()), mode
+
+
+@pytest.mark.parametrize("mode,L,n_dir,n_iter", [("TRWP", 96, 4, 2), ("TRWP", 40, 8, 1), ("ISGMR", 96, 8, 2),
+                                                 ("ISGMR", 40, 8, 3), ("ISGMR", 70, 4, 3), ("ISGMR", 12, 8, 2)])
+def test_given_initial_messages_are_used(gpu, oracle, mode, L, n_dir, n_iter):
+  """Under the reference's contract `msg` holds the initial messages.  The library looks at them
+  on the device and takes its shortcuts only when they are all zero: messages that are not zero
+  (here: the result of an earlier call, and a tensor with a single entry that is not zero) must
+  come out as the oracle continues from them."""
+  rng = np.random.default_rng(L + n_dir)
+  B, H, W = 1, 7, 9
+  rho = 0.5 if mode == "TRWP" else 1.0
+  unary = (rng.random((B, 1, H, W, L)) * 3).astype(np.float32)
+  ctx = (0.3 * np.minimum(np.arange(L), 3)).astype(np.float32)
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  first = oracle.forward(mode, unary, ctx, ew, n_dir, 1, rho)["msg"]
+  single = np.zeros_like(first)
+  single[n_dir - 1, 0, 0, H - 1, W - 1, L - 1] = 0.75  # the last element of the last plane
+  for init in (first, single):
+    ref = oracle.forward(mode, unary, ctx, ew, n_dir, n_iter, rho, msg_init=init, saving_label=True,
+                         want_gaps=True)
+    got = gpu.gpu_forward(mode, unary, ctx, ew, n_dir, n_iter, rho, msg_init=init,
+                          saving_label=True)
+    gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=ref["cost_final"])
+    gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
+    tol = 2e-5 * max(1.0, float(np.abs(ref["cost_final"]).max()))
+    gpu.assert_indices_match_off_ties(got["msg_min_index"], ref["msg_min_index"], ref["gap_min"],
+                                      tol, "msg_min_index")
+    gpu.assert_labels_match_off_ties(got["label_all"], ref["label_all"], ref["gap_label"], tol)
