@@ -29,6 +29,8 @@
 
 #include <algorithm>
 #include <atomic>
+#include <exception>
+#include <stdexcept>
 #include <thread>
 #include <vector>
 
@@ -55,23 +57,29 @@ void parallel_for(int64_t n, int64_t block, const Fn& fn) {
   const int hw = (int)std::thread::hardware_concurrency();
   const int workers = (int)std::min<int64_t>(std::min(n_threads(), hw > 0 ? hw : 1), n_blocks);
   std::atomic<int64_t> next{0};
+  std::atomic<bool> failed{false};
   auto body = [&]() {
-    for (;;) {
-      const int64_t b = next.fetch_add(1, std::memory_order_relaxed);
-      if (b >= n_blocks) return;
-      const int64_t end = std::min(n, (b + 1) * block);
-      for (int64_t i = b * block; i < end; ++i) fn(i);
+    try {
+      for (;;) {
+        const int64_t b = next.fetch_add(1, std::memory_order_relaxed);
+        if (b >= n_blocks) return;
+        const int64_t end = std::min(n, (b + 1) * block);
+        for (int64_t i = b * block; i < end; ++i) fn(i);
+      }
+    } catch (...) {  // (an allocation the host refused: reported by the calling thread)
+      failed.store(true, std::memory_order_relaxed);
     }
   };
-  if (workers <= 1) {
-    body();
-    return;
-  }
   std::vector<std::thread> pool;
-  pool.reserve(workers - 1);
-  for (int t = 1; t < workers; ++t) pool.emplace_back(body);
+  try {
+    if (workers > 1) pool.reserve(workers - 1);
+    for (int t = 1; t < workers; ++t) pool.emplace_back(body);
+  } catch (...) {
+    // fewer threads than asked for: the ones that started, and this one, do all the work
+  }
   body();
   for (auto& th : pool) th.join();
+  if (failed.load(std::memory_order_relaxed)) throw std::runtime_error("a worker thread failed");
 }
 
 // direction table of MPLayers/common.cpp:28-76
@@ -235,15 +243,19 @@ int mpl_trwp_forward_cpu(const mpl_shape* shape, float rho, int n_iter, const fl
   if (!unary || !context || !msg || !cost_final)
     return mpl::fail(MPL_EINVAL, "trwp_forward_cpu: null tensor pointer");
   const int64_t LL = (int64_t)g.L * g.L;
-  for (int it = 0; it < n_iter; ++it) {
-    for (int d = 0; d < g.n_dir; ++d)  // in place, one direction after the other: TRWP.cpp:210-228
-      sweep(g, d, rho, unary, msg, msg + (int64_t)d * g.N, context + d * LL, false);
-    if (label_all != nullptr) {
-      aggregate(g, unary, msg, cost_final);
-      labels(g, cost_final, label_all + (int64_t)it * g.P);
+  try {  // (a thread or an allocation the host refuses must not unwind through the C boundary)
+    for (int it = 0; it < n_iter; ++it) {
+      for (int d = 0; d < g.n_dir; ++d)  // in place, one direction after the other: TRWP.cpp:210-228
+        sweep(g, d, rho, unary, msg, msg + (int64_t)d * g.N, context + d * LL, false);
+      if (label_all != nullptr) {
+        aggregate(g, unary, msg, cost_final);
+        labels(g, cost_final, label_all + (int64_t)it * g.P);
+      }
     }
+    aggregate(g, unary, msg, cost_final);
+  } catch (const std::exception& e) {
+    return mpl::fail(MPL_ELAUNCH, "trwp_forward_cpu: %s", e.what());
   }
-  aggregate(g, unary, msg, cost_final);
   return MPL_OK;
 }
 
@@ -257,26 +269,30 @@ int mpl_isgmr_forward_cpu(const mpl_shape* shape, int enable_sgm, float rho, int
     return mpl::fail(MPL_EINVAL, "isgmr_forward_cpu: null tensor pointer");
   const int64_t LL = (int64_t)g.L * g.L;
   const size_t all = (size_t)g.n_dir * (size_t)g.N * sizeof(float);
-  for (int it = 0; it < n_iter; ++it) {
-    for (int d = 0; d < g.n_dir; ++d)  // every direction from the old messages: ISGMR.cpp:232-251
-      sweep(g, d, rho, unary, msg, msg_update + (int64_t)d * g.N, context + d * LL, enable_sgm != 0);
-    memcpy(msg, msg_update, all);
-    if (enable_sgm) {
-      aggregate(g, nullptr, msg_update, unary);  // the unary terms become the sum of the messages
-      memset(msg, 0, all);
-      if (label_all != nullptr) {
-        memcpy(cost_final, unary, (size_t)g.N * sizeof(float));
+  try {
+    for (int it = 0; it < n_iter; ++it) {
+      for (int d = 0; d < g.n_dir; ++d)  // every direction from the old messages: ISGMR.cpp:232-251
+        sweep(g, d, rho, unary, msg, msg_update + (int64_t)d * g.N, context + d * LL, enable_sgm != 0);
+      memcpy(msg, msg_update, all);
+      if (enable_sgm) {
+        aggregate(g, nullptr, msg_update, unary);  // the unary terms become the sum of the messages
+        memset(msg, 0, all);
+        if (label_all != nullptr) {
+          memcpy(cost_final, unary, (size_t)g.N * sizeof(float));
+          labels(g, cost_final, label_all + (int64_t)it * g.P);
+        }
+      } else if (label_all != nullptr) {
+        aggregate(g, unary, msg_update, cost_final);
         labels(g, cost_final, label_all + (int64_t)it * g.P);
       }
-    } else if (label_all != nullptr) {
-      aggregate(g, unary, msg_update, cost_final);
-      labels(g, cost_final, label_all + (int64_t)it * g.P);
     }
+    if (enable_sgm)
+      memcpy(cost_final, unary, (size_t)g.N * sizeof(float));
+    else
+      aggregate(g, unary, msg_update, cost_final);
+  } catch (const std::exception& e) {
+    return mpl::fail(MPL_ELAUNCH, "isgmr_forward_cpu: %s", e.what());
   }
-  if (enable_sgm)
-    memcpy(cost_final, unary, (size_t)g.N * sizeof(float));
-  else
-    aggregate(g, unary, msg_update, cost_final);
   return MPL_OK;
 }
 

@@ -178,7 +178,7 @@ def test_product_never_touches_the_oracle_or_scratch_files():
   offenders = []
   for dirpath, _, files in os.walk(pkg):
     for name in files:
-      if not name.endswith((".py", ".hip", ".h")):
+      if not name.endswith((".py", ".hip", ".h", ".cpp")):
         continue
       text = open(os.path.join(dirpath, name)).read()
       if re.search(r"^\s*(from|import)\s+oracle\b", text, re.M) or re.search(r"(^|[\"'/\s])_work/", text):
