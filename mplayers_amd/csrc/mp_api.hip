@@ -594,32 +594,40 @@ int decide_pack(const mpl_shape* s, const Params& p, const CallOpts& o) {
 }
 
 // Wavefronts per chain for the forward scan of a launch whose caller declared a dense 1-D table
-// (MPL_F_DENSE_TABLE) with several labels per lane.  Four wavefronts, one on every SIMD of a
-// compute unit, each scanning a quarter of the front labels: the only count that keeps the SIMDs
-// of a unit evenly loaded, which matters because the wavefronts of a chain meet at a barrier every
-// pixel (2, 3, 6 and 8 wavefronts were measured slower than 4 at every size, 6 and 8 slower than
-// one).  A wavefront that shares its SIMD with others hides the wait states of the scan's
-// broadcasts and lane shifts, so the split gains more than the idle SIMDs it fills; it stops
-// paying once one wavefront per chain loads every SIMD evenly.  Measured on 192 labels, forward
-// scan, one wavefront against four (ms per launch): keeping argmin labels, 384 chains 11.6 / 5.8,
-// 768 chains 30.1 / 15.7, 1248 chains 55.3 / 40.2, 1536 chains 34.5 / 29.3, 2496 chains
-// 79.5 / 76.2, 3072 chains 48.3 / 55.7; without them 384 chains 6.6 / 3.9, 1248 chains
-// 34.0 / 29.8, 1536 chains 21.2 / 21.8, 2496 chains 51.3 / 57.2.
+// (MPL_F_DENSE_TABLE) with several labels per lane: four (one on every SIMD of a compute unit, each
+// scanning a quarter of the front labels of a pixel), two, or one.  A lone wavefront on a SIMD
+// reaches some 70 % of what the SIMD issues with three of them, and the wavefronts of a chain meet
+// at a barrier every pixel and repeat what is not the scan (loads, the update of the unary term,
+// normalisation), so the split pays as long as it fills idle SIMDs and stops paying once one
+// wavefront per chain loads every SIMD.  Measured on 192 labels, forward scan, ms per launch with
+// 1 / 2 / 4 / 8 wavefronts per chain; keeping argmin labels: 384 chains 6.9 / 5.6 / 3.6 / 6.7,
+// 768 chains 6.9 / 5.6 / 4.7 / 9.9, 1248 chains 33.3 / 25.1 / 23.8 / 53.4, 1536 chains
+// 10.3 / 7.9 / 8.7 / 19.8, 1920 chains 12.4 / 12.2 / 11.3 / 26.4, 2496 chains
+// 46.2 / 41.6 / 44.4 / 107, 3072 chains 14.4 / 15.0 / 16.4 / 39.6; without them: 384 chains
+// 4.5 / 2.9 / 1.9 / 3.2, 768 chains 4.1 / 2.9 / 3.2 / 4.8, 1248 chains 18.4 / 15.9 / 15.7 / 26.0,
+// 1536 chains 5.9 / 6.0 / 5.6 / 9.6, 1920 chains 5.8 / 6.1 / 7.3 / 12.8, 2496 chains
+// 29.9 / 27.5 / 29.2 / 51.8, 3072 chains 8.9 / 9.2 / 10.7 / 19.2.  In chains per SIMD: four
+// wavefronts up to 1.25 (0.5 without argmin labels), two up to 2.5 (1.5), one beyond.
 template <typename Params>
 int choose_split(const mpl_shape* s, const Params& p, const CallOpts& o, bool train) {
   if (!o.dense_table || s->ctx2d || s->n_disp <= kWave || p.pack >= 2) return 0;
   const int L = s->n_disp, R = labels_per_lane(L);
   const int forced = g_split_waves.load(std::memory_order_relaxed);
-  int w = 4;
+  int w;
   if (forced > 0) {
     w = forced;
   } else {
-    const int64_t chains = p.block_prefix[p.n_dirs];
-    const int n_simd = launch_policy().n_simd;
-    if (2 * chains > (train ? 5 : 3) * (int64_t)n_simd) return 0;  // 2.5 / 1.5 chains per SIMD
+    const int64_t chains4 = 4 * (int64_t)p.block_prefix[p.n_dirs];  // in quarters of a chain
+    const int64_t n_simd = launch_policy().n_simd;
+    if (chains4 <= (train ? 5 : 2) * n_simd)
+      w = 4;
+    else if (chains4 <= (train ? 10 : 6) * n_simd)
+      w = 2;
+    else
+      return 0;
   }
-  // every wavefront needs a share of the front labels (they are visited R at a time)
-  while (w > 1 && (w - 1) * (((L + R * w - 1) / (R * w)) * R) >= L) --w;
+  // every wavefront needs a share of the front labels
+  while (w > 1 && (w - 1) * split_share(L, R, w) >= L) --w;
   return w >= 2 ? w : 0;
 }
 

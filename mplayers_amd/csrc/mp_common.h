@@ -587,8 +587,22 @@ void launch_swm_fwd(const float* msg, int n_trees, int L, float* out, uint8_t* m
 void launch_swm_bwd(const float* dout, const float* msg, const uint8_t* min_ind, int n_trees, int L,
                     float* dmsg, hipStream_t st);
 
+// LDS of the forward scan with several labels per lane: after the 1-D table c[0 .. L-1] (padded to
+// whole groups of four) stands the table moved down by one entry, c1[i] = c[i + 1], which the dense
+// scan reads four entries at a time up to two trips past the last label
+__host__ __device__ inline int dense_c1_offset(int L) { return (L + 3) & ~3; }
+__host__ __device__ inline int dense_c1_floats(int L) { return ((L + 3) & ~3) + 32; }
+
+// Front labels per wavefront where `waves` wavefronts scan a pixel together: whole trips of the
+// dense scan (4 R front labels)
+__host__ __device__ inline int split_share(int L, int R, int waves) {
+  const int trip = 4 * R;
+  return ((L + trip * waves - 1) / (trip * waves)) * trip;
+}
+
 inline size_t fwd_lds_bytes(int L, int ctx2d) {
-  return sizeof(float) * (kMaxL + ((ctx2d || L <= kWave) ? L * L : L));
+  if (ctx2d || L <= kWave) return sizeof(float) * (kMaxL + L * L);
+  return sizeof(float) * (kMaxL + dense_c1_offset(L) + dense_c1_floats(L));
 }
 
 }  // namespace mpl

@@ -61,68 +61,121 @@ __device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&val
   __syncthreads();
 }
 
-// Dense O(L^2) step for 1-D contexts and several labels per lane, without LDS in its loop.  The
-// front labels are visited in ascending order; a[fd] is broadcast with v_readlane, and the context
-// values c[|cd - fd|] of the lane's labels are kept in registers and moved one label up per front
-// label (c[|cd - (fd+1)|] of label cd is c[|(cd-1) - fd|] of label cd - 1; c[fd+1] enters at
-// label 0).  `<=` on the ascending scan keeps the largest front label among equals, as the
-// reference's descending scan with `<` does.
-// The scan covers the front labels fd_lo .. fd_hi - 1 (fd_lo a multiple of R): all of them, or the
-// share of one wavefront where several scan a pixel together (split_combine below).
-template <int R, bool TRAIN, bool WHOLE>  // WHOLE: L is a multiple of R
-__device__ __forceinline__ void dense1d_step(const float (&a)[R], float w, int L, int lab0,
-                                             const float* ctx_s, float (&v)[R], int (&fd_idx)[R],
-                                             const int fd_lo, const int fd_hi) {
-  float c_own[R], cv[R];  // c[label] of the lane's labels; the sliding c[|label - fd|]
+// Dense O(L^2) step for 1-D contexts and several labels per lane.  The front labels are visited
+// in ascending order; the context values c[|cd - fd|] of the lane's labels are kept in registers and
+// moved one label up per front label (c[|cd - (fd+1)|] of label cd is c[|(cd-1) - fd|] of label
+// cd - 1; c[fd+1] enters at label 0) with one lane shift.  Both a[fd] and the entering c[fd+1] are
+// the same for every lane: they are read from LDS, every lane from the same address (a_w: this
+// wavefront's own copy of a[], written at the start of the step; c1_s: the table moved down by one
+// entry, c1_s[i] = c[i+1]), four front labels per read, one trip of T = 4 R front labels ahead of
+// their use, so the loop waits for none of them.  The shift writes into the register the read
+// filled (lane 0 has no source lane and keeps c[fd+1]): no instruction sets up a fill.
+// Two front labels are folded per minimum (v_min3); the argmin label of a lane is kept relative to
+// the trip's first front label, so that the select takes a literal and no register has to carry fd
+// (`<=` on the ascending scan keeps the largest front label among equals, as the reference's
+// descending scan with `<` does; for the second label of a pair, `<=` against the minimum of all
+// three is the same comparison, as that minimum cannot lie above it).
+// The scan covers the front labels fd_lo .. fd_hi - 1 (fd_lo a multiple of T): all of them, or the
+// share of one wavefront where several scan a pixel together (split_combine below).  cv0: the
+// sliding values at fd_lo, c[|cd - fd_lo|].
+template <int R>
+constexpr int dense_trip() { return 4 * R; }
+
+template <int R, bool TRAIN>
+__device__ __forceinline__ void dense1d_step(const float (&a)[R], const float w, const int lab0,
+                                             float* a_w, const float* c1_s, const float (&cv0)[R],
+                                             float (&v)[R], int (&fd_idx)[R], const int fd_lo,
+                                             const int fd_hi) {
+  constexpr int T = dense_trip<R>();
+  float cv[R];
+  int rel[R];
 #pragma unroll
   for (int j = 0; j < R; ++j) {
-    const int l = lab0 + j < L ? lab0 + j : L - 1;
-    c_own[j] = ctx_s[l];
-    cv[j] = fd_lo == 0 ? c_own[j] : ctx_s[l > fd_lo ? l - fd_lo : fd_lo - l];
+    a_w[lab0 + j] = a[j];
+    cv[j] = cv0[j];
     v[j] = INFINITY;
-    fd_idx[j] = L - 1;
+    rel[j] = 0;
   }
-  // the weight in a vector register: a multiply-add takes one scalar operand, and that is a[fd]
-  float wv = w;
-  asm volatile("" : "+v"(wv));
-  // one front label: fd = fd0 + u is owned by lane src = fd0 / R, register u
-  auto visit = [&](const int fd, const int u, const int src) __attribute__((always_inline)) {
-    const float af = readlane_f(a[u], src);
-    // c[fd + 1]: the next label's own entry (past the last label the value is never used)
-    const float cn = u + 1 < R ? readlane_f(c_own[u + 1 < R ? u + 1 : 0], src)
-                               : readlane_f(c_own[0], (src + 1) & 63);
-#pragma unroll
-    for (int j = 0; j < R; ++j) {
-      const float val = fmaf(wv, cv[j], af);
-      if (TRAIN) {
-        // (the minimum and the comparison are independent instructions; a select of the value
-        // would wait for the comparison's lane mask like the select of the label does)
-        const bool take = val <= v[j];
-        v[j] = fminf(v[j], val);
-        fd_idx[j] = take ? fd : fd_idx[j];
-      } else {
-        v[j] = fminf(v[j], val);
-      }
-    }
-    const float in0 = wave_shr1(cv[R - 1], cn);
+  auto shift = [&](const float fill) __attribute__((always_inline)) {
+    const float in0 = wave_shr1(cv[R - 1], fill);
 #pragma unroll
     for (int j = R - 1; j > 0; --j) cv[j] = cv[j - 1];
     cv[0] = in0;
   };
-  // Two rounds of R front labels per trip: after R one-label shifts the sliding values sit in
-  // registers the shifts created, after 2 R they can be back in the ones the trip started with,
-  // so the loop carries no register moves.
+  float ba[T], bc[T];  // a[fd0 + u], c[fd0 + u + 1]
+  auto read4 = [&](const float* src, float (&dst)[T], const int q) __attribute__((always_inline)) {
+    const f32x4 x = *reinterpret_cast<const f32x4*>(src + 4 * q);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dst[4 * q + i] = x[i];
+  };
+  // The register a read of c fills becomes a sliding value and stays one for R shifts: the four of
+  // group q are free again after shift 4 q + 3 + R of a trip, and that is where the group's next
+  // read stands -- in the same trip for the trip after it (kNext groups), or, for the last groups,
+  // at the start of the trip that uses them.
+  constexpr int kNext = (T - 3 - R + 3) / 4;  // groups q with 4 q + 3 + R < T
   int fd0 = fd_lo;
-  int src0 = fd_lo / R;  // the lane that owns front label fd0 (counted along: no division per trip)
-  for (; fd0 + 2 * R <= fd_hi; fd0 += 2 * R, src0 += 2) {
 #pragma unroll
-    for (int u = 0; u < 2 * R; ++u) visit(fd0 + u, u % R, src0 + u / R);
-  }
-  for (; fd0 < fd_hi; fd0 += R, ++src0) {
+  for (int q = 0; q < R; ++q) read4(a_w + fd0, ba, q);
 #pragma unroll
-    for (int u = 0; u < R; ++u)
-      if (WHOLE || fd0 + u < fd_hi) visit(fd0 + u, u, src0);  // wave-uniform
+  for (int q = 0; q < kNext; ++q) read4(c1_s + fd0, bc, q);
+  for (; fd0 + T <= fd_hi; fd0 += T) {
+    if (TRAIN) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) rel[j] -= T;
+    }
+#pragma unroll
+    for (int u = 0; u < T; u += 2) {
+      float v0[R], v1[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) v0[j] = fmaf(w, cv[j], ba[u]);
+      shift(bc[u]);
+#pragma unroll
+      for (int j = 0; j < R; ++j) v1[j] = fmaf(w, cv[j], ba[u + 1]);
+      shift(bc[u + 1]);
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        const float old = v[j];
+        v[j] = fminf(fminf(old, v0[j]), v1[j]);
+        if (TRAIN) {
+          rel[j] = v0[j] <= old ? u : rel[j];
+          rel[j] = v1[j] <= v[j] ? u + 1 : rel[j];
+        }
+      }
+      // reads that stand after the shifts u and u + 1
+#pragma unroll
+      for (int s = u; s < u + 2; ++s) {
+        if ((s & 3) == 3) read4(a_w + fd0 + T, ba, s / 4);  // a: free once its four labels are done
+        if (s >= 3 + R && ((s - 3 - R) & 3) == 0) read4(c1_s + fd0 + T, bc, (s - 3 - R) / 4);
+        if (s + T >= 3 + R && s + T - 3 - R < T && ((s + T - 3 - R) & 3) == 0 &&
+            (s + T - 3 - R) / 4 >= kNext)
+          read4(c1_s + fd0, bc, (s + T - 3 - R) / 4);
+      }
+    }
   }
+  // what is left of the share: fewer than T front labels, one at a time
+  if (fd0 < fd_hi) {
+#pragma unroll
+    for (int q = kNext; q < R; ++q) read4(c1_s + fd0, bc, q);
+    if (TRAIN) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) rel[j] -= T;
+    }
+#pragma unroll
+    for (int u = 0; u < T - 1; ++u) {
+      if (fd0 + u < fd_hi) {  // wave-uniform
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          const float val = fmaf(w, cv[j], ba[u]);
+          if (TRAIN) rel[j] = val <= v[j] ? u : rel[j];
+          v[j] = fminf(v[j], val);
+        }
+        shift(bc[u]);
+      }
+    }
+    fd0 += T;
+  }
+#pragma unroll
+  for (int j = 0; j < R; ++j) fd_idx[j] = rel[j] + (fd0 - T);
 }
 
 // Several wavefronts on one chain (launches with far fewer chains than the chip has SIMDs, dense
@@ -484,13 +537,28 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   const int wave = SPLIT ? uniform_i((int)(threadIdx.x / kWave)) : 0;
   const int n_waves = SPLIT ? (int)(blockDim.x / kWave) : 1;
   const bool store_ok = !SPLIT || wave == 0;
-  // front labels per wavefront: a multiple of R (the scan visits them R at a time)
+  // front labels per wavefront: whole trips of the dense scan
   // (the division by the number of wavefronts runs on the vector unit: without the explicit
-  // read-back the bounds, and with them the loop counter of the scan and every lane index it
-  // forms, would stay in vector registers)
-  const int fd_chunk = SPLIT ? uniform_i(((L + R * n_waves - 1) / (R * n_waves)) * R) : L;
+  // read-back the bounds, and with them the loop counter of the scan and every address it forms,
+  // would stay in vector registers)
+  const int fd_chunk = SPLIT ? uniform_i(split_share(L, R, n_waves)) : L;
   const int fd_lo = SPLIT ? uniform_i(min(wave * fd_chunk, L)) : 0;
   const int fd_hi = SPLIT ? uniform_i(min(fd_lo + fd_chunk, L)) : L;
+  // dense scan, several labels per lane: this wavefront's copy of a[], the table moved down by one
+  // entry, and the sliding table values of the lane's labels at the first front label
+  float* a_w = a_s + (SPLIT ? wave * kMaxL : 0);
+  const float* c1_s = ctx_s + dense_c1_offset(L);
+  // (only where the dense scan is the kernel's step: a kernel compiled for a band or a
+  // truncated-linear table meets it at pixels with a negative edge weight and takes dense_step)
+  constexpr bool kDenseMain = R > 1 && (KT == -1 || KT == -3);
+  float cv0_chain[R];
+  if constexpr (kDenseMain) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int l = lab0 + j < L ? lab0 + j : L - 1;
+      cv0_chain[j] = ctx_s[l > fd_lo ? l - fd_lo : fd_lo - l];
+    }
+  }
 
   bool valid[R];
 #pragma unroll
@@ -722,7 +790,13 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         }
       } else if (live) {
         if constexpr (R > 1) {  // (2-D tables exist for one label per lane only)
-          dense1d_step<R, TRAIN, VEC>(a, w, L, lab0, ctx_s, v, fd_idx, fd_lo, fd_hi);
+          if constexpr (kDenseMain) {
+            dense1d_step<R, TRAIN>(a, w, lab0, a_w, c1_s, cv0_chain, v, fd_idx, fd_lo, fd_hi);
+          } else {
+            // a pixel with a negative edge weight in a kernel compiled for a band or a
+            // truncated-linear table: the same candidates, one table entry per pair from LDS
+            dense_step<R, TRAIN>(a, valid, w, L, 0, lab0, a_s, ctx_s, v, fd_idx);
+          }
           if constexpr (SPLIT) split_combine<R, TRAIN>(xchg, n_waves, wave, lane, t & 1, v, fd_idx);
         } else {
           dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
@@ -796,9 +870,9 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
 
 template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI>
 __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
-  extern __shared__ float smem[];
+  extern __shared__ __align__(16) float smem[];
   float* a_s = smem;            // kMaxL floats
-  float* ctx_s = smem + kMaxL;  // L or L*L floats
+  float* ctx_s = smem + kMaxL;  // L or L*L floats; several labels per lane: + the table moved down by one
   const int lane = threadIdx.x;
   const int L = p.L;
   const ChainCtx ch = locate_chain(p);
@@ -826,6 +900,10 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
   } else {
     const int n_ctx = p.ctx2d ? L * L : L;
     for (int i = lane; i < n_ctx; i += kWave) ctx_s[i] = p.ctx[i];
+    if (R > 1 && desc.band_k == 0) {  // (the dense scan is this kernel's step)
+      float* c1_s = ctx_s + dense_c1_offset(L);
+      for (int i = lane; i < dense_c1_floats(L); i += kWave) c1_s[i] = i + 1 < L ? p.ctx[i + 1] : 0.f;
+    }
   }
   __syncthreads();
 
@@ -888,11 +966,12 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
 constexpr int kSplitMaxWaves = 8;
 template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI>
 __global__ void __launch_bounds__(kSplitMaxWaves * kWave) sweep_fwd_split_kernel(const SweepParams p) {
-  extern __shared__ float smem[];
-  float* a_s = smem;            // kMaxL floats (unused by this scan)
-  float* ctx_s = smem + kMaxL;  // L floats
-  float* xchg = ctx_s + ((p.L + 3) & ~3);
+  extern __shared__ __align__(16) float smem[];
   const int L = p.L;
+  float* a_s = smem;  // kMaxL floats per wavefront
+  float* ctx_s = smem + (blockDim.x / kWave) * kMaxL;  // L floats, and the table moved down by one
+  float* c1_s = ctx_s + dense_c1_offset(L);
+  float* xchg = c1_s + dense_c1_floats(L);
   const ChainCtx ch = locate_chain(p);
   if (!JACOBI && !p.pair_q && ch.n < 2) return;  // nothing to write (the same for every wavefront)
   CtxDesc desc;
@@ -903,6 +982,7 @@ __global__ void __launch_bounds__(kSplitMaxWaves * kWave) sweep_fwd_split_kernel
   desc.linear = 0;
   desc.slope = 0.f;
   for (int i = threadIdx.x; i < L; i += blockDim.x) ctx_s[i] = p.ctx[i];
+  for (int i = threadIdx.x; i < dense_c1_floats(L); i += blockDim.x) c1_s[i] = i + 1 < L ? p.ctx[i + 1] : 0.f;
   __syncthreads();
   const int halves = (!JACOBI && p.fused_pair) ? 2 : 1;
 #pragma clang loop unroll(disable)
@@ -922,7 +1002,8 @@ __global__ void __launch_bounds__(kSplitMaxWaves * kWave) sweep_fwd_split_kernel
 }
 
 inline size_t split_lds_bytes(int L, int R, int waves, bool train) {
-  return sizeof(float) * (kMaxL + ((L + 3) & ~3) + (size_t)2 * waves * kWave * (train ? 2 * R : R));
+  return sizeof(float) * ((size_t)waves * kMaxL + dense_c1_offset(L) + dense_c1_floats(L) +
+                          (size_t)2 * waves * kWave * (train ? 2 * R : R));
 }
 
 template <int R, bool VEC, bool MASK>
