@@ -178,6 +178,69 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], const float w,
   for (int j = 0; j < R; ++j) fd_idx[j] = rel[j] + (fd0 - T);
 }
 
+// The same scan with both broadcasts taken from the lanes that hold the values (v_readlane of a[]
+// and of the lane's own table entries c[label]) instead of LDS: no staging, no reads in flight, and
+// little state outside the step.  Two more issue slots per front label than dense1d_step; it is the
+// step that a kernel compiled for a band or a truncated-linear table takes at a pixel with a
+// negative edge weight, where the band and the label scans do not hold.
+// `<=` on the ascending scan keeps the largest front label among equals, as the reference's
+// descending scan with `<` does.  fd_lo a multiple of R.
+template <int R, bool TRAIN, bool WHOLE>  // WHOLE: L is a multiple of R
+__device__ __forceinline__ void dense1d_step_lanes(const float (&a)[R], float w, int L, int lab0,
+                                             const float* ctx_s, float (&v)[R], int (&fd_idx)[R],
+                                             const int fd_lo, const int fd_hi) {
+  float c_own[R], cv[R];  // c[label] of the lane's labels; the sliding c[|label - fd|]
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int l = lab0 + j < L ? lab0 + j : L - 1;
+    c_own[j] = ctx_s[l];
+    cv[j] = fd_lo == 0 ? c_own[j] : ctx_s[l > fd_lo ? l - fd_lo : fd_lo - l];
+    v[j] = INFINITY;
+    fd_idx[j] = L - 1;
+  }
+  // the weight in a vector register: a multiply-add takes one scalar operand, and that is a[fd]
+  float wv = w;
+  asm volatile("" : "+v"(wv));
+  // one front label: fd = fd0 + u is owned by lane src = fd0 / R, register u
+  auto visit = [&](const int fd, const int u, const int src) __attribute__((always_inline)) {
+    const float af = readlane_f(a[u], src);
+    // c[fd + 1]: the next label's own entry (past the last label the value is never used)
+    const float cn = u + 1 < R ? readlane_f(c_own[u + 1 < R ? u + 1 : 0], src)
+                               : readlane_f(c_own[0], (src + 1) & 63);
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const float val = fmaf(wv, cv[j], af);
+      if (TRAIN) {
+        // (the minimum and the comparison are independent instructions; a select of the value
+        // would wait for the comparison's lane mask like the select of the label does)
+        const bool take = val <= v[j];
+        v[j] = fminf(v[j], val);
+        fd_idx[j] = take ? fd : fd_idx[j];
+      } else {
+        v[j] = fminf(v[j], val);
+      }
+    }
+    const float in0 = wave_shr1(cv[R - 1], cn);
+#pragma unroll
+    for (int j = R - 1; j > 0; --j) cv[j] = cv[j - 1];
+    cv[0] = in0;
+  };
+  // Two rounds of R front labels per trip: after R one-label shifts the sliding values sit in
+  // registers the shifts created, after 2 R they can be back in the ones the trip started with,
+  // so the loop carries no register moves.
+  int fd0 = fd_lo;
+  int src0 = fd_lo / R;  // the lane that owns front label fd0 (counted along: no division per trip)
+  for (; fd0 + 2 * R <= fd_hi; fd0 += 2 * R, src0 += 2) {
+#pragma unroll
+    for (int u = 0; u < 2 * R; ++u) visit(fd0 + u, u % R, src0 + u / R);
+  }
+  for (; fd0 < fd_hi; fd0 += R, ++src0) {
+#pragma unroll
+    for (int u = 0; u < R; ++u)
+      if (WHOLE || fd0 + u < fd_hi) visit(fd0 + u, u, src0);  // wave-uniform
+  }
+}
+
 // Several wavefronts on one chain (launches with far fewer chains than the chip has SIMDs, dense
 // table): every wavefront of the workgroup walks the chain and holds the same state, but scans only
 // its share of the front labels of a pixel; the partial minima (and their labels) meet in LDS,
@@ -549,7 +612,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   float* a_w = a_s + (SPLIT ? wave * kMaxL : 0);
   const float* c1_s = ctx_s + dense_c1_offset(L);
   // (only where the dense scan is the kernel's step: a kernel compiled for a band or a
-  // truncated-linear table meets it at pixels with a negative edge weight and takes dense_step)
+  // truncated-linear table meets it at pixels with a negative edge weight and takes
+  // dense1d_step_lanes)
   constexpr bool kDenseMain = R > 1 && (KT == -1 || KT == -3);
   float cv0_chain[R];
   if constexpr (kDenseMain) {
@@ -794,8 +858,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
             dense1d_step<R, TRAIN>(a, w, lab0, a_w, c1_s, cv0_chain, v, fd_idx, fd_lo, fd_hi);
           } else {
             // a pixel with a negative edge weight in a kernel compiled for a band or a
-            // truncated-linear table: the same candidates, one table entry per pair from LDS
-            dense_step<R, TRAIN>(a, valid, w, L, 0, lab0, a_s, ctx_s, v, fd_idx);
+            // truncated-linear table: the same candidates, broadcast from the lanes
+            dense1d_step_lanes<R, TRAIN, VEC>(a, w, L, lab0, ctx_s, v, fd_idx, 0, L);
           }
           if constexpr (SPLIT) split_combine<R, TRAIN>(xchg, n_waves, wave, lane, t & 1, v, fd_idx);
         } else {
