@@ -598,16 +598,16 @@ int decide_pack(const mpl_shape* s, const Params& p, const CallOpts& o) {
 // scanning a quarter of the front labels of a pixel), two, or one.  A lone wavefront on a SIMD
 // reaches some 70 % of what the SIMD issues with three of them, and the wavefronts of a chain meet
 // at a barrier every pixel and repeat what is not the scan (loads, the update of the unary term,
-// normalisation), so the split pays as long as it fills idle SIMDs and stops paying once one
-// wavefront per chain loads every SIMD.  Measured on 192 labels, forward scan, ms per launch with
-// 1 / 2 / 4 / 8 wavefronts per chain; keeping argmin labels: 384 chains 6.9 / 5.6 / 3.6 / 6.7,
-// 768 chains 6.9 / 5.6 / 4.7 / 9.9, 1248 chains 33.3 / 25.1 / 23.8 / 53.4, 1536 chains
-// 10.3 / 7.9 / 8.7 / 19.8, 1920 chains 12.4 / 12.2 / 11.3 / 26.4, 2496 chains
-// 46.2 / 41.6 / 44.4 / 107, 3072 chains 14.4 / 15.0 / 16.4 / 39.6; without them: 384 chains
-// 4.5 / 2.9 / 1.9 / 3.2, 768 chains 4.1 / 2.9 / 3.2 / 4.8, 1248 chains 18.4 / 15.9 / 15.7 / 26.0,
+// normalisation; the first one also finds the argmin labels), so the split pays as long as it fills
+// idle SIMDs and stops paying once one wavefront per chain loads every SIMD.  Measured on 192
+// labels, forward scan, ms per launch with 1 / 2 / 4 / 8 wavefronts per chain; keeping argmin
+// labels: 384 chains 5.6 / 4.4 / 3.3 / 6.4, 768 chains 5.4 / 4.5 / 3.8 / 9.4, 1248 chains
+// 22.7 / 18.5 / 21.3 / 50.8, 1536 chains 7.3 / 5.9 / 7.4 / 18.9, 1920 chains 8.6 / 9.6 / 10.0 / 25.1,
+// 2496 chains 32.3 / 30.9 / 40.1 / 102, 3072 chains 10.2 / 12.4 / 14.3 / 37.8; without them: 384
+// chains 4.5 / 2.9 / 1.9 / 3.2, 768 chains 4.1 / 2.9 / 3.2 / 4.8, 1248 chains 18.4 / 15.9 / 15.7 / 26.0,
 // 1536 chains 5.9 / 6.0 / 5.6 / 9.6, 1920 chains 5.8 / 6.1 / 7.3 / 12.8, 2496 chains
 // 29.9 / 27.5 / 29.2 / 51.8, 3072 chains 8.9 / 9.2 / 10.7 / 19.2.  In chains per SIMD: four
-// wavefronts up to 1.25 (0.5 without argmin labels), two up to 2.5 (1.5), one beyond.
+// wavefronts up to 1 (0.5 without argmin labels), two up to 1.5, one beyond.
 template <typename Params>
 int choose_split(const mpl_shape* s, const Params& p, const CallOpts& o, bool train) {
   if (!o.dense_table || s->ctx2d || s->n_disp <= kWave || p.pack >= 2) return 0;
@@ -619,9 +619,9 @@ int choose_split(const mpl_shape* s, const Params& p, const CallOpts& o, bool tr
   } else {
     const int64_t chains4 = 4 * (int64_t)p.block_prefix[p.n_dirs];  // in quarters of a chain
     const int64_t n_simd = launch_policy().n_simd;
-    if (chains4 <= (train ? 5 : 2) * n_simd)
+    if (chains4 <= (train ? 4 : 2) * n_simd)
       w = 4;
-    else if (chains4 <= (train ? 10 : 6) * n_simd)
+    else if (chains4 <= 6 * n_simd)
       w = 2;
     else
       return 0;

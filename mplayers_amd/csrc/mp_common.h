@@ -600,9 +600,14 @@ __host__ __device__ inline int split_share(int L, int R, int waves) {
   return ((L + trip * waves - 1) / (trip * waves)) * trip;
 }
 
+// ... and, for the argmin labels of the dense scan, the table around its centre: entries for every
+// difference of two labels that R * 64 lanes of labels can form
+__host__ __device__ inline int dense_sym_floats(int R) { return 2 * R * kWave; }
+
 inline size_t fwd_lds_bytes(int L, int ctx2d) {
   if (ctx2d || L <= kWave) return sizeof(float) * (kMaxL + L * L);
-  return sizeof(float) * (kMaxL + dense_c1_offset(L) + dense_c1_floats(L));
+  const int R = (L + kWave - 1) / kWave;
+  return sizeof(float) * (kMaxL + dense_c1_offset(L) + dense_c1_floats(L) + dense_sym_floats(R));
 }
 
 }  // namespace mpl

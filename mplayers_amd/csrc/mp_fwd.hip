@@ -70,11 +70,14 @@ __device__ __forceinline__ void dense_step(const float (&a)[R], const bool (&val
 // entry, c1_s[i] = c[i+1]), four front labels per read, one trip of T = 4 R front labels ahead of
 // their use, so the loop waits for none of them.  The shift writes into the register the read
 // filled (lane 0 has no source lane and keeps c[fd+1]): no instruction sets up a fill.
-// Two front labels are folded per minimum (v_min3); the argmin label of a lane is kept relative to
-// the trip's first front label, so that the select takes a literal and no register has to carry fd
-// (`<=` on the ascending scan keeps the largest front label among equals, as the reference's
-// descending scan with `<` does; for the second label of a pair, `<=` against the minimum of all
-// three is the same comparison, as that minimum cannot lie above it).
+// Two front labels are folded per minimum (v_min3).
+// TRAIN: the argmin label is found in two steps.  The scan only notes, per label, the trip whose
+// candidates last reached the running minimum (the minimum over a trip's candidates against the
+// minimum so far, `<=`: one comparison and one select per trip instead of one per front label), and
+// returns that trip's first front label in `trip0`; dense1d_argmin then evaluates the T candidates
+// of that one trip again.  The argmin the reference keeps is the largest front label whose candidate
+// equals the final minimum (its descending scan with `<`): it lies in the last trip that holds such
+// a candidate, and that is the last trip whose own minimum is <= the minimum before it.
 // The scan covers the front labels fd_lo .. fd_hi - 1 (fd_lo a multiple of T): all of them, or the
 // share of one wavefront where several scan a pixel together (split_combine below).  cv0: the
 // sliding values at fd_lo, c[|cd - fd_lo|].
@@ -84,11 +87,11 @@ constexpr int dense_trip() { return 4 * R; }
 template <int R, bool TRAIN>
 __device__ __forceinline__ void dense1d_step(const float (&a)[R], const float w, const int lab0,
                                              float* a_w, const float* c1_s, const float (&cv0)[R],
-                                             float (&v)[R], int (&fd_idx)[R], const int fd_lo,
+                                             float (&v)[R], int (&trip0)[R], const int fd_lo,
                                              const int fd_hi) {
   constexpr int T = dense_trip<R>();
   float cv[R];
-  int rel[R];
+  int rel[R];  // the noted trip, counted back from the current one (0, -1, ...)
 #pragma unroll
   for (int j = 0; j < R; ++j) {
     a_w[lab0 + j] = a[j];
@@ -101,6 +104,15 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], const float w,
 #pragma unroll
     for (int j = R - 1; j > 0; --j) cv[j] = cv[j - 1];
     cv[0] = in0;
+  };
+  // the end of a trip: fold its minimum into the running one and note the trip where it reaches it
+  auto close_trip = [&](const float (&lm)[R]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const bool take = lm[j] <= v[j];
+      v[j] = fminf(v[j], lm[j]);
+      rel[j] = take ? 0 : rel[j] - 1;
+    }
   };
   float ba[T], bc[T];  // a[fd0 + u], c[fd0 + u + 1]
   auto read4 = [&](const float* src, float (&dst)[T], const int q) __attribute__((always_inline)) {
@@ -119,10 +131,7 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], const float w,
 #pragma unroll
   for (int q = 0; q < kNext; ++q) read4(c1_s + fd0, bc, q);
   for (; fd0 + T <= fd_hi; fd0 += T) {
-    if (TRAIN) {
-#pragma unroll
-      for (int j = 0; j < R; ++j) rel[j] -= T;
-    }
+    float lm[R];  // TRAIN: the minimum over this trip's candidates
 #pragma unroll
     for (int u = 0; u < T; u += 2) {
       float v0[R], v1[R];
@@ -134,12 +143,10 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], const float w,
       shift(bc[u + 1]);
 #pragma unroll
       for (int j = 0; j < R; ++j) {
-        const float old = v[j];
-        v[j] = fminf(fminf(old, v0[j]), v1[j]);
-        if (TRAIN) {
-          rel[j] = v0[j] <= old ? u : rel[j];
-          rel[j] = v1[j] <= v[j] ? u + 1 : rel[j];
-        }
+        if (TRAIN)
+          lm[j] = u == 0 ? fminf(v0[j], v1[j]) : fminf(fminf(lm[j], v0[j]), v1[j]);
+        else
+          v[j] = fminf(fminf(v[j], v0[j]), v1[j]);
       }
       // reads that stand after the shifts u and u + 1
 #pragma unroll
@@ -151,31 +158,81 @@ __device__ __forceinline__ void dense1d_step(const float (&a)[R], const float w,
           read4(c1_s + fd0, bc, (s + T - 3 - R) / 4);
       }
     }
+    if (TRAIN) close_trip(lm);
   }
   // what is left of the share: fewer than T front labels, one at a time
   if (fd0 < fd_hi) {
 #pragma unroll
     for (int q = kNext; q < R; ++q) read4(c1_s + fd0, bc, q);
-    if (TRAIN) {
+    float lm[R];
 #pragma unroll
-      for (int j = 0; j < R; ++j) rel[j] -= T;
-    }
+    for (int j = 0; j < R; ++j) lm[j] = INFINITY;
 #pragma unroll
     for (int u = 0; u < T - 1; ++u) {
       if (fd0 + u < fd_hi) {  // wave-uniform
 #pragma unroll
         for (int j = 0; j < R; ++j) {
           const float val = fmaf(w, cv[j], ba[u]);
-          if (TRAIN) rel[j] = val <= v[j] ? u : rel[j];
-          v[j] = fminf(v[j], val);
+          if (TRAIN)
+            lm[j] = fminf(lm[j], val);
+          else
+            v[j] = fminf(v[j], val);
         }
         shift(bc[u]);
       }
     }
+    if (TRAIN) close_trip(lm);
     fd0 += T;
   }
 #pragma unroll
-  for (int j = 0; j < R; ++j) fd_idx[j] = rel[j] + (fd0 - T);
+  for (int j = 0; j < R; ++j) trip0[j] = (fd0 - T) + rel[j] * T;
+}
+
+// The argmin labels of dense1d_step: for every label of the lane, the largest front label of the
+// trip starting at trip0 whose candidate a[fd] + w * c[|cd - fd|] equals the minimum v (the same
+// multiply-add on the same operands as in the scan: the same bits).  a_w: the wavefront's copy of
+// a[] (front labels past the last one read as +inf or as whatever lies there: their candidates
+// are not the minimum); csym_s: the table laid out around its centre, csym_s[dense_sym_centre<R>() + d]
+// = c[|d|], so that a lane reads the entries of consecutive front labels at consecutive addresses.
+template <int R>
+constexpr int dense_sym_centre() { return R * kWave; }  // |cd - fd| < R * 64
+
+template <int R>
+__device__ __forceinline__ void fill_dense_sym(float* csym_s, const float* ctx, int L, int tid,
+                                               int n_threads) {
+  for (int i = tid; i < dense_sym_floats(R); i += n_threads) {
+    const int d = i < dense_sym_centre<R>() ? dense_sym_centre<R>() - i : i - dense_sym_centre<R>();
+    csym_s[i] = d < L ? ctx[d] : 0.f;
+  }
+}
+
+template <int R>
+__device__ __forceinline__ void dense1d_argmin(const float (&v)[R], const int (&trip0)[R],
+                                               const float w, const int lab0, const int L,
+                                               const float* a_w, const float* csym_s,
+                                               int (&fd_idx)[R]) {
+  constexpr int T = dense_trip<R>();
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int t0 = trip0[j];
+    const int l = lab0 + j < L ? lab0 + j : L - 1;
+    float af[T];
+#pragma unroll
+    for (int q = 0; q < T / 4; ++q) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(a_w + t0 + 4 * q);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) af[4 * q + i] = x[i];
+    }
+    const float* cp = csym_s + (dense_sym_centre<R>() + l - t0 - (T - 1));  // entry of front label t0 + T - 1
+    int arg = 0;
+#pragma unroll
+    for (int u = 0; u < T; ++u) {
+      const float val = fmaf(w, cp[T - 1 - u], af[u]);
+      arg = val == v[j] ? u : arg;
+    }
+    const int fd = t0 + arg;
+    fd_idx[j] = fd < L ? fd : L - 1;  // (only where no candidate is finite)
+  }
 }
 
 // The same scan with both broadcasts taken from the lanes that hold the values (v_readlane of a[]
@@ -611,6 +668,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // entry, and the sliding table values of the lane's labels at the first front label
   float* a_w = a_s + (SPLIT ? wave * kMaxL : 0);
   const float* c1_s = ctx_s + dense_c1_offset(L);
+  const float* csym_s = c1_s + dense_c1_floats(L);  // the table around its centre (dense1d_argmin)
   // (only where the dense scan is the kernel's step: a kernel compiled for a band or a
   // truncated-linear table meets it at pixels with a negative edge weight and takes
   // dense1d_step_lanes)
@@ -856,12 +914,15 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         if constexpr (R > 1) {  // (2-D tables exist for one label per lane only)
           if constexpr (kDenseMain) {
             dense1d_step<R, TRAIN>(a, w, lab0, a_w, c1_s, cv0_chain, v, fd_idx, fd_lo, fd_hi);
+            if constexpr (SPLIT) split_combine<R, TRAIN>(xchg, n_waves, wave, lane, t & 1, v, fd_idx);
+            // (fd_idx holds the first front label of the trip with the argmin; only a wavefront
+            // that stores needs the label itself)
+            if (TRAIN && store_ok) dense1d_argmin<R>(v, fd_idx, w, lab0, L, a_w, csym_s, fd_idx);
           } else {
             // a pixel with a negative edge weight in a kernel compiled for a band or a
             // truncated-linear table: the same candidates, broadcast from the lanes
             dense1d_step_lanes<R, TRAIN, VEC>(a, w, L, lab0, ctx_s, v, fd_idx, 0, L);
           }
-          if constexpr (SPLIT) split_combine<R, TRAIN>(xchg, n_waves, wave, lane, t & 1, v, fd_idx);
         } else {
           dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
         }
@@ -967,6 +1028,7 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
     if (R > 1 && desc.band_k == 0) {  // (the dense scan is this kernel's step)
       float* c1_s = ctx_s + dense_c1_offset(L);
       for (int i = lane; i < dense_c1_floats(L); i += kWave) c1_s[i] = i + 1 < L ? p.ctx[i + 1] : 0.f;
+      if (TRAIN) fill_dense_sym<R>(c1_s + dense_c1_floats(L), p.ctx, L, lane, kWave);
     }
   }
   __syncthreads();
@@ -1035,7 +1097,8 @@ __global__ void __launch_bounds__(kSplitMaxWaves * kWave) sweep_fwd_split_kernel
   float* a_s = smem;  // kMaxL floats per wavefront
   float* ctx_s = smem + (blockDim.x / kWave) * kMaxL;  // L floats, and the table moved down by one
   float* c1_s = ctx_s + dense_c1_offset(L);
-  float* xchg = c1_s + dense_c1_floats(L);
+  float* csym_s = c1_s + dense_c1_floats(L);
+  float* xchg = csym_s + dense_sym_floats(R);
   const ChainCtx ch = locate_chain(p);
   if (!JACOBI && !p.pair_q && ch.n < 2) return;  // nothing to write (the same for every wavefront)
   CtxDesc desc;
@@ -1047,6 +1110,7 @@ __global__ void __launch_bounds__(kSplitMaxWaves * kWave) sweep_fwd_split_kernel
   desc.slope = 0.f;
   for (int i = threadIdx.x; i < L; i += blockDim.x) ctx_s[i] = p.ctx[i];
   for (int i = threadIdx.x; i < dense_c1_floats(L); i += blockDim.x) c1_s[i] = i + 1 < L ? p.ctx[i + 1] : 0.f;
+  if (TRAIN) fill_dense_sym<R>(csym_s, p.ctx, L, (int)threadIdx.x, (int)blockDim.x);
   __syncthreads();
   const int halves = (!JACOBI && p.fused_pair) ? 2 : 1;
 #pragma clang loop unroll(disable)
@@ -1067,7 +1131,7 @@ __global__ void __launch_bounds__(kSplitMaxWaves * kWave) sweep_fwd_split_kernel
 
 inline size_t split_lds_bytes(int L, int R, int waves, bool train) {
   return sizeof(float) * ((size_t)waves * kMaxL + dense_c1_offset(L) + dense_c1_floats(L) +
-                          (size_t)2 * waves * kWave * (train ? 2 * R : R));
+                          dense_sym_floats(R) + (size_t)2 * waves * kWave * (train ? 2 * R : R));
 }
 
 template <int R, bool VEC, bool MASK>
