@@ -13,6 +13,8 @@
 //
 // Compiled once per R (labels per lane) with -DMPL_INST_R=<R>.
 
+#include <type_traits>
+
 #include "mp_common.h"
 
 namespace mpl {
@@ -426,25 +428,69 @@ __device__ __forceinline__ void argmin_and_lane_min_21(const float (&val)[21], f
       : "vcc");
 }
 
+// Two labels per lane, no argmin labels: the wavefront minimum of the beliefs and, in the issue slots
+// its six lane-shift minima leave (a lane shift may read a register two slots after it was written,
+// and a wavefront that has its SIMD to itself pays for every idle slot), the centre tap and the
+// first tap of the band step: on exit v[j] = min(a[j] + w c[0], min(a[label-1], a[label+1]) + w c[1]),
+// up / dn hold the beliefs of the labels one up and one down, and `red` holds in lane 63 the minimum
+// of a[] over the wavefront.  The same operations on the same operands as wave_min_fast and
+// band_step's first tap: the same bits.
+__device__ __forceinline__ void band_head_r2(const float (&a)[2], float w, float c0, float c1,
+                                             float& red, float (&v)[2], float (&up)[2],
+                                             float (&dn)[2]) {
+  float tu, td, q0, q1, p0, p1;
+  red = fminf(a[0], a[1]);
+  asm("v_mov_b32 %1, 0x7f800000\n\t"
+      "v_mov_b32 %2, 0x7f800000\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fma_f32 %5, %9, %10, %7\n\t"
+      "v_fma_f32 %6, %9, %10, %8\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+      "v_mov_b32_dpp %1, %7 wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_mov_b32_dpp %2, %8 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+      "v_min_f32 %3, %8, %2\n\t"
+      "v_min_f32 %4, %1, %7\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+      "v_fmac_f32 %3, %9, %11\n\t"
+      "v_fmac_f32 %4, %9, %11\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      "v_min_f32 %5, %5, %3\n\t"
+      "v_min_f32 %6, %6, %4\n\t"
+      "v_min_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf"
+      : "+v"(red), "=&v"(tu), "=&v"(td), "=&v"(q0), "=&v"(q1), "=&v"(p0), "=&v"(p1)
+      : "v"(a[0]), "v"(a[1]), "v"(w), "v"(c0), "v"(c1));
+  v[0] = p0;
+  v[1] = p1;
+  up[0] = a[1];
+  up[1] = tu;
+  dn[0] = td;
+  dn[1] = a[0];
+}
+
 // Band O(L*K) step for 1-D contexts with a constant tail (c[k] == cmax for k >= K, c[k] <= cmax
 // below), exact for w >= 0:
 //   v[cd] = min( min_{|k|<K} a[cd+k] + w*c[|k|],  min_fd a[fd] + w*cmax )
 // The second term is an upper bound for every label and is attained by all labels farther than the
 // band from argmin(a); fp32 addition is monotone, so the values are bit-identical to the dense scan.
 // KT > 0: KT - 1 taps with c[] in registers (KT >= K).  KT == 0: K at run time, taps in LDS.
-template <int R, bool TRAIN, int KT>
+// HEAD (band_head_r2 ran: KT >= 2 in registers, no argmin labels): v, up and dn come in as the
+// first tap left them, and the taps go on from the second.
+template <int R, bool TRAIN, int KT, bool HEAD = false>
 __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, const float* c_reg,
                                           const float* ctx_s, float cmax, float amin, int fstar,
-                                          int lab0, float (&v)[R], int (&fd_idx)[R]) {
+                                          int lab0, float (&v)[R], int (&fd_idx)[R],
+                                          const float* up_in = nullptr, const float* dn_in = nullptr) {
+  static_assert(!HEAD || (KT >= 2 && !TRAIN), "the head covers the first tap of a band in registers");
   const float inf = INFINITY;
   float up[R], dn[R];
   int off[R];
   const float c0 = KT > 0 ? c_reg[0] : ctx_s[0];
 #pragma unroll
   for (int j = 0; j < R; ++j) {
-    up[j] = a[j];
-    dn[j] = a[j];
-    v[j] = fmaf(w, c0, a[j]);
+    up[j] = HEAD ? up_in[j] : a[j];
+    dn[j] = HEAD ? dn_in[j] : a[j];
+    if (!HEAD) v[j] = fmaf(w, c0, a[j]);
     off[j] = 0;
   }
   // `refill`: up[0] / dn[R-1] still hold unshifted beliefs, so the vacated lane is set to +inf;
@@ -479,7 +525,7 @@ __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, c
   };
   if (KT > 0) {
 #pragma unroll
-    for (int k = 1; k < KT; ++k) tap(k, c_reg[k], k <= R);
+    for (int k = HEAD ? 2 : 1; k < KT; ++k) tap(k, c_reg[k], k <= R);
   } else {
     // R taps per trip: the R one-label rotations of up[] / dn[] then cancel, so the loop carries
     // no register moves, and the R coefficients are fetched from LDS together
@@ -608,7 +654,9 @@ __device__ __forceinline__ void linear_step(const float (&a)[R], float w, float 
 // exactly 21 labels, -2 truncated linear context of any width (linear_step), -3 dense 1-D table with
 // the front labels split over the wavefronts of the workgroup (split_combine; xchg: its LDS slots).
 // VEC: L % R == 0 (vector accesses).  MASK: some lanes own labels >= L.
-template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI, int KT>
+// C0: the table's entry 0 is its smallest (band steps only; CtxDesc::c0_is_min), which gives the
+// normalisation minimum without a second reduction.
+template <int R, bool VEC, bool MASK, bool TRAIN, int JACOBI, int KT, bool C0 = false>
 __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDesc& desc,
                                               const ChainCtx& ch, float* a_s, const float* ctx_s,
                                               const bool skip_s_store_in, float* xchg = nullptr) {
@@ -683,8 +731,14 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   }
 
   bool valid[R];
+  // a lane's labels beyond the last one are kept at +inf by a maximum with +inf (-inf for the
+  // others, which changes nothing): one instruction in the short encoding, no lane masks to hold
+  float floor_l[R];
 #pragma unroll
-  for (int j = 0; j < R; ++j) valid[j] = MASK ? (lab0 + j < L) : true;
+  for (int j = 0; j < R; ++j) {
+    valid[j] = MASK ? (lab0 + j < L) : true;
+    floor_l[j] = valid[j] ? -INFINITY : INFINITY;
+  }
 
   float c_reg[KT > 0 ? KT : 1];
   if (KT > 0) {
@@ -699,8 +753,10 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     for (int fd = 0; fd < LT; ++fd) tcol[fd] = ctx_s[fd * LT + (lane < LT ? lane : LT - 1)];
   }
   const int K = desc.band_k;
-  const float cmax = desc.cmax;
-  const bool c0min = desc.c0_is_min != 0;
+  // (in a vector register for the whole chain: the far candidate multiplies it by the edge weight
+  // and adds the minimum, both scalars, and a multiply-add takes one scalar operand)
+  float cmax = desc.cmax;
+  asm volatile("" : "+v"(cmax));
 
   // first Gauss-Seidel iteration over all-zero initial messages: the plane of this direction has
   // not been swept yet, and neither has the opposite one when this direction is the even one
@@ -723,6 +779,13 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   // (all-zero initial messages, the odd sweep's own old messages) or stored get an empty descriptor.
   const bool lane_ok = !MASK || lab0 < L;
   const int img_bytes = (int)(unsigned)(HW * L * 4);
+  // (VEC and MASK: a lane without labels carries the size of the image in place of its offset, which
+  // takes every access of its past the end of every plane without a select per access; the host
+  // gives images beyond 2 GiB, where that sum could wrap, to the kernels that form a descriptor per
+  // access)
+  // (one label per lane: every image goes through these kernels, and the select stays)
+  constexpr bool kAddDead = R > 1;
+  const unsigned foff_ok = lane_ok ? (unsigned)foff : (unsigned)img_bytes;
   const rsrc_t rS = make_rsrc(bS, img_bytes);
   const rsrc_t rMd0 = make_rsrc(bMd, md_zero ? 0 : img_bytes);  // chain start
   const rsrc_t rMd = make_rsrc(bMd, (md_zero || pair_second) ? 0 : img_bytes);
@@ -741,7 +804,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
     const unsigned pp = (unsigned)uniform_i((VEC || ld_t < n) ? ld_p : last_p);
     const unsigned so = pp * (unsigned)vbytes;
     if constexpr (VEC) {
-      const int vo = (int)(lane_ok ? so + (unsigned)foff : kDeadWide);
+      const int vo = (int)(kAddDead ? so + foff_ok : (lane_ok ? so + (unsigned)foff : kDeadWide));
       buf_load<R, true>(rS, vo, 0u, r.s);
       if (JACOBI == 0) {
         buf_load<R, true>(first ? rMd0 : rMd, vo, 0u, r.md);
@@ -833,8 +896,10 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   }
 
   int st_p = ch.pix0 + ch.pstep;
-  auto step = [&](const PixF<R>& px, const int t) __attribute__((always_inline)) {
-      const bool live = t < n;  // steps past the end compute on stale data and store nothing
+  // in_chain: a constant `true` where the caller knows that step t lies inside the chain
+  auto step = [&](const PixF<R>& px, const int t, const auto in_chain) __attribute__((always_inline)) {
+      // steps past the end compute on stale data and store nothing
+      const bool live = decltype(in_chain)::value || t < n;
       float tt[R], un[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) {
@@ -846,20 +911,37 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         } else {
           tt[j] = 0.f;
         }
-        un[j] = valid[j] ? x : inf;
+        un[j] = MASK ? fmaxf(x, floor_l[j]) : x;
       }
       const float w = uniform_f(px.w);
       float a[R], v[R];
       int fd_idx[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) a[j] = fmaf(rho, prev[j], uf[j]);
+      // the normalisation minimum of v (every path ends with it or with a cheaper way to it: the
+      // usual path then runs through without a flag to test)
       float nmin;
-      bool need_nmin = true;
-      if ((KT >= 0 || KT == -2) && __builtin_expect(w >= 0.f, 1)) {  // (the usual case falls through)
-        float am = a[0];
+      auto norm_min = [&]() __attribute__((always_inline)) {
+        float vm = inf;
 #pragma unroll
-        for (int j = 1; j < R; ++j) am = fminf(am, a[j]);
-        const float amin = wave_min_fast(am);
+        for (int j = 0; j < R; ++j) vm = fminf(vm, MASK ? fmaxf(v[j], floor_l[j]) : v[j]);
+        return wave_min_fast(vm);
+      };
+      if ((KT >= 0 || KT == -2) && __builtin_expect(w >= 0.f, 1)) {  // (the usual case falls through)
+        // (two labels per lane without argmin labels: the reduction and the first tap in one block)
+        constexpr bool kHead = R == 2 && !TRAIN && KT >= 2;
+        float amin;
+        float hup[R], hdn[R];
+        if constexpr (kHead) {
+          float red;
+          band_head_r2(a, px.w, c_reg[0], c_reg[1], red, v, hup, hdn);
+          amin = readlane_f(red, 63);
+        } else {
+          float am = a[0];
+#pragma unroll
+          for (int j = 1; j < R; ++j) am = fminf(am, a[j]);
+          amin = wave_min_fast(am);
+        }
         int fstar = L - 1;
         if (TRAIN) {
           bool pr[R];
@@ -871,13 +953,16 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
           linear_step<R, TRAIN>(a, w, desc.slope, cmax, amin, fstar, lab0, lane, L, a_s, ctx_s, v,
                                 fd_idx);
         } else {
-          band_step<R, TRAIN, (KT > 0 ? KT : 0)>(a, w, K, c_reg, ctx_s, cmax, amin, fstar, lab0, v,
-                                                 fd_idx);
+          // (after the head the weight is taken from the vector register every lane loaded it
+          // into: the minimum arrives in a scalar register, and a multiply-add reads one scalar)
+          band_step<R, TRAIN, (KT > 0 ? KT : 0), kHead>(a, kHead ? px.w : w, K, c_reg, ctx_s, cmax, amin,
+                                                        fstar, lab0, v, fd_idx, hup, hdn);
         }
-        if (KT != -2 && c0min) {
+        if constexpr (KT != -2 && C0) {
           // every candidate is >= amin + w*c[0], which the centre tap of label argmin(a) attains
-          nmin = fmaf(w, KT > 0 ? c_reg[0] : ctx_s[0], amin);
-          need_nmin = false;
+          nmin = fmaf(kHead ? px.w : w, KT > 0 ? c_reg[0] : ctx_s[0], amin);
+        } else {
+          nmin = norm_min();
         }
       } else if (R == 1 && KT < 0 && desc.band_k == 0) {  // (the full table is in LDS then)
         if constexpr (LT > 0) {
@@ -903,12 +988,13 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
             float red = valid[0] ? best : inf;
             argmin_and_lane_min_21(val, best, red, fd_idx[0]);
             nmin = readlane_f(red, 31);
-            need_nmin = false;
           } else {
             fd_idx[0] = LT - 1;
+            nmin = norm_min();
           }
         } else {
           dense_step_r1<TRAIN>(a[0], L, w, lane, ctx_s, v[0], fd_idx[0]);
+          nmin = norm_min();
         }
       } else if (live) {
         if constexpr (R > 1) {  // (2-D tables exist for one label per lane only)
@@ -926,18 +1012,14 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         } else {
           dense_step<R, TRAIN>(a, valid, w, L, p.ctx2d, lab0, a_s, ctx_s, v, fd_idx);
         }
+        nmin = norm_min();
       } else {
 #pragma unroll
         for (int j = 0; j < R; ++j) {
           v[j] = 0.f;
           fd_idx[j] = 0;
         }
-      }
-      if (need_nmin) {
-        float vm = inf;
-#pragma unroll
-        for (int j = 0; j < R; ++j) vm = fminf(vm, valid[j] ? v[j] : inf);
-        nmin = wave_min_fast(vm);
+        nmin = 0.f;
       }
       float m[R], sn[R];
 #pragma unroll
@@ -952,7 +1034,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       const unsigned sob = sp * (unsigned)L;
       if constexpr (VEC) {
         const bool on = lane_ok && live && store_ok;  // nothing is stored past the end
-        const int vo = (int)(on ? so + (unsigned)foff : kDeadWide);
+        const int vo = (int)(kAddDead ? ((live && store_ok) ? so + foff_ok : kDeadWide)
+                                      : (on ? so + (unsigned)foff : kDeadWide));
         buf_store<R, true>(rMo, vo, 0u, m);
         if (!JACOBI) buf_store<R, true>(rSo, vo, 0u, sn);
         if (TRAIN) buf_store_u8<R, true>(rImin, (int)(on ? sob + (unsigned)lab0 : kDeadWide), 0u, fd_idx);
@@ -973,14 +1056,36 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       }
       st_p += ch.pstep;
   };
-  for (int t0 = 1; t0 < n; t0 += 2 * D) {
+  // Trips of 2 D steps that lie inside the chain: nothing in them asks whether a step is past the
+  // end.  Without argmin labels only (the scans of the usual training sizes share their SIMDs and
+  // wait for memory, not for issue slots; their code is large enough as it is).
+  int t0 = 1;
+  if constexpr (!TRAIN) {
+    for (; t0 + 2 * D <= n; t0 += 2 * D) {
+#pragma unroll
+      for (int u = 0; u < D; ++u) {
+        // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
+        wait_vmem<(D - 1) * kOps>();
+        const PixF<R> px = ring[u];
+        ring2[u] = load_next();
+        step(px, t0 + u, std::true_type());
+      }
+#pragma unroll
+      for (int u = 0; u < D; ++u) {
+        wait_vmem<(D - 1) * kOps>();
+        const PixF<R> px = ring2[u];
+        ring[u] = load_next();
+        step(px, t0 + D + u, std::true_type());
+      }
+    }
+  }
+  for (; t0 < n; t0 += 2 * D) {
 #pragma unroll
     for (int u = 0; u < D; ++u) {
-      // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
       wait_vmem<(D - 1) * kOps>();
       const PixF<R> px = ring[u];
       ring2[u] = load_next();
-      step(px, t0 + u);
+      step(px, t0 + u, std::false_type());
     }
     if (t0 + D >= n) break;  // wave-uniform
 #pragma unroll
@@ -988,7 +1093,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       wait_vmem<(D - 1) * kOps>();
       const PixF<R> px = ring2[u];
       ring[u] = load_next();
-      step(px, t0 + D + u);
+      step(px, t0 + D + u, std::false_type());
     }
   }
 }
@@ -1055,6 +1160,12 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
       run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -2>(p, desc, c, a_s, ctx_s, skip_s);
       continue;
     }
+    // (a band whose entry 0 is not its smallest -- no Potts, linear or quadratic table -- takes the
+    // taps at run time and reduces for the normalisation minimum)
+    if (desc.band_k > 0 && !desc.c0_is_min) {
+      run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0, false>(p, desc, c, a_s, ctx_s, skip_s);
+      continue;
+    }
     switch (desc.band_k) {
       case 0:
         if (R == 1 && L == 21)
@@ -1062,9 +1173,9 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
         else
           run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, -1>(p, desc, c, a_s, ctx_s, skip_s);
         break;
-      case 2: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 2>(p, desc, c, a_s, ctx_s, skip_s); break;
-      case 3: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 3>(p, desc, c, a_s, ctx_s, skip_s); break;
-      case 4: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 4>(p, desc, c, a_s, ctx_s, skip_s); break;
+      case 2: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 2, true>(p, desc, c, a_s, ctx_s, skip_s); break;
+      case 3: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 3, true>(p, desc, c, a_s, ctx_s, skip_s); break;
+      case 4: run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 4, true>(p, desc, c, a_s, ctx_s, skip_s); break;
       default:
         // wider bands with the taps in registers: the table is constant from band_k on, so the
         // taps between band_k and the compiled width are the dense scan's own candidates
@@ -1072,15 +1183,15 @@ __global__ void __launch_bounds__(kWave) sweep_fwd_kernel(const SweepParams p) {
         // and pay for the larger kernel)
         if constexpr (R >= 2) {
           if (desc.band_k <= 8) {
-            run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 8>(p, desc, c, a_s, ctx_s, skip_s);
+            run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 8, true>(p, desc, c, a_s, ctx_s, skip_s);
             break;
           }
           if (desc.band_k <= 16) {
-            run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 16>(p, desc, c, a_s, ctx_s, skip_s);
+            run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 16, true>(p, desc, c, a_s, ctx_s, skip_s);
             break;
           }
         }
-        run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0>(p, desc, c, a_s, ctx_s, skip_s);
+        run_chain_fwd<R, VEC, MASK, TRAIN, JACOBI, 0, true>(p, desc, c, a_s, ctx_s, skip_s);
         break;
     }
   }
@@ -1190,8 +1301,11 @@ void launch_vm(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
 template <int R>
 void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
   if (p.block_prefix[p.n_dirs] <= 0) return;
-  const bool vec = (p.L % R) == 0;
   const bool mask = p.L != R * kWave;
+  // one descriptor per plane for the whole kernel: whole lanes of labels, and, where some lanes have
+  // none, an image of at most 2 GiB (run_chain_fwd, foff_ok)
+  const bool vec = (p.L % R) == 0 &&
+                   (!mask || (int64_t)p.H * p.W * p.L * 4 <= (int64_t)1 << 31);
   if constexpr (R > 1) {
     if (!vec) {
       launch_vm<R, false, true>(p, train, jacobi, st);
