@@ -1057,10 +1057,11 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       st_p += ch.pstep;
   };
   // Trips of 2 D steps that lie inside the chain: nothing in them asks whether a step is past the
-  // end.  Without argmin labels only (the scans of the usual training sizes share their SIMDs and
-  // wait for memory, not for issue slots; their code is large enough as it is).
+  // end.  Without argmin labels, or with one label per lane (the scans of the usual training sizes
+  // with more labels share their SIMDs and wait for memory, not for issue slots; their code is
+  // large enough as it is).
   int t0 = 1;
-  if constexpr (!TRAIN) {
+  if constexpr (!TRAIN || R == 1) {
     for (; t0 + 2 * D <= n; t0 += 2 * D) {
 #pragma unroll
       for (int u = 0; u < D; ++u) {
