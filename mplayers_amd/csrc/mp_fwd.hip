@@ -428,33 +428,33 @@ __device__ __forceinline__ void argmin_and_lane_min_21(const float (&val)[21], f
       : "vcc");
 }
 
-// Two labels per lane, no argmin labels: the wavefront minimum of the beliefs and, in the issue slots
-// its six lane-shift minima leave (a lane shift may read a register two slots after it was written,
-// and a wavefront that has its SIMD to itself pays for every idle slot), the centre tap and the
-// first tap of the band step: on exit v[j] = min(a[j] + w c[0], min(a[label-1], a[label+1]) + w c[1]),
+// Several labels per lane, no argmin labels: the wavefront minimum of the beliefs and, in the issue
+// slots its six lane-shift minima leave (a lane shift may read a register two slots after it was
+// written, and a wavefront that has its SIMD to itself pays for every idle slot), the centre tap and
+// the first tap of the band step: on exit v[j] = min(a[j] + w c[0], min(a[label-1], a[label+1]) + w c[1]),
 // up / dn hold the beliefs of the labels one up and one down, and `red` holds in lane 63 the minimum
 // of a[] over the wavefront.  The same operations on the same operands as wave_min_fast and
-// band_step's first tap: the same bits.
-__device__ __forceinline__ void band_head_r2(const float (&a)[2], float w, float c0, float c1,
-                                             float& red, float (&v)[2], float (&up)[2],
-                                             float (&dn)[2]) {
+// band_step's first tap: the same bits.  w: the edge weight in a vector register.
+#define MPL_RED(CTRL) "v_min_f32_dpp %0, %0, %0 " CTRL " bank_mask:0xf\n\t"
+__device__ __forceinline__ void band_head(const float (&a)[2], float w, float c0, float c1, float& red,
+                                          float (&v)[2], float (&up)[2], float (&dn)[2]) {
   float tu, td, q0, q1, p0, p1;
   red = fminf(a[0], a[1]);
   asm("v_mov_b32 %1, 0x7f800000\n\t"
       "v_mov_b32 %2, 0x7f800000\n\t"
-      "v_min_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      MPL_RED("row_shr:1 row_mask:0xf")
       "v_fma_f32 %5, %9, %10, %7\n\t"
       "v_fma_f32 %6, %9, %10, %8\n\t"
-      "v_min_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+      MPL_RED("row_shr:2 row_mask:0xf")
       "v_mov_b32_dpp %1, %7 wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
       "v_mov_b32_dpp %2, %8 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
-      "v_min_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+      MPL_RED("row_shr:4 row_mask:0xf")
       "v_min_f32 %3, %8, %2\n\t"
       "v_min_f32 %4, %1, %7\n\t"
-      "v_min_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf\n\t"
+      MPL_RED("row_shr:8 row_mask:0xf")
       "v_fmac_f32 %3, %9, %11\n\t"
       "v_fmac_f32 %4, %9, %11\n\t"
-      "v_min_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+      MPL_RED("row_bcast:15 row_mask:0xa")
       "v_min_f32 %5, %5, %3\n\t"
       "v_min_f32 %6, %6, %4\n\t"
       "v_min_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf"
@@ -468,13 +468,102 @@ __device__ __forceinline__ void band_head_r2(const float (&a)[2], float w, float
   dn[1] = a[0];
 }
 
+__device__ __forceinline__ void band_head(const float (&a)[3], float w, float c0, float c1, float& red,
+                                          float (&v)[3], float (&up)[3], float (&dn)[3]) {
+  float tu, td, q0, q1, q2, p0, p1, p2;
+  red = fminf(fminf(a[0], a[1]), a[2]);
+  // %0 red  %1 tu  %2 td  %3..%5 q  %6..%8 p  %9..%11 a  %12 w  %13 c0  %14 c1
+  asm("v_mov_b32 %1, 0x7f800000\n\t"
+      "v_mov_b32 %2, 0x7f800000\n\t"
+      MPL_RED("row_shr:1 row_mask:0xf")
+      "v_fma_f32 %6, %12, %13, %9\n\t"
+      "v_fma_f32 %7, %12, %13, %10\n\t"
+      MPL_RED("row_shr:2 row_mask:0xf")
+      "v_mov_b32_dpp %1, %9 wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_mov_b32_dpp %2, %11 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      MPL_RED("row_shr:4 row_mask:0xf")
+      "v_fma_f32 %8, %12, %13, %11\n\t"
+      "v_min_f32 %4, %11, %9\n\t"
+      MPL_RED("row_shr:8 row_mask:0xf")
+      "v_min_f32 %3, %10, %2\n\t"
+      "v_min_f32 %5, %1, %10\n\t"
+      MPL_RED("row_bcast:15 row_mask:0xa")
+      "v_fmac_f32 %3, %12, %14\n\t"
+      "v_fmac_f32 %4, %12, %14\n\t"
+      MPL_RED("row_bcast:31 row_mask:0xc")
+      "v_fmac_f32 %5, %12, %14\n\t"
+      "v_min_f32 %6, %6, %3\n\t"
+      "v_min_f32 %7, %7, %4\n\t"
+      "v_min_f32 %8, %8, %5"
+      : "+v"(red), "=&v"(tu), "=&v"(td), "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(p0), "=&v"(p1),
+        "=&v"(p2)
+      : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(w), "v"(c0), "v"(c1));
+  v[0] = p0;
+  v[1] = p1;
+  v[2] = p2;
+  up[0] = a[1];
+  up[1] = a[2];
+  up[2] = tu;
+  dn[0] = td;
+  dn[1] = a[0];
+  dn[2] = a[1];
+}
+
+__device__ __forceinline__ void band_head(const float (&a)[4], float w, float c0, float c1, float& red,
+                                          float (&v)[4], float (&up)[4], float (&dn)[4]) {
+  float tu, td, q0, q1, q2, q3, p0, p1, p2, p3;
+  red = fminf(fminf(a[0], a[1]), fminf(a[2], a[3]));
+  // %0 red  %1 tu  %2 td  %3..%6 q  %7..%10 p  %11..%14 a  %15 w  %16 c0  %17 c1
+  asm("v_mov_b32 %1, 0x7f800000\n\t"
+      "v_mov_b32 %2, 0x7f800000\n\t"
+      MPL_RED("row_shr:1 row_mask:0xf")
+      "v_fma_f32 %7, %15, %16, %11\n\t"
+      "v_fma_f32 %8, %15, %16, %12\n\t"
+      MPL_RED("row_shr:2 row_mask:0xf")
+      "v_mov_b32_dpp %1, %11 wave_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+      "v_mov_b32_dpp %2, %14 wave_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+      MPL_RED("row_shr:4 row_mask:0xf")
+      "v_fma_f32 %9, %15, %16, %13\n\t"
+      "v_fma_f32 %10, %15, %16, %14\n\t"
+      MPL_RED("row_shr:8 row_mask:0xf")
+      "v_min_f32 %4, %13, %11\n\t"
+      "v_min_f32 %5, %14, %12\n\t"
+      MPL_RED("row_bcast:15 row_mask:0xa")
+      "v_min_f32 %3, %12, %2\n\t"
+      "v_min_f32 %6, %1, %13\n\t"
+      MPL_RED("row_bcast:31 row_mask:0xc")
+      "v_fmac_f32 %3, %15, %17\n\t"
+      "v_fmac_f32 %4, %15, %17\n\t"
+      "v_fmac_f32 %5, %15, %17\n\t"
+      "v_fmac_f32 %6, %15, %17\n\t"
+      "v_min_f32 %7, %7, %3\n\t"
+      "v_min_f32 %8, %8, %4\n\t"
+      "v_min_f32 %9, %9, %5\n\t"
+      "v_min_f32 %10, %10, %6"
+      : "+v"(red), "=&v"(tu), "=&v"(td), "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(p0),
+        "=&v"(p1), "=&v"(p2), "=&v"(p3)
+      : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(w), "v"(c0), "v"(c1));
+  v[0] = p0;
+  v[1] = p1;
+  v[2] = p2;
+  v[3] = p3;
+  up[0] = a[1];
+  up[1] = a[2];
+  up[2] = a[3];
+  up[3] = tu;
+  dn[0] = td;
+  dn[1] = a[0];
+  dn[2] = a[1];
+  dn[3] = a[2];
+}
+#undef MPL_RED
 // Band O(L*K) step for 1-D contexts with a constant tail (c[k] == cmax for k >= K, c[k] <= cmax
 // below), exact for w >= 0:
 //   v[cd] = min( min_{|k|<K} a[cd+k] + w*c[|k|],  min_fd a[fd] + w*cmax )
 // The second term is an upper bound for every label and is attained by all labels farther than the
 // band from argmin(a); fp32 addition is monotone, so the values are bit-identical to the dense scan.
 // KT > 0: KT - 1 taps with c[] in registers (KT >= K).  KT == 0: K at run time, taps in LDS.
-// HEAD (band_head_r2 ran: KT >= 2 in registers, no argmin labels): v, up and dn come in as the
+// HEAD (band_head ran: KT >= 2 in registers, several labels per lane, no argmin labels): v, up and dn come in as the
 // first tap left them, and the taps go on from the second.
 template <int R, bool TRAIN, int KT, bool HEAD = false>
 __device__ __forceinline__ void band_step(const float (&a)[R], float w, int K, const float* c_reg,
@@ -928,13 +1017,14 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         return wave_min_fast(vm);
       };
       if ((KT >= 0 || KT == -2) && __builtin_expect(w >= 0.f, 1)) {  // (the usual case falls through)
-        // (two labels per lane without argmin labels: the reduction and the first tap in one block)
-        constexpr bool kHead = R == 2 && !TRAIN && KT >= 2;
+        // (several labels per lane without argmin labels: the reduction and the first tap in one
+        // block)
+        constexpr bool kHead = R >= 2 && !TRAIN && KT >= 2;
         float amin;
         float hup[R], hdn[R];
         if constexpr (kHead) {
           float red;
-          band_head_r2(a, px.w, c_reg[0], c_reg[1], red, v, hup, hdn);
+          band_head(a, px.w, c_reg[0], c_reg[1], red, v, hup, hdn);
           amin = readlane_f(red, 63);
         } else {
           float am = a[0];
