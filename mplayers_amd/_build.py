@@ -2,8 +2,9 @@
 measurement probes (csrc/mp_probe.hip) into libmplayers_probe.so, which only the benchmark and the
 tests load.
 
-The scan kernels are instantiated once per R (labels per lane, 1..4); each instantiation is its
-own translation unit so that they compile in parallel.
+The scan kernels are instantiated once per R (labels per lane, 1..4), the forward scans also once
+with and once without argmin labels; each instantiation is its own translation unit so that they
+compile in parallel.
 """
 import os
 import subprocess
@@ -30,8 +31,10 @@ def _units():
            ("mp_soft", "mp_soft.hip", []), ("mp_pack", "mp_pack.hip", []),
            ("mp_terms", "mp_terms.hip", []), ("mp_probe", "mp_probe.hip", []),
            ("mp_layout", "mp_layout.hip", [])]
-  for r in (1, 2, 3, 4):
-    units.append(("mp_fwd_r%d" % r, "mp_fwd.hip", ["-DMPL_INST_R=%d" % r]))
+  for r in (4, 3, 2, 1):  # (the largest units first)
+    for t in (1, 0):
+      units.append(("mp_fwd_r%d_t%d" % (r, t), "mp_fwd.hip",
+                    ["-DMPL_INST_R=%d" % r, "-DMPL_INST_TRAIN=%d" % t]))
     units.append(("mp_bwd_r%d" % r, "mp_bwd.hip", ["-DMPL_INST_R=%d" % r]))
   return units
 

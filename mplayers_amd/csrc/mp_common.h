@@ -535,8 +535,15 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int set_cpu_threads(int n);
 
 // launchers, one translation unit per R so that the instantiations compile in parallel
+template <int R, bool TRAIN>
+void launch_sweep_fwd_t(const SweepParams& p, bool jacobi, hipStream_t st);
 template <int R>
-void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st);
+inline void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+  if (train)
+    launch_sweep_fwd_t<R, true>(p, jacobi, st);
+  else
+    launch_sweep_fwd_t<R, false>(p, jacobi, st);
+}
 template <int R>
 void launch_sweep_bwd(const BackParams& p, bool jacobi, hipStream_t st);
 

@@ -11,7 +11,8 @@
 // over directions) forms U on the fly from S, m_dir, m_inv and keeps S up to date; ISGMR (Jacobi)
 // finds U of every direction precomputed in place of the old messages.
 //
-// Compiled once per R (labels per lane) with -DMPL_INST_R=<R>.
+// Compiled once per R (labels per lane) and per kind of scan (with or without argmin labels) with
+// -DMPL_INST_R=<R> -DMPL_INST_TRAIN=<0|1>.
 
 #include <type_traits>
 
@@ -1336,61 +1337,44 @@ inline size_t split_lds_bytes(int L, int R, int waves, bool train) {
                           dense_sym_floats(R) + (size_t)2 * waves * kWave * (train ? 2 * R : R));
 }
 
-template <int R, bool VEC, bool MASK>
-void launch_vm_split(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+template <int R, bool VEC, bool MASK, bool TRAIN>
+void launch_vm_split(const SweepParams& p, bool jacobi, hipStream_t st) {
   const int blocks = p.block_prefix[p.n_dirs];
   const int threads = p.split * kWave;
-  const size_t lds = split_lds_bytes(p.L, R, p.split, train);
+  const size_t lds = split_lds_bytes(p.L, R, p.split, TRAIN);
   const int mode = jacobi ? (p.u_fused ? 2 : 1) : 0;
-  if (train) {
-    if (mode == 2)
-      sweep_fwd_split_kernel<R, VEC, MASK, true, 2><<<blocks, threads, lds, st>>>(p);
-    else if (mode == 1)
-      sweep_fwd_split_kernel<R, VEC, MASK, true, 1><<<blocks, threads, lds, st>>>(p);
-    else
-      sweep_fwd_split_kernel<R, VEC, MASK, true, 0><<<blocks, threads, lds, st>>>(p);
-  } else {
-    if (mode == 2)
-      sweep_fwd_split_kernel<R, VEC, MASK, false, 2><<<blocks, threads, lds, st>>>(p);
-    else if (mode == 1)
-      sweep_fwd_split_kernel<R, VEC, MASK, false, 1><<<blocks, threads, lds, st>>>(p);
-    else
-      sweep_fwd_split_kernel<R, VEC, MASK, false, 0><<<blocks, threads, lds, st>>>(p);
-  }
+  if (mode == 2)
+    sweep_fwd_split_kernel<R, VEC, MASK, TRAIN, 2><<<blocks, threads, lds, st>>>(p);
+  else if (mode == 1)
+    sweep_fwd_split_kernel<R, VEC, MASK, TRAIN, 1><<<blocks, threads, lds, st>>>(p);
+  else
+    sweep_fwd_split_kernel<R, VEC, MASK, TRAIN, 0><<<blocks, threads, lds, st>>>(p);
 }
 
-template <int R, bool VEC, bool MASK>
-void launch_vm(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+template <int R, bool VEC, bool MASK, bool TRAIN>
+void launch_vm(const SweepParams& p, bool jacobi, hipStream_t st) {
   if constexpr (R > 1) {
     if (p.split >= 2 && !p.ctx2d) {
-      launch_vm_split<R, VEC, MASK>(p, train, jacobi, st);
+      launch_vm_split<R, VEC, MASK, TRAIN>(p, jacobi, st);
       return;
     }
   }
   const int blocks = p.block_prefix[p.n_dirs];
   const size_t lds = fwd_lds_bytes(p.L, p.ctx2d);
   const int mode = jacobi ? (p.u_fused ? 2 : 1) : 0;
-  if (train) {
-    if (mode == 2)
-      sweep_fwd_kernel<R, VEC, MASK, true, 2><<<blocks, kWave, lds, st>>>(p);
-    else if (mode == 1)
-      sweep_fwd_kernel<R, VEC, MASK, true, 1><<<blocks, kWave, lds, st>>>(p);
-    else
-      sweep_fwd_kernel<R, VEC, MASK, true, 0><<<blocks, kWave, lds, st>>>(p);
-  } else {
-    if (mode == 2)
-      sweep_fwd_kernel<R, VEC, MASK, false, 2><<<blocks, kWave, lds, st>>>(p);
-    else if (mode == 1)
-      sweep_fwd_kernel<R, VEC, MASK, false, 1><<<blocks, kWave, lds, st>>>(p);
-    else
-      sweep_fwd_kernel<R, VEC, MASK, false, 0><<<blocks, kWave, lds, st>>>(p);
-  }
+  if (mode == 2)
+    sweep_fwd_kernel<R, VEC, MASK, TRAIN, 2><<<blocks, kWave, lds, st>>>(p);
+  else if (mode == 1)
+    sweep_fwd_kernel<R, VEC, MASK, TRAIN, 1><<<blocks, kWave, lds, st>>>(p);
+  else
+    sweep_fwd_kernel<R, VEC, MASK, TRAIN, 0><<<blocks, kWave, lds, st>>>(p);
 }
 
 }  // namespace
 
-template <int R>
-void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t st) {
+// (the scans that keep argmin labels and those that do not are compiled as separate units)
+template <int R, bool TRAIN>
+void launch_sweep_fwd_t(const SweepParams& p, bool jacobi, hipStream_t st) {
   if (p.block_prefix[p.n_dirs] <= 0) return;
   const bool mask = p.L != R * kWave;
   // one descriptor per plane for the whole kernel: whole lanes of labels, and, where some lanes have
@@ -1399,16 +1383,16 @@ void launch_sweep_fwd(const SweepParams& p, bool train, bool jacobi, hipStream_t
                    (!mask || (int64_t)p.H * p.W * p.L * 4 <= (int64_t)1 << 31);
   if constexpr (R > 1) {
     if (!vec) {
-      launch_vm<R, false, true>(p, train, jacobi, st);
+      launch_vm<R, false, true, TRAIN>(p, jacobi, st);
       return;
     }
   }
   if (mask)
-    launch_vm<R, true, true>(p, train, jacobi, st);
+    launch_vm<R, true, true, TRAIN>(p, jacobi, st);
   else
-    launch_vm<R, true, false>(p, train, jacobi, st);
+    launch_vm<R, true, false, TRAIN>(p, jacobi, st);
 }
 
-template void launch_sweep_fwd<MPL_INST_R>(const SweepParams&, bool, bool, hipStream_t);
+template void launch_sweep_fwd_t<MPL_INST_R, (MPL_INST_TRAIN != 0)>(const SweepParams&, bool, hipStream_t);
 
 }  // namespace mpl
