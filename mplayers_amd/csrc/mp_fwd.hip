@@ -986,10 +986,12 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
   }
 
   int st_p = ch.pix0 + ch.pstep;
-  // in_chain: a constant `true` where the caller knows that step t lies inside the chain
+  // in_chain: a constant `true` where the caller knows that step t lies inside the chain and that
+  // no edge weight of the chain is negative
   auto step = [&](const PixF<R>& px, const int t, const auto in_chain) __attribute__((always_inline)) {
+      constexpr bool kPlain = decltype(in_chain)::value;
       // steps past the end compute on stale data and store nothing
-      const bool live = decltype(in_chain)::value || t < n;
+      const bool live = kPlain || t < n;
       float tt[R], un[R];
 #pragma unroll
       for (int j = 0; j < R; ++j) {
@@ -1017,7 +1019,8 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         for (int j = 0; j < R; ++j) vm = fminf(vm, MASK ? fmaxf(v[j], floor_l[j]) : v[j]);
         return wave_min_fast(vm);
       };
-      if ((KT >= 0 || KT == -2) && __builtin_expect(w >= 0.f, 1)) {  // (the usual case falls through)
+      // (the usual case falls through; the trips of steps that the caller vouches for do not ask)
+      if ((KT >= 0 || KT == -2) && (kPlain || __builtin_expect(w >= 0.f, 1))) {
         // (several labels per lane without argmin labels: the reduction and the first tap in one
         // block)
         constexpr bool kHead = R >= 2 && !TRAIN && KT >= 2;
@@ -1147,13 +1150,28 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
       }
       st_p += ch.pstep;
   };
-  // Trips of 2 D steps that lie inside the chain: nothing in them asks whether a step is past the
-  // end.  Without argmin labels, or with one label per lane (the scans of the usual training sizes
-  // with more labels share their SIMDs and wait for memory, not for issue slots; their code is
-  // large enough as it is).
+  // Trips of 2 D steps that lie inside the chain, on a chain without negative edge weights (the
+  // band and the label scans hold for every step then): nothing in them asks whether a step is past
+  // the end or which way its weight points, and the step for negative weights is not part of their
+  // code.  A chain with such a weight takes the loop below from its first step.  Without argmin
+  // labels, or with one label per lane (the scans of the usual training sizes with more labels
+  // share their SIMDs and wait for memory, not for issue slots; their code is large enough as it is).
   int t0 = 1;
   if constexpr (!TRAIN || R == 1) {
-    for (; t0 + 2 * D <= n; t0 += 2 * D) {
+    bool plain = true;
+    if constexpr (KT >= 0 || KT == -2) {
+      if (n > 2 * D) {  // (there is such a trip)
+        bool bad = false;
+        for (int i = lane; i < n; i += kWave) {
+          const unsigned pi = (unsigned)(ch.pix0 + i * ch.pstep);
+          const float wi = __builtin_bit_cast(
+              float, __builtin_amdgcn_raw_buffer_load_b32(dW, (int)(pi * 4u), 0, 0));
+          bad |= !(wi >= 0.f);
+        }
+        plain = ballot(bad) == 0;
+      }
+    }
+    for (; plain && t0 + 2 * D <= n; t0 += 2 * D) {
 #pragma unroll
       for (int u = 0; u < D; ++u) {
         // the loads of this ring slot were followed by at most D-1 steps' worth of memory operations
@@ -1161,6 +1179,9 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         const PixF<R> px = ring[u];
         ring2[u] = load_next();
         step(px, t0 + u, std::true_type());
+        // (the steps have no branch left between them; kept apart, the scalars of one step do not
+        // pile up on those of the next, and none of them is spilled inside the loop)
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int u = 0; u < D; ++u) {
@@ -1168,6 +1189,7 @@ __device__ __forceinline__ void run_chain_fwd(const SweepParams& p, const CtxDes
         const PixF<R> px = ring2[u];
         ring[u] = load_next();
         step(px, t0 + D + u, std::true_type());
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
