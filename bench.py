@@ -439,7 +439,7 @@ def contract_bytes(cfg, training, soft=False):
   return fwd_b, bwd_b
 
 
-# the workload BASELINE.json names for each of the smaller configurations
+# the workload of each of the smaller benchmark configurations as the benchmark definition states it
 SMALL_CONFIGS = (("C1", ["ISGMR"], True), ("C2", ["TRWP"], False), ("C3", ["ISGMR"], False),
                  ("C4", ["TRWP", "ISGMR"], True))
 
