@@ -58,6 +58,8 @@ CASES = [
     ("TRWP", 8, 2, 5, 39, 24, "tq4"), ("TRWP", 4, 1, 5, 40, 48, "bump"), ("ISGMR", 4, 1, 5, 41, 96, "tl2"),
     ("ISGMR", 8, 1, 5, 38, 192, "tl3"), ("ISGMR", 4, 1, 4, 37, 256, "tq9"), ("ISGMR", 4, 1, 6, 43, 16, "tq4"),
     ("ISGMR", 4, 1, 5, 40, 100, "bump"), ("ISGMR", 16, 1, 6, 40, 96, "tl2"),
+    # label counts that leave a lane with some of its labels only (a descriptor per access)
+    ("TRWP", 4, 1, 5, 40, 97, "tl3"), ("ISGMR", 4, 1, 5, 38, 131, "tq4"), ("TRWP", 8, 1, 5, 37, 203, "tq9"),
 ]
 
 
