@@ -206,6 +206,15 @@ int mpl_profile_end(mpl_kernel_stat* stats, int n_stats);
  * direction outside the table. */
 int mpl_n_chains(int dir, int height, int width);
 
+/* Whether the forward scans take their O(L^2) step on the 1-D pairwise table `context` (n_disp
+ * floats in HOST memory): 1 when it has neither a constant tail from entry 32 at the latest with no
+ * entry above the tail (the band scan) nor the shape c[k] = min(c[1] * k, c[n_disp - 1]) with
+ * c[0] = 0 (the label scan of a truncated linear table), else 0; -1 for a NULL table or n_disp < 1.
+ * It is what a caller who builds its table on the host passes on as MPL_F_DENSE_TABLE; the library
+ * itself looks at the table on the device, after its launches are sized.  Host-only helper, no
+ * counterpart in the reference. */
+int mpl_table_is_dense(const float* context, int n_disp);
+
 /* Edge-weight producer, the layer's immediate upstream: replaces getEdgeShift of
  * utils/edge_weights.py:45-111.  image (batch, channels, H, W) fp32 -> out (n_dirs, batch, channels,
  * H, W) fp32, fully written: for direction d with step r_d and every pixel p whose front neighbour

@@ -7,7 +7,7 @@ LIB_PATH = os.environ.get("MPLAYERS_HIP_LIB", os.path.join(HERE, "libmplayers_hi
 
 SYMBOLS = ("mpl_trwp_forward", "mpl_trwp_backward", "mpl_isgmr_forward", "mpl_isgmr_backward",
            "mpl_trwp_forward_cpu", "mpl_isgmr_forward_cpu",
-           "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains",
+           "mpl_profile_begin", "mpl_profile_end", "mpl_n_chains", "mpl_table_is_dense",
            "mpl_last_error", "mpl_version", "mpl_edge_shift", "mpl_edge_shift_static",
            "mpl_trwp_soft_forward",
            "mpl_trwp_soft_backward", "mpl_soft_weighted_message", "mpl_soft_weighted_message_back", "mpl_set_option",
@@ -71,6 +71,7 @@ def load():
   lib.mpl_mrf_energy.argtypes = [sp, ci, vp, vp, vp, vp, vp, vp]
   lib.mpl_transpose.argtypes = [vp, vp, ci, ctypes.c_int64, ctypes.c_int64, vp]
   lib.mpl_n_chains.argtypes = [ci, ci, ci]
+  lib.mpl_table_is_dense.argtypes = [vp, ci]
   lib.mpl_profile_begin.argtypes = []
   lib.mpl_profile_end.argtypes = [ctypes.POINTER(KernelStat), ci]
   for name in SYMBOLS:
@@ -110,6 +111,19 @@ def profile_end():
   stats = (KernelStat * len(KERNEL_KINDS))()
   check(load().mpl_profile_end(stats, len(KERNEL_KINDS)), "profile_end")
   return {k: (stats[i].launches, stats[i].total_ms) for i, k in enumerate(KERNEL_KINDS)}
+
+
+def table_is_dense(table):
+  """mpl_table_is_dense on a 1-D table given as a sequence, numpy array or tensor of floats (copied
+  to host memory): True when the forward scans take their O(L^2) step on it."""
+  import numpy as np
+  if hasattr(table, "detach"):
+    table = table.detach().cpu().numpy()
+  row = np.ascontiguousarray(table, dtype=np.float32).reshape(-1)
+  rc = load().mpl_table_is_dense(row.ctypes.data, int(row.size))
+  if rc < 0:
+    raise ValueError("table_is_dense: an empty table")
+  return bool(rc)
 
 
 def check(rc, what):

@@ -847,6 +847,28 @@ int mpl_profile_end(mpl_kernel_stat* stats, int n_stats) {
   return rc;
 }
 
+// The rule of analyze_context_kernel on a table in host memory: neither a band nor truncated linear.
+int mpl_table_is_dense(const float* context, int n_disp) {
+  if (!context || n_disp < 1) return -1;
+  const int L = n_disp;
+  const float tail = context[L - 1], c0 = context[0], slope = L >= 2 ? context[1] : 0.f;
+  unsigned tail_bits;
+  memcpy(&tail_bits, &tail, sizeof tail_bits);
+  if ((tail_bits & 0x7fffffffu) > 0x7f800000u) return 1;  // a NaN tail: no fast path
+  int last_ne = -1;
+  bool below = true, lin = true;
+  for (int i = 0; i < L; ++i) {
+    const float v = context[i];
+    if (!(v == tail)) last_ne = i;
+    below = below && (v <= tail);
+    lin = lin && (v == fminf(slope * (float)i, tail));
+  }
+  if (!below) return 1;
+  const bool band = last_ne + 1 <= kMaxBandK;
+  const bool linear = L >= 2 && c0 == 0.f && slope >= 0.f && lin;
+  return (band || linear) ? 0 : 1;
+}
+
 int mpl_n_chains(int dir, int height, int width) {
   if (dir < 0 || dir >= kMaxDirs || height < 1 || width < 1) return -1;
   return make_dir(dir, height, width).n_chains;

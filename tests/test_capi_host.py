@@ -39,6 +39,31 @@ def test_chain_counts_match_reference_tree_counts(oracle):
   assert lib.mpl_n_chains(16, 4, 4) == -1
 
 
+def test_table_kind_on_the_host():
+  """mpl_table_is_dense: the tables the band and label scans take are not dense, the others are."""
+  from mplayers_amd import _lib
+  k = np.arange(96, dtype=np.float32)
+  rng = np.random.default_rng(3)
+  not_dense = {
+      "potts": np.minimum(k, 1) * 0.7, "tl2": np.minimum(k, 2) * 0.25, "tq5": np.minimum(k * k, 25) * 0.1,
+      "band of 32": np.minimum(k, 32) ** 1.5, "linear": k * 10, "tl95": np.minimum(k, 95) * 10,
+      "constant": np.full(96, 0.3), "bump": np.concatenate([[0.3, 0.1, 0.4], np.full(93, 0.5)]),
+      "one label": np.zeros(1)}
+  dense = {
+      "band of 33": np.minimum(k, 33) ** 1.5, "tq40": np.minimum(k * k, 1600) * 0.01,
+      "quadratic": k * k, "random": np.concatenate([[0], rng.random(95)]),
+      "above its tail": np.concatenate([[0, 2.0], np.ones(94)]),
+      "linear from 1": 1 + k, "nan tail": np.concatenate([np.minimum(k[:95], 2), [np.nan]])}
+  for name, t in not_dense.items():
+    assert _lib.table_is_dense(t) is False, name
+  for name, t in dense.items():
+    assert _lib.table_is_dense(t) is True, name
+  assert _lib.table_is_dense(torch.tensor(dense["tq40"])) is True
+  assert _lib.load().mpl_table_is_dense(None, 4) == -1
+  with pytest.raises(ValueError):
+    _lib.table_is_dense(np.zeros(0))
+
+
 def test_shape_validation_answers_before_any_launch():
   from mplayers_amd import _lib
   lib = _lib.load()

@@ -218,3 +218,25 @@ def test_energy_minimisation_driver(gpu, tmp_path, mode, n_dir):
   assert (mat["seg_all"][:, :, -1] == labels[-1]).all()
   # a second run finds the file and does nothing, as the reference's driver does
   assert energy_min.main(argv) is None
+
+
+def test_driver_declares_a_wide_quadratic_table_dense(gpu):
+  """The driver looks at its fixed table on the host and declares a dense one to the library, whose
+  launches then put several wavefronts on a chain; the labels, energies and costs are those of the
+  same run with one wavefront per chain, bit for bit."""
+  from mplayers_amd import _lib, energy_min
+  argv = ["--synthetic", "20", "44", "--mode", "TRWP", "--n_dir", "4", "--n_iter", "4", "--n_disp",
+          "96", "--context", "TQ", "--truncated", "50", "--p_weight", "1"]
+  k = np.arange(96, dtype=np.float32)
+  assert _lib.table_is_dense(np.minimum(k * k, 2500)) and not _lib.table_is_dense(np.minimum(k, 50))
+  res = energy_min.main(argv)
+  _lib.set_option(_lib.OPT_DENSE_SPLIT_WAVES, 1)
+  try:
+    one = energy_min.main(argv)
+  finally:
+    _lib.set_option(_lib.OPT_DENSE_SPLIT_WAVES, 0)
+  assert (res["labels"].cpu().numpy() == one["labels"].cpu().numpy()).all()
+  assert (res["energy"].cpu().numpy() == one["energy"].cpu().numpy()).all()
+  a, b = res["cost_final"].cpu().numpy(), one["cost_final"].cpu().numpy()
+  assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+  assert len(np.unique(res["labels"][-1].cpu().numpy())) > 1
