@@ -181,6 +181,21 @@ class MPModule(torch.nn.Module):
     if enable_create_label_context:
       self.create_label_context()
 
+  def _fixed_table_is_dense(self, label_context):
+    """Whether the forward scans take their O(L^2) step on the 1-D table the kernels read (the
+    first n_classes entries of label_context), asked once per table: the answer is kept until the
+    stored table is replaced or written to.  It only matters above 64 labels."""
+    n_disp = int(self.args.n_classes)
+    if n_disp <= 64 or not label_context.is_cuda:
+      return False
+    key = (self.label_context.data_ptr(), self.label_context._version)
+    if getattr(self, "_dense_key", None) != key:
+      if torch.cuda.is_current_stream_capturing():
+        return False  # no copy to the host inside a capture; the flag is a hint
+      self._dense_key = key
+      self._dense_answer = _lib.table_is_dense(label_context.reshape(-1)[:n_disp])
+    return self._dense_answer
+
   def get_label_context(self):
     return self.label_context, self.label_context_loc, self.label_context_diag_loc
 
@@ -224,9 +239,12 @@ class MPModule(torch.nn.Module):
       assert self.args.mpnet_max_iter == 1
     label_context = self._effective_label_context()
     self.args.training = self.training
-    # a table that is being learned is dense in general; args.mpnet_dense_table overrides the guess
+    # a table that is being learned is dense in general and a fixed one is looked at once, on the
+    # host; args.mpnet_dense_table overrides both
     dense = getattr(self.args, "mpnet_dense_table", None)
-    self.args.dense_table = bool(self.label_context.requires_grad if dense is None else dense)
+    if dense is None:
+      dense = self.label_context.requires_grad or self._fixed_table_is_dense(label_context)
+    self.args.dense_table = bool(dense)
     if self.args.mpnet_mrf_mode in {'ISGMR', 'SGM'}:
       cost_final, cost_all = ISGMRFunction.apply(unary, label_context, edge_weights, self.args)
     elif self.args.mpnet_mrf_mode == 'TRWP':

@@ -21,7 +21,7 @@ import time
 import numpy as np
 import torch
 
-from . import _lib, compute_terms
+from . import compute_terms
 from .label_context import create_label_context
 from .MP_module import MPModule
 
@@ -126,10 +126,7 @@ def minimise(args, unary, table, n_disp):
   height, width = unary.shape[:2]
   module_args = argparse.Namespace(
       n_classes=n_disp, mpnet_n_dirs=n_dir, mpnet_max_iter=n_iter, mpnet_term_weight=args.p_weight,
-      mpnet_smoothness_train=None, mpnet_mrf_mode=args.mode, rho=args.rho,
-      # the table is fixed and at hand: say so when it is dense (a hint to the launch policy, the
-      # results do not depend on it); the 21-label problems pass an (L, L) table, which is not asked
-      mpnet_dense_table=(n_disp != 21 and _lib.table_is_dense(table.reshape(n_disp, n_disp)[0])))
+      mpnet_smoothness_train=None, mpnet_mrf_mode=args.mode, rho=args.rho)
   module = MPModule(module_args, enable_create_label_context=False, enable_saving_label=True,
                     enable_min_a_dir=args.enable_min_a_dir)
   # one table per direction, as the reference driver passes it (main.py:177-178); the kernels read

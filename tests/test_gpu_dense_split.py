@@ -131,3 +131,39 @@ def test_flag_changes_nothing_for_a_band_table(gpu):
 def test_split_option_is_validated(gpu):
   from mplayers_amd import _lib
   assert _lib.load().mpl_set_option(_lib.OPT_DENSE_SPLIT_WAVES, 9) != 0
+
+
+def test_module_asks_once_whether_a_fixed_table_is_dense(gpu):
+  """MPModule with a table that is not being trained: above 64 labels it asks the library's rule
+  once per table and declares a dense one; a band table, a short table and an explicit
+  args.mpnet_dense_table are left alone, and a table written to is asked about again."""
+  import argparse
+  import torch
+  from mplayers_amd.MP_module import MPModule
+  B, H, W, n_dir = 1, 6, 9, 4
+
+  def module_for(L, table, **extra):
+    args = argparse.Namespace(n_classes=L, mpnet_n_dirs=n_dir, mpnet_max_iter=2, mpnet_term_weight=1,
+                              mpnet_smoothness_train=None, mpnet_mrf_mode="TRWP", **extra)
+    m = MPModule(args, enable_create_label_context=False).eval()
+    m.set_label_context(table.cuda(), None, None)
+    return m
+
+  k96 = torch.arange(96, dtype=torch.float32)
+  unary = torch.rand(B, 1, 96, H, W, generator=torch.Generator().manual_seed(1)).cuda()
+  wide = module_for(96, (k96 * k96).clamp(max=2500.) * 0.01)
+  cost_wide = wide(unary)[0]
+  assert wide.args.dense_table is True
+  band = module_for(96, k96.clamp(max=3.) * 0.3)
+  band(unary)
+  assert band.args.dense_table is False
+  # the same dense table with the declaration switched off: the same bits
+  off = module_for(96, (k96 * k96).clamp(max=2500.) * 0.01, mpnet_dense_table=False)
+  assert torch.equal(off(unary)[0], cost_wide) and off.args.dense_table is False
+  # a table that is written to is looked at again
+  band.label_context.copy_((k96 * k96).clamp(max=2500.) * 0.01)
+  assert torch.equal(band(unary)[0], cost_wide) and band.args.dense_table is True
+  k40 = torch.arange(40, dtype=torch.float32)
+  short = module_for(40, k40 * k40 * 0.01)
+  short(unary[:, :, :40].contiguous())
+  assert short.args.dense_table is False

@@ -221,7 +221,7 @@ def test_energy_minimisation_driver(gpu, tmp_path, mode, n_dir):
 
 
 def test_driver_declares_a_wide_quadratic_table_dense(gpu):
-  """The driver looks at its fixed table on the host and declares a dense one to the library, whose
+  """The module looks at a fixed table on the host and declares a dense one to the library, whose
   launches then put several wavefronts on a chain; the labels, energies and costs are those of the
   same run with one wavefront per chain, bit for bit."""
   from mplayers_amd import _lib, energy_min
