@@ -76,8 +76,11 @@ typedef struct mpl_shape {
  * O(L^2) step.  With more than 64 labels, launches with fewer chains than about three per SIMD then
  * put several wavefronts on every chain, each scanning a share of the front labels of a pixel.
  * The kind of the table is otherwise only known on the device, after the launch is sized.  The
- * results are the same bit for bit with and without the flag, whatever the table; a band table
- * runs slower with it (its launches take the dense step). */
+ * launches that get several wavefronts per chain take the dense step whatever the table: a band
+ * table (a constant tail from entry 32 at the latest) then runs slower and gives the same bits as
+ * without the flag; a wider truncated linear table loses its O(L) label scan, whose values may
+ * differ from the dense step's in the last bits where the table is not integer-valued, both within
+ * the tolerance of the parity tests. */
 #define MPL_F_ALL 0x7fu
 
 /* Replaces lib_*.TRWP.forward: MPLayers/TRWP/TRWP.cpp:245-283 (Forward) -> TRWP_forward.cu:378-560.

@@ -128,6 +128,34 @@ def test_flag_changes_nothing_for_a_band_table(gpu):
                               float(np.abs(a[k].astype(np.float64) - b[k]).max())))
 
 
+def test_flag_on_a_wide_truncated_linear_table(gpu, oracle):
+  """A truncated linear table of more than 32 entries takes the O(L) label scan without the flag and
+  the dense step in the launches that the flag splits.  The scan picks its candidates from
+  products t * slope, so where sums round the two may differ in the last bits: both are held to the
+  oracle's values.  Where nothing rounds the bits are the same: ISGMR on an integer-valued problem
+  (TRWP halves the message of the pixel before at every step of a chain, so its sums round from some
+  twenty pixels on whatever the inputs)."""
+  from mplayers_amd import _lib
+  rng = np.random.default_rng(11)
+  L, n_dir, H, W = 128, 4, 5, 37
+  ew = (0.1 + 0.9 * rng.random((n_dir, 1, 1, H, W))).astype(np.float32)
+  unary = (rng.random((1, 1, H, W, L)) * 3).astype(np.float32)
+  ctx = (0.05 * np.minimum(np.arange(L), 40)).astype(np.float32)
+  for mode, rho in (("TRWP", 0.5), ("ISGMR", 1.0)):
+    ref = oracle.forward(mode, unary, ctx, ew, n_dir, 2, rho, training=True, want_gaps=True)
+    for flags in (0, _lib.F_DENSE_TABLE):
+      got = _forward(gpu, mode, unary, ctx, ew, n_dir, 2, rho, True, flags)
+      gpu.assert_values_close(got["msg"], ref["msg"], what="msg", belief=ref["cost_final"])
+      gpu.assert_values_close(got["cost_final"], ref["cost_final"], what="cost_final")
+  unary_i = rng.integers(0, 60, (1, 1, H, W, L)).astype(np.float32)
+  ctx_i = (2.0 * np.minimum(np.arange(L), 40)).astype(np.float32)
+  ones = np.ones_like(ew)
+  a = _forward(gpu, "ISGMR", unary_i, ctx_i, ones, n_dir, 2, 1.0, True, 0)
+  b = _forward(gpu, "ISGMR", unary_i, ctx_i, ones, n_dir, 2, 1.0, True, _lib.F_DENSE_TABLE)
+  for k in ("msg", "cost_final", "label_all", "msg_min_index", "msg_norm_index"):
+    assert np.array_equal(a[k], b[k]), k
+
+
 def test_split_option_is_validated(gpu):
   from mplayers_amd import _lib
   assert _lib.load().mpl_set_option(_lib.OPT_DENSE_SPLIT_WAVES, 9) != 0
