@@ -99,3 +99,56 @@ def test_a_negative_weight_changes_only_what_it_reaches(gpu, L, kind):
   rows = [0, 1, 3, 4, 5]
   assert np.array_equal(base["msg"][:, :, :, rows].view(np.uint8), other["msg"][:, :, :, rows].view(np.uint8))
   assert not np.array_equal(base["msg"][:, :, :, 2], other["msg"][:, :, :, 2])
+
+
+def _random_long_case(seed):
+  rng = np.random.default_rng(10000 + seed)
+  mode = ["TRWP", "ISGMR"][rng.integers(2)]
+  n_dir = [4, 8, 16][rng.integers(3)]
+  B = int(rng.integers(1, 3))
+  a, b = int(rng.integers(3, 9)), int(rng.integers(30, 72))
+  H, W = (a, b) if rng.integers(2) else (b, a)
+  if rng.integers(4) == 0:
+    H, W = int(rng.integers(20, 40)), int(rng.integers(20, 40))
+  L = [16, 24, 33, 48, 64, 65, 90, 96, 97, 128, 131, 160, 192, 200, 203, 255, 256][rng.integers(17)]
+  kind = ["tl2", "tl3", "tq4", "tq9", "tq20", "tl40", "bump", "dense"][rng.integers(8)]
+  if kind == "tq20" and L < 24:
+    kind = "tq4"
+  training = bool(rng.integers(2))
+  # sixteen directions at rho = 0.5 amplify rounding several times per iteration: two iterations there
+  n_iter = int(rng.integers(1, 3 if n_dir == 16 else 4))
+  unary = (rng.random((B, 1, H, W, L)) * 3).astype(np.float32)
+  ctx = _table(kind, L, rng).astype(np.float32)
+  ew = (0.1 + 0.9 * rng.random((n_dir, B, 1, H, W))).astype(np.float32)
+  negative = int(rng.integers(3))
+  if negative == 1:
+    ew[rng.random(ew.shape) < 0.01] = -0.4
+  elif negative == 2:
+    ew[:, :, :, int(rng.integers(H)), int(rng.integers(W))] = -0.7
+  msg_init = None
+  if rng.integers(3) == 0:
+    msg_init = (rng.random((n_dir, B, 1, H, W, L)) * 0.5).astype(np.float32)
+  return mode, n_dir, n_iter, unary, ctx, ew, training, msg_init, (B, H, W, L, kind, negative)
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_long_chains(gpu, oracle, seed):
+  """Seeded random problems with chains of 20 to 70 pixels: every kind of table, 16 to 256 labels,
+  4 / 8 / 16 directions, 1 to 3 iterations, negative weights nowhere, scattered or at one pixel,
+  zero or given initial messages, with and without argmin labels."""
+  mode, n_dir, n_iter, unary, ctx, ew, training, msg_init, what = _random_long_case(seed)
+  rho = 0.5 if mode == "TRWP" else 1.0
+  print("case", seed, mode, n_dir, n_iter, training, msg_init is not None, what, flush=True)
+  kw = dict(training=training, saving_label=True, msg_init=msg_init)
+  ref = oracle.forward(mode, unary, ctx, ew, n_dir, n_iter, rho, want_gaps=True, **kw)
+  out = gpu.gpu_forward(mode, unary, ctx, ew, n_dir, n_iter, rho, **kw)
+  belief = ref["cost_final"]
+  tol = 1e-5 * max(1.0, float(np.abs(belief).max()))
+  gpu.assert_values_close(out["msg"], ref["msg"], what="msg", belief=belief)
+  gpu.assert_values_close(out["cost_final"], ref["cost_final"], what="cost_final")
+  gpu.assert_labels_match_off_ties(out["label_all"], ref["label_all"], ref["gap_label"], 4 * tol)
+  if training:
+    gpu.assert_indices_match_off_ties(out["msg_min_index"], ref["msg_min_index"], ref["gap_min"],
+                                      4 * tol, "min index")
+    gpu.assert_indices_match_off_ties(out["msg_norm_index"], ref["msg_norm_index"], ref["gap_norm"],
+                                      4 * tol, "norm index")
