@@ -262,6 +262,35 @@ def test_large_config_properties_at_full_size(gpu, mode):
   assert float(dedge[0, 0, 0, :, 1:].abs().max()) > 0.0
 
 
+def _check_rows_inference(gpu, oracle, mode, unary, ctx, ew, n_iter, rho, what):
+  """The forward pass without argmin labels (the kernels compiled for inference), the two horizontal
+  directions on device tensors: first rows, a middle row and the last rows against the oracle."""
+  import torch
+  from mplayers_amd import lib_stereo
+  B, _, H, W, L = unary.shape
+  n_dir = 2
+  dev = unary.device
+  msg = torch.zeros(n_dir, B, 1, H, W, L, device=dev)
+  cost = torch.zeros(B, 1, H, W, L, device=dev)
+  scratch = torch.zeros(B, 1, H, W, L, device=dev)
+  empty = torch.empty(0, dtype=torch.uint8)
+  print(what, mode, "inference", flush=True)
+  if mode == "TRWP":
+    lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg, cost, empty, empty, scratch, empty)
+  else:
+    msg_tmp = torch.zeros_like(msg)
+    lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, ctx, ew, msg, cost, empty, empty, scratch,
+                             msg_tmp, empty)
+    del msg_tmp
+  torch.cuda.synchronize()
+  rows = [0, 1, H // 2, H - 2, H - 1]
+  sub = lambda t, ax: t.index_select(ax, torch.tensor(rows, device=t.device)).cpu().numpy()
+  ref = oracle.forward(mode, sub(unary, 2), ctx.cpu().numpy(), sub(ew, 3), n_dir, n_iter, rho,
+                       training=False)
+  gpu.assert_values_close(sub(msg, 3), ref["msg"], what="msg rows", belief=ref["cost_final"])
+  gpu.assert_values_close(sub(cost, 2), ref["cost_final"], what="cost rows")
+
+
 def _check_rows(gpu, oracle, mode, unary, ctx, ew, dcost, n_iter, rho, what):
   """Runs forward and backward with the two horizontal directions on device tensors and checks the
   first rows, a middle row and the last rows against the oracle."""
@@ -319,9 +348,10 @@ def test_full_size_rows_match_oracle(gpu, oracle, mode):
   from mplayers_amd import synthetic
   cfg = synthetic.make_config("C5", seed=0, mode=mode)
   dev = "cuda:0"
-  _check_rows(gpu, oracle, mode, cfg["unary"].to(dev), cfg["context"].to(dev),
-              cfg["edge_weights"][:2].contiguous().to(dev), synthetic.upstream_grad(cfg).to(dev),
-              cfg["n_iter"], cfg["rho"], "full-size rows")
+  unary, ctx, ew = cfg["unary"].to(dev), cfg["context"].to(dev), cfg["edge_weights"][:2].contiguous().to(dev)
+  _check_rows(gpu, oracle, mode, unary, ctx, ew, synthetic.upstream_grad(cfg).to(dev), cfg["n_iter"],
+              cfg["rho"], "full-size rows")
+  _check_rows_inference(gpu, oracle, mode, unary, ctx, ew, cfg["n_iter"], cfg["rho"], "full-size rows")
 
 
 @pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
@@ -339,6 +369,11 @@ def test_rows_of_the_largest_image_match_oracle(gpu, oracle, mode):
   ctx = (0.25 * torch.clamp(torch.arange(L, dtype=torch.float32), max=3.0)).to(dev)
   rho = 0.5 if mode == "TRWP" else 1.0
   _check_rows(gpu, oracle, mode, unary, ctx, ew, dcost, 1, rho, "largest image rows")
+  del dcost
+  # the kernels compiled for inference, and with them a negative weight in the last row
+  _check_rows_inference(gpu, oracle, mode, unary, ctx, ew, 1, rho, "largest image rows")
+  ew[:, :, :, H - 1, 700] = -0.3
+  _check_rows_inference(gpu, oracle, mode, unary, ctx, ew, 1, rho, "largest image rows, a negative weight")
 
 
 @pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
