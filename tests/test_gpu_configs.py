@@ -436,6 +436,15 @@ def test_full_size_chains_match_oracle(gpu, oracle, mode, pair):
     lib_stereo.ISGMR.backward(0, rho, ctx, ew, dcost, imin, inorm, dunary, dctx, dedge, scratch,
                               scratch, dmsg)
     del msg_tmp
+  # the same run through the kernels compiled for inference (no argmin labels)
+  msg_inf, cost_inf = torch.zeros_like(msg), torch.zeros_like(cost)
+  if mode == "TRWP":
+    lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg_inf, cost_inf, empty, empty, scratch, empty)
+  else:
+    msg_tmp = torch.zeros_like(msg)
+    lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, ctx, ew, msg_inf, cost_inf, empty, empty, scratch,
+                             msg_tmp, empty)
+    del msg_tmp
   torch.cuda.synchronize()
   # messages of the switched-off directions vanish
   for d in range(n_dir):
@@ -465,6 +474,10 @@ def test_full_size_chains_match_oracle(gpu, oracle, mode, pair):
     gpu.assert_values_close(got_msg, ref["msg"], what="chain msg", belief=belief)
     gpu.assert_values_close(cost[:, :, hh, ww, :].cpu().numpy()[:, :, None], ref["cost_final"],
                             what="chain cost")
+    gpu.assert_values_close(msg_inf[[pair, pair + 1]][:, :, :, hh, ww, :].cpu().numpy()[:, :, :, None],
+                            ref["msg"], what="chain msg, inference", belief=belief)
+    gpu.assert_values_close(cost_inf[:, :, hh, ww, :].cpu().numpy()[:, :, None], ref["cost_final"],
+                            what="chain cost, inference")
     gi = imin[:, [pair, pair + 1]][:, :, :, :, hh, ww, :].cpu().numpy()[:, :, :, :, None]
     gn = inorm[:, [pair, pair + 1]][:, :, :, :, hh, ww].cpu().numpy()[:, :, :, :, None]
     gpu.assert_indices_match_off_ties(gi, ref["msg_min_index"], ref["gap_min"], 4 * tol, "min idx")
