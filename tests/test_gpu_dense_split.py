@@ -195,3 +195,65 @@ def test_module_asks_once_whether_a_fixed_table_is_dense(gpu):
   short = module_for(40, k40 * k40 * 0.01)
   short(unary[:, :, :40].contiguous())
   assert short.args.dense_table is False
+
+
+@pytest.mark.parametrize("mode", ["TRWP", "ISGMR"])
+@pytest.mark.parametrize("pair", [0, 2])
+def test_split_scans_at_the_measured_size(gpu, oracle, mode, pair):
+  """384 x 1248 pixels, 192 labels, a dense table declared dense: the launches of the size whose
+  rate is reported (four wavefronts per chain on the 384 rows, two on the 1248 columns for TRWP,
+  one for ISGMR's launch of all directions).  Zero edge weights switch the other pair of directions
+  off, so single rows / columns are two-direction problems on a 1 x n image for the oracle;
+  with and without argmin labels."""
+  import torch
+  from mplayers_amd import _lib, lib_stereo
+  H, W, L, n_dir, n_iter = 384, 1248, 192, 4, 2
+  rho = 0.5 if mode == "TRWP" else 1.0
+  dev = "cuda:0"
+  g = torch.Generator(device=dev)
+  g.manual_seed(5)
+  unary = torch.rand(1, 1, H, W, L, device=dev, generator=g) * 3
+  ew = 0.1 + 0.9 * torch.rand(n_dir, 1, 1, H, W, device=dev, generator=g)
+  for d in range(n_dir):
+    if d not in (pair, pair + 1):
+      ew[d] = 0
+  ctx = torch.cat([torch.zeros(1, device=dev), torch.rand(L - 1, device=dev, generator=g)])
+  empty = torch.empty(0, dtype=torch.uint8)
+  runs = {}
+  for training in (True, False):
+    msg = torch.zeros(n_dir, 1, 1, H, W, L, device=dev)
+    cost = torch.zeros(1, 1, H, W, L, device=dev)
+    scratch = torch.zeros(1, 1, H, W, L, device=dev)
+    imin = torch.zeros(n_iter, n_dir, 1, 1, H, W, L, dtype=torch.uint8, device=dev) if training else empty
+    inorm = torch.zeros(n_iter, n_dir, 1, 1, H, W, dtype=torch.uint8, device=dev) if training else empty
+    print("measured size", mode, pair, training, flush=True)
+    if mode == "TRWP":
+      lib_stereo.TRWP.forward(rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch, empty,
+                              flags=_lib.F_DENSE_TABLE)
+    else:
+      lib_stereo.ISGMR.forward(0, rho, n_iter, 0, unary, ctx, ew, msg, cost, imin, inorm, scratch,
+                               torch.zeros_like(msg), empty, flags=_lib.F_DENSE_TABLE)
+    torch.cuda.synchronize()
+    runs[training] = (msg, cost, imin, inorm)
+  ctx_np = ctx.cpu().numpy()
+  for k in ([0, 191, 383] if pair == 0 else [0, 700, 1247]):
+    if pair == 0:
+      hh, ww = torch.full((W,), k, device=dev), torch.arange(W, device=dev)
+    else:
+      hh, ww = torch.arange(H, device=dev), torch.full((H,), k, device=dev)
+    un = unary[:, :, hh, ww, :].cpu().numpy()[:, :, None]
+    en = ew[[pair, pair + 1]][:, :, :, hh, ww].cpu().numpy()[:, :, :, None]
+    ref = oracle.forward(mode, un, ctx_np, en, 2, n_iter, rho, want_gaps=True)
+    belief = ref["cost_final"]
+    tol = 1e-5 * max(1.0, float(np.abs(belief).max()))
+    for training, (msg, cost, imin, inorm) in runs.items():
+      what = "chain %d, %s" % (k, "training" if training else "inference")
+      gpu.assert_values_close(msg[[pair, pair + 1]][:, :, :, hh, ww, :].cpu().numpy()[:, :, :, None],
+                              ref["msg"], what="msg, " + what, belief=belief)
+      gpu.assert_values_close(cost[:, :, hh, ww, :].cpu().numpy()[:, :, None], ref["cost_final"],
+                              what="cost, " + what)
+      if training:
+        gi = imin[:, [pair, pair + 1]][:, :, :, :, hh, ww, :].cpu().numpy()[:, :, :, :, None]
+        gn = inorm[:, [pair, pair + 1]][:, :, :, :, hh, ww].cpu().numpy()[:, :, :, :, None]
+        gpu.assert_indices_match_off_ties(gi, ref["msg_min_index"], ref["gap_min"], 4 * tol, "min idx")
+        gpu.assert_indices_match_off_ties(gn, ref["msg_norm_index"], ref["gap_norm"], 4 * tol, "norm idx")
