@@ -73,8 +73,8 @@ typedef struct mpl_shape {
 #define MPL_F_DENSE_TABLE 0x40u
 /* forward calls: the caller declares that its 1-D pairwise table is dense (a learned table, an
  * untruncated one): no constant tail that the O(L) band scan could use, so the scans take their
- * O(L^2) step.  With more than 64 labels, launches with fewer chains than about three per SIMD then
- * put several wavefronts on every chain, each scanning a share of the front labels of a pixel.
+ * O(L^2) step.  With more than 64 labels, launches of at most one and a half chains per SIMD then
+ * put four or two wavefronts on every chain, each scanning a share of the front labels of a pixel.
  * The kind of the table is otherwise only known on the device, after the launch is sized.  The
  * launches that get several wavefronts per chain take the dense step whatever the table: a band
  * table (a constant tail from entry 32 at the latest) then runs slower and gives the same bits as
