@@ -256,7 +256,9 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, int bytes) {
 
 // Cache-policy bits of the label-vector accesses (gfx94x/95x: 1 = sc0, 2 = nt, 16 = sc1).  Every
 // plane is streamed once per sweep and is far larger than the caches, so loads and stores carry the
-// non-temporal hint; measured on the 1500x2000x192 forward sweep: 2.98 ms without, 2.54 ms with.
+// non-temporal hint; measured on the 1500x2000x192 forward sweep: 2.98 ms without, 2.54 ms with
+// (with the present kernels 2.15 ms against 2.39 ms with the hint on the loads only, 2.17 ms on the
+// stores only, and 3.48 ms with sc1 added to both).
 #ifndef MPL_LD_AUX
 #define MPL_LD_AUX 2
 #endif
