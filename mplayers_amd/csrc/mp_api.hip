@@ -513,13 +513,16 @@ int launch_ok(const char* what) {
   return MPL_OK;
 }
 
+// Workgroups of an element-wise kernel over n accesses (of 4 floats or of 1): one access per thread.
 // One pass over the data with as many workgroups as it takes measured 3-8 % faster than a
-// grid-stride loop of 32 workgroups per CU on the 2.3 GB planes; the cap only bounds the grid.
+// grid-stride loop of 32 workgroups per CU on the 2.3 GB planes, and 2 / 4 / 8 accesses per thread
+// measured 2 / 5 / 9 % slower than one (workgroups of 64, 128 and 512 threads: 4 to 5 % slower than
+// 256); the cap only bounds the grid.
 #ifndef MPL_EW_BLOCKS_PER_CU
 #define MPL_EW_BLOCKS_PER_CU 4096
 #endif
 int elementwise_blocks(int64_t n) {
-  int64_t b = (n + 256 * 4 - 1) / (256 * 4);
+  int64_t b = (n + 256 - 1) / 256;
   if (b < 1) b = 1;
   if (b > 256 * MPL_EW_BLOCKS_PER_CU) b = 256 * MPL_EW_BLOCKS_PER_CU;
   return (int)b;
