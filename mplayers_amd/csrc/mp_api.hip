@@ -686,17 +686,22 @@ SweepParams base_fwd_params(const mpl_shape* s, float rho, const float* edge, co
   return p;
 }
 
-// plain zero fill (a kernel, so that a caller may capture the call in a graph)
+// plain zero fill (a kernel, so that a caller may capture the call in a graph); V floats per store
+template <int V>
 __global__ void __launch_bounds__(256) zero_fill_kernel(float* __restrict__ dst, int64_t n) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (int64_t)gridDim.x * blockDim.x)
-    dst[i] = 0.f;
+  Pack<V> z;
+#pragma unroll
+  for (int j = 0; j < V; ++j) z.v[j] = 0.f;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * V; i < n;
+       i += (int64_t)gridDim.x * blockDim.x * V)
+    st_pack<V>(dst + i, z);
 }
 
 void zero_fill(float* dst, int64_t n, hipStream_t st) {
-  int64_t blocks = (n + 255) / 256;
-  if (blocks > 256 * 64) blocks = 256 * 64;
-  zero_fill_kernel<<<(int)blocks, 256, 0, st>>>(dst, n);
+  if ((n & 3) == 0 && aligned16(dst))
+    zero_fill_kernel<4><<<elementwise_blocks(n / 4), 256, 0, st>>>(dst, n);
+  else
+    zero_fill_kernel<1><<<elementwise_blocks(n), 256, 0, st>>>(dst, n);
 }
 
 // The sweeps keep the belief plane up to date by differences, S <- (S - m_old) + m_new, where the
